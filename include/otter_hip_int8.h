@@ -1,0 +1,175 @@
+/*
+ * otter_hip_int8.h -- C ABI of the MI355X (gfx950) implementation of Otter's int8 convolution path.
+ *
+ * This is the only boundary that touches HIP. Plain pointers and sizes, int status codes, no C++ types.
+ * Every tensor pointer is a DEVICE pointer unless a parameter says "host". Every call that launches work
+ * takes the hipStream_t to launch on (as void*, NULL = the default stream) and returns without waiting
+ * for the GPU. Handles are immutable after creation and may be used from several host threads.
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to the reference
+ * repository root).
+ *
+ * Status codes follow the reference's Layer convention (Tensor/Layer.cpp:50-59): 0 ok, -1 not supported,
+ * -100 allocation failure; -2 invalid argument and -3 HIP runtime error are added. Nothing throws across
+ * this boundary; otter_hip_last_error() returns the text for the calling thread's last failure.
+ */
+#ifndef OTTER_HIP_INT8_H
+#define OTTER_HIP_INT8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OTTER_HIP_OK 0
+#define OTTER_HIP_ERR_UNSUPPORTED (-1)
+#define OTTER_HIP_ERR_INVALID (-2)
+#define OTTER_HIP_ERR_RUNTIME (-3)
+#define OTTER_HIP_ERR_ALLOC (-100)
+
+/* Tensor layouts = the reference's dtype x elempack (Tensor/ScalarType.hpp:45-74). A packed tensor with
+ * logical shape [N,C,H,W] is stored [N, C/p, H, W, p] (Tensor/TensorPacking.cpp:1397-1552). "I8" holds
+ * signed int8 in the reference's Byte dtype. */
+typedef enum {
+    OTTER_HIP_F32 = 0,    /* Float   [N,C,H,W]     */
+    OTTER_HIP_F32_P4 = 1, /* Float4  [N,C/4,H,W,4] */
+    OTTER_HIP_F32_P8 = 2, /* Float8  [N,C/8,H,W,8] */
+    OTTER_HIP_I8 = 3,     /* Byte    [N,C,H,W]     */
+    OTTER_HIP_I8_P8 = 4,  /* Byte8   [N,C/8,H,W,8] */
+    OTTER_HIP_I32 = 5,    /* Int     [N,C,H,W]     */
+    OTTER_HIP_I32_P4 = 6, /* Int4    [N,C/4,H,W,4] */
+    OTTER_HIP_I32_P8 = 7  /* Int8    [N,C/8,H,W,8] (eight int32 lanes, the depthwise accumulator type) */
+} otter_hip_layout;
+
+/* what a convolution handle produces */
+typedef enum {
+    OTTER_HIP_OUT_I32 = 0, /* raw accumulators: what otter::convolution returns on int8 input */
+    OTTER_HIP_OUT_F32 = 1, /* dequantize_from_int32 (+ the activation layer), int8_scale_term <= 100 */
+    OTTER_HIP_OUT_I8 = 2   /* requantize_from_int32_to_int8, int8_scale_term > 100 */
+} otter_hip_out_kind;
+
+/* rounding primitive of fp32 -> int8 (both saturate to [-127, 127]) */
+typedef enum {
+    OTTER_HIP_ROUND_SSE = 0,  /* trunc(v + copysign(0.5f, v)): float2int8_sse, Tensor/VecIntrinsic.hpp:71-95;
+                                 what every packed (elempack 4/8) quantize / requantize loop uses */
+    OTTER_HIP_ROUND_EXACT = 1 /* round half away from zero: float2int8, Tensor/QuantizeX86.cpp:18-23;
+                                 what the unpacked loops use */
+} otter_hip_round_mode;
+
+/* ------------------------------------------------------------------------------------------------ */
+/* library                                                                                          */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* Selects the GPU and checks that it is a gfx950. No counterpart in the reference (Device has the single
+ * value CPU, Tensor/Device.hpp:15-18). */
+int otter_hip_init(int device);
+int otter_hip_shutdown(void);
+const char* otter_hip_last_error(void);
+
+/* compute units, engine clock in MHz, memory clock in MHz, memory bus width in bits: inputs of the roofline */
+int otter_hip_device_info(int* compute_units, int* clock_mhz, int* mem_clock_mhz, int* mem_bus_bits);
+
+/* Device memory + copies for hosts that do not link HIP themselves. Stand in for otter::empty() /
+ * Tensor::data_ptr() ownership of blobs (Tensor/TensorFactory.hpp, Tensor/Net.cpp:413-505). */
+int otter_hip_malloc(void** ptr, size_t bytes);
+int otter_hip_free(void* ptr);
+int otter_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+int otter_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+int otter_hip_stream_create(void** stream);
+int otter_hip_stream_destroy(void* stream);
+int otter_hip_stream_synchronize(void* stream);
+
+/* ------------------------------------------------------------------------------------------------ */
+/* convolution layer                                                                                */
+/* ------------------------------------------------------------------------------------------------ */
+
+typedef struct otter_hip_conv otter_hip_conv_t;
+
+/* Mirrors the state of otter::ConvolutionLayer after load_param (Tensor/ConvolutionLayer.hpp:40-77,
+ * Tensor/ConvolutionLayer.cpp:185-206). */
+typedef struct {
+    int in_channels, out_channels;
+    int kernel_h, kernel_w;
+    int stride_h, stride_w;
+    int pad_h, pad_w;
+    int dilation_h, dilation_w;
+    int groups;
+    int activation_type;     /* 0 none, 1 ReLU, 2 LeakyReLU, 3 clip [0,6], 4 sigmoid
+                                (Tensor/ConvolutionLayer.cpp:113-122, Tensor/QuantizeX86.hpp:72-106) */
+    float activation_param0; /* LeakyReLU slope */
+    int out_kind;            /* otter_hip_out_kind */
+    int out_round_mode;      /* otter_hip_round_mode used when out_kind is I8 */
+    int in_round_mode;       /* otter_hip_round_mode used when forward() is handed fp32 input */
+} otter_hip_conv_desc;
+
+/* ConvolutionLayer::create_pipeline_int8 (Tensor/ConvolutionLayer.cpp:666-752): uploads and re-lays-out the
+ * int8 weights once. All array arguments are HOST pointers:
+ *   weight    [K, C/groups, kh, kw] int8  (ConvolutionLayer::weight_data)
+ *   scale_in  [K]  = 1/(in_scale*weight_scale[k]), computed by the caller exactly as :667-679 does; it is
+ *                    never recomputed on the device
+ *   bias      [K] or NULL                  (ConvolutionLayer::bias_data)
+ *   in_scale  bottom_blob_int8_scales[0], used only when forward() receives fp32 input
+ *   out_scale [n_out_scale] (1 or K), top_blob_int8_scales, used only for OTTER_HIP_OUT_I8 */
+int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight, const float* scale_in,
+                          const float* bias, float in_scale, const float* out_scale, int n_out_scale,
+                          otter_hip_conv_t** handle);
+int otter_hip_conv_destroy(otter_hip_conv_t* handle);
+
+/* Output geometry (Tensor/ConvolutionUtils.hpp:173-191) and the layout the reference would produce for
+ * this layer in packing mode (Tensor/ConvolutionLayer.cpp:777-787, Tensor/QuantizeX86.cpp:650-653,1729). */
+int otter_hip_conv_output_shape(const otter_hip_conv_t* handle, int in_h, int in_w, int* out_h, int* out_w);
+int otter_hip_conv_default_out_layout(const otter_hip_conv_t* handle);
+
+/* Bytes of device scratch forward() needs for this input (0 unless the input is fp32: the quantized copy). */
+size_t otter_hip_conv_workspace_bytes(const otter_hip_conv_t* handle, int in_layout, int n, int in_h, int in_w);
+
+/* ConvolutionLayer::forward_int8 (Tensor/ConvolutionLayer.cpp:754-847) for a whole batch:
+ * [quantize_to_int8 ->] convolution -> dequantize_from_int32 (+activation) | requantize_from_int32_to_int8.
+ *   in_layout : I8_P8 or I8 (already quantized blob, :770-775) or F32 / F32_P4 / F32_P8 (quantized first
+ *               with in_scale; needs `workspace`)
+ *   out_layout: any layout whose element type matches out_kind and whose pack divides K
+ * Batch images are independent (the reference runs them one by one, Tensor/Padding.cpp:26-29). */
+int otter_hip_conv_forward(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h, int in_w,
+                           void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
+ * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel. For tests and profiling. */
+int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, int n, int in_h, int in_w,
+                               int out_layout);
+
+/* Tuning / test hook with no counterpart in the reference: force the MFMA tile of a handle to tm output
+ * channels x tn pixels (tm in {32,64,128}, tn in {64,128,256}; 0,0 = automatic choice). */
+int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
+
+/* ------------------------------------------------------------------------------------------------ */
+/* standalone quantize / dequantize / requantize                                                    */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* otter::quantize_to_int8 (Tensor/Quantize.hpp:15, Tensor/QuantizeX86.cpp:47-644):
+ * q = sat127(round(x * scale[n_scales == 1 ? 0 : c])). scales is a DEVICE array. */
+int otter_hip_quantize(const float* src, int src_layout, int n, int c, int h, int w, const float* scales,
+                       int n_scales, int round_mode, int8_t* dst, int dst_layout, void* stream);
+
+/* otter::dequantize_from_int32 (Tensor/Quantize.hpp:17, Tensor/QuantizeX86.cpp:646-1161):
+ * y = fma(float(acc), scale[c], bias[c]) (bias may be NULL). scale / bias are DEVICE arrays. */
+int otter_hip_dequantize(const int32_t* src, int src_layout, int n, int c, int h, int w, const float* scale,
+                         int n_scale, const float* bias, int n_bias, float* dst, int dst_layout, void* stream);
+
+/* otter::requantize_from_int32_to_int8 (Tensor/Quantize.hpp:19, Tensor/QuantizeX86.cpp:1163-2129):
+ * v = fma(float(acc), scale_in[c], bias[c]); v = act(v); q = sat127(round(v * scale_out[c])). */
+int otter_hip_requantize(const int32_t* src, int src_layout, int n, int c, int h, int w, const float* scale_in,
+                         int n_scale_in, const float* scale_out, int n_scale_out, const float* bias, int n_bias,
+                         int activation_type, float activation_param0, int round_mode, int8_t* dst,
+                         int dst_layout, void* stream);
+
+/* Tensor::packing (Tensor/Tensor.cpp:29-35, Tensor/TensorPacking.cpp:141-158): re-pack between layouts of
+ * the same element type on the device (what Net::convert_layout does on the host, Tensor/Net.cpp:380-411). */
+int otter_hip_repack(const void* src, int src_layout, int n, int c, int h, int w, void* dst, int dst_layout,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OTTER_HIP_INT8_H */

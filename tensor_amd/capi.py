@@ -1,0 +1,216 @@
+"""ctypes binding of include/otter_hip_int8.h. Fails loudly when the library or the GPU is missing:
+there is no CPU fallback anywhere in this package."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libotter_hip_int8.so")
+
+# otter_hip_layout
+F32, F32_P4, F32_P8, I8, I8_P8, I32, I32_P4, I32_P8 = range(8)
+OUT_I32, OUT_F32, OUT_I8 = 0, 1, 2
+ROUND_SSE, ROUND_EXACT = 0, 1
+ACT = {"": 0, None: 0, "Relu": 1, "LRelu": 2, "Relu6": 3, "Sigmoid": 4}
+
+_PACK = {F32: 1, F32_P4: 4, F32_P8: 8, I8: 1, I8_P8: 8, I32: 1, I32_P4: 4, I32_P8: 8}
+_NP = {F32: np.float32, F32_P4: np.float32, F32_P8: np.float32, I8: np.int8, I8_P8: np.int8, I32: np.int32,
+       I32_P4: np.int32, I32_P8: np.int32}
+
+
+def layout_pack(layout):
+    return _PACK[layout]
+
+
+def layout_dtype(layout):
+    return _NP[layout]
+
+
+def layout_for(dtype, pack):
+    base = {np.dtype(np.float32): F32, np.dtype(np.int8): I8, np.dtype(np.int32): I32}[np.dtype(dtype)]
+    return base + {1: 0, 4: 1, 8: 2 if base != I8 else 1}[pack]
+
+
+def pack_np(a, p):
+    """[N,C,H,W] -> the reference's packed storage [N,C/p,H,W,p] (numpy, host side test helper)."""
+    if p == 1:
+        return np.ascontiguousarray(a)
+    n, c, h, w = a.shape
+    return np.ascontiguousarray(a.reshape(n, c // p, p, h, w).transpose(0, 1, 3, 4, 2))
+
+
+def unpack_np(a, p, shape):
+    if p == 1:
+        return np.ascontiguousarray(a).reshape(shape)
+    n, c, h, w = shape
+    return np.ascontiguousarray(a.reshape(n, c // p, h, w, p).transpose(0, 1, 4, 2, 3)).reshape(shape)
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in ("in_channels", "out_channels", "kernel_h", "kernel_w", "stride_h", "stride_w",
+                                       "pad_h", "pad_w", "dilation_h", "dilation_w", "groups", "activation_type")] + \
+               [("activation_param0", C.c_float), ("out_kind", C.c_int), ("out_round_mode", C.c_int),
+                ("in_round_mode", C.c_int)]
+
+
+class HipError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("otter_hip error %d: %s" % (code, msg))
+        self.code = code
+
+
+EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otter_hip_device_info", "otter_hip_malloc",
+           "otter_hip_free", "otter_hip_memcpy_h2d", "otter_hip_memcpy_d2h", "otter_hip_stream_create",
+           "otter_hip_stream_destroy", "otter_hip_stream_synchronize", "otter_hip_conv_create",
+           "otter_hip_conv_destroy", "otter_hip_conv_output_shape", "otter_hip_conv_default_out_layout",
+           "otter_hip_conv_workspace_bytes", "otter_hip_conv_forward", "otter_hip_conv_kernel_kind",
+           "otter_hip_quantize", "otter_hip_dequantize", "otter_hip_requantize", "otter_hip_repack"]
+
+
+def load_cdll():
+    if not os.path.exists(LIB_PATH):
+        raise OSError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                      "(tensor_amd/csrc/build.sh)" % LIB_PATH)
+    return C.CDLL(LIB_PATH)
+
+
+class Library:
+    """The GPU library on cuda:0. Tensors are torch CUDA tensors holding the reference's packed storage."""
+
+    def __init__(self, device=0):
+        import torch
+        self.torch = torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: the int8 convolution path has no CPU fallback")
+        L = self.lib = load_cdll()
+        L.otter_hip_last_error.restype = C.c_char_p
+        L.otter_hip_conv_workspace_bytes.restype = C.c_size_t
+        self.device = torch.device("cuda", device)
+        self._check(L.otter_hip_init(C.c_int(device)))
+
+    # -- plumbing -------------------------------------------------------------------------------------
+    def _check(self, rc):
+        if rc != 0:
+            raise HipError(rc, self.lib.otter_hip_last_error().decode(errors="replace"))
+
+    def stream(self):
+        return C.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+
+    def to_device(self, a):
+        return self.torch.from_numpy(np.ascontiguousarray(a)).to(self.device)
+
+    def empty(self, count, dtype):
+        t = {np.float32: self.torch.float32, np.int8: self.torch.int8, np.int32: self.torch.int32}[dtype]
+        return self.torch.empty(int(count), dtype=t, device=self.device)
+
+    @staticmethod
+    def ptr(t):
+        return C.c_void_p(t.data_ptr())
+
+    def device_info(self):
+        v = [C.c_int() for _ in range(4)]
+        self._check(self.lib.otter_hip_device_info(*[C.byref(x) for x in v]))
+        return dict(compute_units=v[0].value, clock_mhz=v[1].value, mem_clock_mhz=v[2].value, mem_bus_bits=v[3].value)
+
+    # -- standalone ops (device tensors in packed storage) ------------------------------------------------
+    def quantize(self, src, src_layout, shape, scales, round_mode, dst_layout, dst=None):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, np.int8) if dst is None else dst
+        self._check(self.lib.otter_hip_quantize(self.ptr(src), src_layout, n, c, h, w, self.ptr(scales),
+                                                C.c_int(scales.numel()), round_mode, self.ptr(dst), dst_layout,
+                                                self.stream()))
+        return dst
+
+    def dequantize(self, src, src_layout, shape, scale, bias, dst_layout, dst=None):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, np.float32) if dst is None else dst
+        self._check(self.lib.otter_hip_dequantize(self.ptr(src), src_layout, n, c, h, w, self.ptr(scale),
+                                                  C.c_int(scale.numel()), self.ptr(bias) if bias is not None else None,
+                                                  C.c_int(0 if bias is None else bias.numel()), self.ptr(dst),
+                                                  dst_layout, self.stream()))
+        return dst
+
+    def requantize(self, src, src_layout, shape, scale_in, scale_out, bias, act, act_p0, round_mode, dst_layout,
+                   dst=None):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, np.int8) if dst is None else dst
+        self._check(self.lib.otter_hip_requantize(
+            self.ptr(src), src_layout, n, c, h, w, self.ptr(scale_in), C.c_int(scale_in.numel()), self.ptr(scale_out),
+            C.c_int(scale_out.numel()), self.ptr(bias) if bias is not None else None,
+            C.c_int(0 if bias is None else bias.numel()), C.c_int(act), C.c_float(act_p0), C.c_int(round_mode),
+            self.ptr(dst), dst_layout, self.stream()))
+        return dst
+
+    def repack(self, src, src_layout, shape, dst_layout, dst=None):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, layout_dtype(src_layout)) if dst is None else dst
+        self._check(self.lib.otter_hip_repack(self.ptr(src), src_layout, n, c, h, w, self.ptr(dst), dst_layout,
+                                              self.stream()))
+        return dst
+
+    def conv(self, **kw):
+        return Conv(self, **kw)
+
+
+class Conv:
+    """otter_hip_conv_t. Arguments follow otter::ConvolutionLayer's members (Tensor/ConvolutionLayer.hpp:40-77)."""
+
+    def __init__(self, lib, *, wq, scale_in, bias=None, in_scale=1.0, out_scale=None, stride=(1, 1), pad=(0, 0),
+                 dil=(1, 1), groups=1, act=0, act_p0=0.0, out_kind=OUT_I32, out_round=ROUND_SSE, in_round=ROUND_SSE):
+        self.L = lib
+        wq = np.ascontiguousarray(wq, np.int8)
+        k, cg, kh, kw = wq.shape
+        self.K, self.C, self.kh, self.kw = k, cg * groups, kh, kw
+        self.stride, self.pad, self.dil, self.groups, self.out_kind = stride, pad, dil, groups, out_kind
+        d = ConvDesc(cg * groups, k, kh, kw, stride[0], stride[1], pad[0], pad[1], dil[0], dil[1], groups, act,
+                     act_p0, out_kind, out_round, in_round)
+        si = np.ascontiguousarray(scale_in, np.float32)
+        assert si.size == k
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        so = None if out_scale is None else np.ascontiguousarray(np.atleast_1d(out_scale), np.float32)
+        self.h = C.c_void_p()
+        f32p = C.POINTER(C.c_float)
+        lib._check(lib.lib.otter_hip_conv_create(
+            C.byref(d), wq.ctypes.data_as(C.c_void_p), si.ctypes.data_as(f32p),
+            b.ctypes.data_as(f32p) if b is not None else None, C.c_float(in_scale),
+            so.ctypes.data_as(f32p) if so is not None else None, C.c_int(0 if so is None else so.size),
+            C.byref(self.h)))
+
+    def out_hw(self, h, w):
+        oh, ow = C.c_int(), C.c_int()
+        self.L._check(self.L.lib.otter_hip_conv_output_shape(self.h, h, w, C.byref(oh), C.byref(ow)))
+        return oh.value, ow.value
+
+    def default_out_layout(self):
+        return self.L.lib.otter_hip_conv_default_out_layout(self.h)
+
+    def kernel_kind(self, in_layout, n, h, w, out_layout):
+        return self.L.lib.otter_hip_conv_kernel_kind(self.h, in_layout, n, h, w, out_layout)
+
+    def set_tile(self, tm, tn):
+        self.L._check(self.L.lib.otter_hip_conv_set_tile(self.h, tm, tn))
+
+    def forward(self, x, in_layout, n, h, w, out_layout=None, out=None, workspace=None):
+        out_layout = self.default_out_layout() if out_layout is None else out_layout
+        oh, ow = self.out_hw(h, w)
+        if out is None:
+            out = self.L.empty(n * self.K * oh * ow, layout_dtype(out_layout))
+        ws_bytes = self.L.lib.otter_hip_conv_workspace_bytes(self.h, in_layout, n, h, w)
+        if ws_bytes and workspace is None:
+            workspace = self.L.empty(ws_bytes, np.int8)
+        self.L._check(self.L.lib.otter_hip_conv_forward(
+            self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout,
+            self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))
+        return out
+
+    def close(self):
+        if self.h:
+            self.L.lib.otter_hip_conv_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

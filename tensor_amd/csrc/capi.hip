@@ -1,0 +1,395 @@
+// extern "C" boundary of the library (include/otter_hip_int8.h): argument checking, handle management,
+// weight re-layout at create time and kernel dispatch. No kernels live here.
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "common.hpp"
+#include "conv_igemm.hpp"
+
+using namespace ohip;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    (void)hipGetLastError();
+    return fail(e == hipErrorOutOfMemory ? OTTER_HIP_ERR_ALLOC : OTTER_HIP_ERR_RUNTIME,
+                std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define OHIP_CHECK(expr)                                  \
+    do {                                                  \
+        hipError_t e__ = (expr);                          \
+        if (e__ != hipSuccess) return hip_fail(e__, #expr); \
+    } while (0)
+
+bool valid_layout(int l) { return l >= OTTER_HIP_F32 && l <= OTTER_HIP_I32_P8; }
+
+int conv_out_size(int in, int k, int s, int p, int d) { return (in + 2 * p - d * (k - 1) - 1) / s + 1; }
+
+template <typename T>
+int upload(T** dev, const T* host, size_t count, size_t padded_count, T pad_value) {
+    std::vector<T> tmp(padded_count, pad_value);
+    if (host) std::memcpy(tmp.data(), host, count * sizeof(T));
+    OHIP_CHECK(hipMalloc((void**)dev, padded_count * sizeof(T)));
+    OHIP_CHECK(hipMemcpy(*dev, tmp.data(), padded_count * sizeof(T), hipMemcpyHostToDevice));
+    return OTTER_HIP_OK;
+}
+
+}  // namespace
+
+struct otter_hip_conv {
+    otter_hip_conv_desc d;
+    bool depthwise = false;
+    int8_t* w_raw = nullptr;     // [K, C/g, kh, kw]           (direct kernel)
+    int8_t* w_igemm = nullptr;   // MFMA lane order            (groups == 1, C % 8 == 0)
+    int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
+    float* scale_in = nullptr;   // [Kpad]
+    float* bias = nullptr;       // [Kpad] or null
+    float* scale_out = nullptr;  // [Kpad] or null
+    float* in_scale = nullptr;   // [1]
+    int force_tm = 0, force_tn = 0;
+};
+
+extern "C" {
+
+const char* otter_hip_last_error(void) { return g_last_error.c_str(); }
+
+int otter_hip_init(int device) {
+    int count = 0;
+    OHIP_CHECK(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_init: no such device");
+    OHIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    OHIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED,
+                    std::string("otter_hip_init: this library is built for gfx950 only, found ") + prop.gcnArchName);
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_shutdown(void) { return OTTER_HIP_OK; }
+
+int otter_hip_device_info(int* compute_units, int* clock_mhz, int* mem_clock_mhz, int* mem_bus_bits) {
+    int dev = 0;
+    OHIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    OHIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+    if (mem_clock_mhz) *mem_clock_mhz = prop.memoryClockRate / 1000;
+    if (mem_bus_bits) *mem_bus_bits = prop.memoryBusWidth;
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_malloc: null");
+    OHIP_CHECK(hipMalloc(ptr, bytes ? bytes : 1));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_free(void* ptr) {
+    if (ptr) OHIP_CHECK(hipFree(ptr));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+    OHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+    OHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_stream_create(void** stream) {
+    hipStream_t s;
+    OHIP_CHECK(hipStreamCreate(&s));
+    *stream = (void*)s;
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_stream_destroy(void* stream) {
+    OHIP_CHECK(hipStreamDestroy((hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_stream_synchronize(void* stream) {
+    OHIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------
+// convolution
+// -----------------------------------------------------------------------------------------------------
+
+int otter_hip_conv_destroy(otter_hip_conv_t* h) {
+    if (!h) return OTTER_HIP_OK;
+    (void)hipFree(h->w_raw);
+    (void)hipFree(h->w_igemm);
+    (void)hipFree(h->w_dw);
+    (void)hipFree(h->scale_in);
+    (void)hipFree(h->bias);
+    (void)hipFree(h->scale_out);
+    (void)hipFree(h->in_scale);
+    delete h;
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight, const float* scale_in,
+                          const float* bias, float in_scale, const float* out_scale, int n_out_scale,
+                          otter_hip_conv_t** handle) {
+    if (!desc || !weight || !scale_in || !handle) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: null");
+    const otter_hip_conv_desc& d = *desc;
+    if (d.in_channels < 1 || d.out_channels < 1 || d.kernel_h < 1 || d.kernel_w < 1 || d.stride_h < 1 ||
+        d.stride_w < 1 || d.pad_h < 0 || d.pad_w < 0 || d.dilation_h < 1 || d.dilation_w < 1 || d.groups < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: bad geometry");
+    if (d.in_channels % d.groups || d.out_channels % d.groups)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: channels not divisible by groups");
+    if (d.out_kind < OTTER_HIP_OUT_I32 || d.out_kind > OTTER_HIP_OUT_I8)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: bad out_kind");
+    if (d.activation_type < 0 || d.activation_type > 4)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_create: activation type not supported");
+    if (d.out_kind == OTTER_HIP_OUT_I8 && (!out_scale || (n_out_scale != 1 && n_out_scale != d.out_channels)))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: int8 output needs 1 or K output scales");
+
+    otter_hip_conv* h = new (std::nothrow) otter_hip_conv();
+    if (!h) return fail(OTTER_HIP_ERR_ALLOC, "otter_hip_conv_create: host allocation failed");
+    h->d = d;
+    const int K = d.out_channels, C = d.in_channels, g = d.groups, maxk = d.kernel_h * d.kernel_w;
+    h->depthwise = (C == g && g == K);
+    const int kpad = (K + 31) / 32 * 32;
+    int rc = OTTER_HIP_OK;
+    do {
+        const size_t wcount = (size_t)K * (C / g) * maxk;
+        if ((rc = upload<int8_t>(&h->w_raw, weight, wcount, wcount, 0))) break;
+        if ((rc = upload<float>(&h->scale_in, scale_in, K, kpad, 0.f))) break;
+        if (bias && (rc = upload<float>(&h->bias, bias, K, kpad, 0.f))) break;
+        if (d.out_kind == OTTER_HIP_OUT_I8) {
+            std::vector<float> so(K);
+            for (int i = 0; i < K; ++i) so[i] = n_out_scale == 1 ? out_scale[0] : out_scale[i];
+            if ((rc = upload<float>(&h->scale_out, so.data(), K, kpad, 1.f))) break;
+        }
+        if ((rc = upload<float>(&h->in_scale, &in_scale, 1, 1, 0.f))) break;
+        if (h->depthwise && C % 8 == 0) {
+            std::vector<int32_t> wm(dw_packed_weight_bytes(C, d.kernel_h, d.kernel_w) / sizeof(int32_t));
+            dw_pack_weights(weight, C, d.kernel_h, d.kernel_w, wm.data());
+            if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
+        } else if (g == 1 && C % 8 == 0) {
+            std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
+            igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
+            if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
+        }
+    } while (0);
+    if (rc != OTTER_HIP_OK) {
+        std::string keep = g_last_error;
+        otter_hip_conv_destroy(h);
+        g_last_error = keep;
+        return rc;
+    }
+    *handle = h;
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_conv_output_shape(const otter_hip_conv_t* h, int in_h, int in_w, int* out_h, int* out_w) {
+    if (!h || !out_h || !out_w) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_output_shape: null");
+    *out_h = conv_out_size(in_h, h->d.kernel_h, h->d.stride_h, h->d.pad_h, h->d.dilation_h);
+    *out_w = conv_out_size(in_w, h->d.kernel_w, h->d.stride_w, h->d.pad_w, h->d.dilation_w);
+    if (*out_h < 1 || *out_w < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_output_shape: empty output");
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_conv_default_out_layout(const otter_hip_conv_t* h) {
+    if (!h) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_default_out_layout: null");
+    const int K = h->d.out_channels;
+    const bool dw8 = h->depthwise && K % 8 == 0;
+    switch (h->d.out_kind) {
+    case OTTER_HIP_OUT_I32:
+        return dw8 ? OTTER_HIP_I32_P8 : (K % 4 == 0 ? OTTER_HIP_I32_P4 : OTTER_HIP_I32);
+    case OTTER_HIP_OUT_F32:
+        return dw8 ? OTTER_HIP_F32_P8 : (K % 4 == 0 ? OTTER_HIP_F32_P4 : OTTER_HIP_F32);
+    default:
+        return K % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
+    }
+}
+
+size_t otter_hip_conv_workspace_bytes(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w) {
+    if (!h || !valid_layout(in_layout) || layout_elem(in_layout) != 0) return 0;
+    return (size_t)n * h->d.in_channels * in_h * in_w;
+}
+
+// testing / tuning hook: force the MFMA tile shape of a handle (0,0 = automatic)
+int otter_hip_conv_set_tile(otter_hip_conv_t* h, int tm, int tn) {
+    if (!h) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_set_tile: null");
+    h->force_tm = tm;
+    h->force_tn = tn;
+    return OTTER_HIP_OK;
+}
+
+static int pick_kernel(const otter_hip_conv* h, int int8_layout) {
+    if (int8_layout == OTTER_HIP_I8_P8) {
+        if (h->w_dw) return 2;
+        if (h->w_igemm) return 1;
+    }
+    return 0;
+}
+
+int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int, int, int, int) {
+    if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
+    int l = in_layout;
+    if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
+    return pick_kernel(h, l);
+}
+
+int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
+                           void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream_) {
+    if (!h || !in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: null");
+    if (!valid_layout(in_layout) || !valid_layout(out_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: unknown layout");
+    const otter_hip_conv_desc& d = h->d;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n < 0 || in_h < 1 || in_w < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: bad shape");
+    if (layout_elem(in_layout) == 2) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: int32 input");
+    if (d.in_channels % layout_pack(in_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: input pack does not divide C");
+    const int want_elem = d.out_kind == OTTER_HIP_OUT_F32 ? 0 : (d.out_kind == OTTER_HIP_OUT_I8 ? 1 : 2);
+    if (layout_elem(out_layout) != want_elem)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: output layout does not match out_kind");
+    if (d.out_channels % layout_pack(out_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: output pack does not divide K");
+
+    ConvGeom g;
+    g.N = n, g.C = d.in_channels, g.H = in_h, g.W = in_w, g.K = d.out_channels;
+    g.kh = d.kernel_h, g.kw = d.kernel_w, g.sh = d.stride_h, g.sw = d.stride_w, g.ph = d.pad_h, g.pw = d.pad_w;
+    g.dh = d.dilation_h, g.dw = d.dilation_w, g.groups = d.groups;
+    g.OH = conv_out_size(in_h, d.kernel_h, d.stride_h, d.pad_h, d.dilation_h);
+    g.OW = conv_out_size(in_w, d.kernel_w, d.stride_w, d.pad_w, d.dilation_w);
+    if (g.OH < 1 || g.OW < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: empty output");
+    if ((size_t)n * g.C * in_h * in_w >= (1ull << 31) || (size_t)n * g.K * g.OH * g.OW >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
+    if (n == 0) return OTTER_HIP_OK;
+
+    // (1) quantize_to_int8 when the blob is not int8 yet (Tensor/ConvolutionLayer.cpp:770-775)
+    const int8_t* xq = (const int8_t*)in;
+    int q_layout = in_layout;
+    if (layout_elem(in_layout) == 0) {
+        const size_t need = (size_t)n * g.C * in_h * in_w;
+        if (!workspace || workspace_bytes < need)
+            return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: fp32 input needs a workspace of N*C*H*W bytes");
+        q_layout = g.C % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
+        OHIP_CHECK(run_quantize((const float*)in, layout_pack(in_layout), (int8_t*)workspace, layout_pack(q_layout), n,
+                                g.C, in_h * in_w, h->in_scale, 1, d.in_round_mode, stream));
+        xq = (const int8_t*)workspace;
+    }
+
+    Epilogue ep;
+    ep.scale_in = h->scale_in, ep.bias = h->bias, ep.scale_out = h->scale_out;
+    ep.act = d.activation_type, ep.act_p0 = d.activation_param0, ep.round_mode = d.out_round_mode;
+    ep.out_kind = d.out_kind, ep.out_layout = out_layout;
+
+    // (2)+(3)+(4) convolution with the fused epilogue
+    switch (pick_kernel(h, q_layout)) {
+    case 2:
+        if ((long)n * (g.C / 8) > 65535) {
+            // the plane index rides on grid.y: run the batch in slices
+            const int per = 65535 / (g.C / 8);
+            if (per < 1) return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: too many channels");
+            for (int b = 0; b < n; b += per) {
+                ConvGeom gs = g;
+                gs.N = (n - b < per) ? n - b : per;
+                const size_t in_off = (size_t)b * g.C * in_h * in_w;
+                const size_t out_off = (size_t)b * g.K * g.OH * g.OW * layout_elem_bytes(out_layout);
+                OHIP_CHECK(run_conv_dw(xq + in_off, h->w_dw, (char*)out + out_off, gs, ep, stream));
+            }
+        } else {
+            OHIP_CHECK(run_conv_dw(xq, h->w_dw, out, g, ep, stream));
+        }
+        break;
+    case 1:
+        OHIP_CHECK(run_conv_igemm(xq, h->w_igemm, out, g, ep, h->force_tm, h->force_tn, stream));
+        break;
+    default:
+        OHIP_CHECK(run_conv_direct(xq, layout_pack(q_layout), h->w_raw, out, g, ep, stream));
+        break;
+    }
+    return OTTER_HIP_OK;
+}
+
+// -----------------------------------------------------------------------------------------------------
+// standalone quantize / dequantize / requantize / repack
+// -----------------------------------------------------------------------------------------------------
+
+static int check_ew(const char* who, const void* src, const void* dst, int sl, int dl, int se, int de, int n, int c,
+                    int h, int w) {
+    if (!src || !dst) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": null");
+    if (!valid_layout(sl) || !valid_layout(dl) || layout_elem(sl) != se || layout_elem(dl) != de)
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": layout / element type mismatch");
+    if (n < 0 || c < 1 || h < 1 || w < 1) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": bad shape");
+    if (c % layout_pack(sl) || c % layout_pack(dl))
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": pack does not divide C");
+    if ((size_t)n * c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, std::string(who) + ": tensor exceeds 2^31 elements");
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_quantize(const float* src, int src_layout, int n, int c, int h, int w, const float* scales, int n_scales,
+                       int round_mode, int8_t* dst, int dst_layout, void* stream) {
+    if (int rc = check_ew("otter_hip_quantize", src, dst, src_layout, dst_layout, 0, 1, n, c, h, w)) return rc;
+    if (!scales || (n_scales != 1 && n_scales != c))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_quantize: need 1 or C scales");
+    OHIP_CHECK(run_quantize(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h * w, scales, n_scales,
+                            round_mode, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_dequantize(const int32_t* src, int src_layout, int n, int c, int h, int w, const float* scale,
+                         int n_scale, const float* bias, int n_bias, float* dst, int dst_layout, void* stream) {
+    if (int rc = check_ew("otter_hip_dequantize", src, dst, src_layout, dst_layout, 2, 0, n, c, h, w)) return rc;
+    if (!scale || (n_scale != 1 && n_scale != c))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_dequantize: need 1 or C scales");
+    if (!bias) n_bias = 0;
+    if (n_bias != 0 && n_bias != 1 && n_bias != c)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_dequantize: need 0, 1 or C biases");
+    OHIP_CHECK(run_dequantize(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h * w, scale, n_scale,
+                              bias, n_bias, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_requantize(const int32_t* src, int src_layout, int n, int c, int h, int w, const float* scale_in,
+                         int n_scale_in, const float* scale_out, int n_scale_out, const float* bias, int n_bias,
+                         int activation_type, float activation_param0, int round_mode, int8_t* dst, int dst_layout,
+                         void* stream) {
+    if (int rc = check_ew("otter_hip_requantize", src, dst, src_layout, dst_layout, 2, 1, n, c, h, w)) return rc;
+    if (!scale_in || (n_scale_in != 1 && n_scale_in != c) || !scale_out || (n_scale_out != 1 && n_scale_out != c))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_requantize: need 1 or C scales");
+    if (!bias) n_bias = 0;
+    if (n_bias != 0 && n_bias != 1 && n_bias != c)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_requantize: need 0, 1 or C biases");
+    if (activation_type < 0 || activation_type > 4)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_requantize: activation type not supported");
+    OHIP_CHECK(run_requantize(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h * w, scale_in,
+                              n_scale_in, scale_out, n_scale_out, bias, n_bias, activation_type, activation_param0,
+                              round_mode, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_repack(const void* src, int src_layout, int n, int c, int h, int w, void* dst, int dst_layout,
+                     void* stream) {
+    if (!valid_layout(src_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_repack: unknown layout");
+    const int e = layout_elem(src_layout);
+    if (int rc = check_ew("otter_hip_repack", src, dst, src_layout, dst_layout, e, e, n, c, h, w)) return rc;
+    OHIP_CHECK(run_repack(src, layout_pack(src_layout), dst, layout_pack(dst_layout), layout_elem_bytes(src_layout), n,
+                          c, h * w, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+}  // extern "C"

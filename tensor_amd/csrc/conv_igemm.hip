@@ -1,0 +1,264 @@
+// Dense int8 convolution as an implicit GEMM on the gfx950 matrix cores (v_mfma_i32_16x16x64_i8).
+//
+//   D[M = out channel][N = pixel] = sum_k  Wp[M][k] * X[k][N],   k = (tap, input channel)
+//
+// Activations stay in the reference's Byte8 layout [N, C/8, H, W, 8] (no im2col, no padded copy): a k-chunk
+// of 64 is one filter tap x 64 input channels = 8 channel octets of one input pixel, and a lane's 16-byte
+// MFMA operand is two neighbouring octets. Out-of-image taps are predicated to zero.
+// Weights are re-laid-out once on the host into the exact lane order the MFMA consumes
+// ([k-chunk][16-row tile][lane][16 B]), so the global->LDS copy and the LDS->register reads are linear.
+// Output rows are permuted (see igemm_row_channel) so that after the MFMA each lane owns 8 consecutive output
+// channels of one pixel: one 8-byte Byte8 store, or two 16-byte Float4 / Int4 stores, per lane, with the 16
+// lanes of a row group covering 16 consecutive pixels -- the reference's packed layouts come out directly.
+#include "common.hpp"
+#include "conv_igemm.hpp"
+
+namespace ohip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+template <int TM, int TN, int WM, int WN>
+struct IgemmCfg {
+    static constexpr int kThreads = 256;
+    static constexpr int FM = TM / WM / 16;          // 16-row fragments per wave
+    static constexpr int FN = TN / WN / 16;          // 16-pixel fragments per wave
+    static constexpr int A_BYTES = TM * 64;          // weights per k-chunk
+    static constexpr int B_BYTES = TN * 64;          // activations per k-chunk
+    static constexpr int A_V = (A_BYTES / 16 + kThreads - 1) / kThreads;  // 16-byte vectors per thread
+    static constexpr int B_V = TN / 64;                                   // (pixel, octet pair) items per thread
+    static_assert(WM * WN == 4, "four waves");
+    static_assert(FM >= 2 && FM % 2 == 0, "row fragments come in pairs");
+    static_assert(TN % 64 == 0, "pixel tile");
+};
+
+template <int TM, int TN, int WM, int WN>
+__global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
+                                                         void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
+                                                         int c_groups, int n_pix_tiles) {
+    using Cfg = IgemmCfg<TM, TN, WM, WN>;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN;
+    __shared__ __attribute__((aligned(16))) int8_t lds_a[2][Cfg::A_BYTES];
+    __shared__ __attribute__((aligned(16))) int8_t lds_b[2][Cfg::B_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+
+    // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of pixel tiles so
+    // that neighbouring tiles (which share halo rows and all weights) meet in the same L2.
+    int pt = blockIdx.x;
+    {
+        const int per = n_pix_tiles / 8;
+        if (per > 0 && pt < per * 8) pt = (pt % 8) * per + pt / 8;
+    }
+    const int mt0 = blockIdx.y * (TM / 16);  // first 16-row tile of this workgroup
+    const int OHW = g.OH * g.OW;
+    const long total_pix = (long)g.N * OHW;
+    const long tile_base = (long)pt * TN;
+    const int C8 = g.C / 8;
+    const int HW = g.H * g.W;
+
+    // ---- per-thread constants of the activation loader -------------------------------------------
+    const int p_l = tid % TN;
+    const int j0 = tid / TN;
+    constexpr int J_STEP = 256 / TN > 0 ? 256 / TN : 1;
+    const long gp = tile_base + p_l;
+    const bool pvalid = gp < total_pix;
+    int iy0 = 0, ix0 = 0;
+    const int8_t* xn = x;
+    if (pvalid) {
+        const int n = (int)(gp / OHW);
+        const int pix = (int)(gp % OHW);
+        const int oy = pix / g.OW, ox = pix % g.OW;
+        iy0 = oy * g.sh - g.ph;
+        ix0 = ox * g.sw - g.pw;
+        xn = x + (size_t)n * C8 * HW * 8;
+    }
+
+    v2i breg[Cfg::B_V][2];
+    v4i areg[Cfg::A_V];
+    const int n_chunks = g.kh * g.kw * c_groups;
+
+    auto load_global = [&](int kc) {
+        const int tap = kc / c_groups, cgp = kc % c_groups;
+        const int u = tap / g.kw, v = tap % g.kw;
+        const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
+        const bool inb = pvalid && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+        const int8_t* px = xn + ((size_t)iy * g.W + ix) * 8;
+#pragma unroll
+        for (int r = 0; r < Cfg::B_V; ++r) {
+            const int o0 = cgp * 8 + 2 * (j0 + r * J_STEP);
+            v2i lo = {0, 0}, hi = {0, 0};
+            if (inb && o0 < C8) lo = *reinterpret_cast<const v2i*>(px + (size_t)o0 * HW * 8);
+            if (inb && o0 + 1 < C8) hi = *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * HW * 8);
+            breg[r][0] = lo;
+            breg[r][1] = hi;
+        }
+        const int8_t* wa = wpk + ((size_t)kc * m_tiles16 + mt0) * 1024;
+#pragma unroll
+        for (int r = 0; r < Cfg::A_V; ++r) {
+            const int vi = tid + r * 256;
+            if (vi * 16 < Cfg::A_BYTES) areg[r] = *reinterpret_cast<const v4i*>(wa + (size_t)vi * 16);
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < Cfg::B_V; ++r) {
+            const int j = j0 + r * J_STEP;
+            v4i t = {breg[r][0][0], breg[r][0][1], breg[r][1][0], breg[r][1][1]};
+            *reinterpret_cast<v4i*>(&lds_b[buf][(j * TN + p_l) * 16]) = t;
+        }
+#pragma unroll
+        for (int r = 0; r < Cfg::A_V; ++r) {
+            const int vi = tid + r * 256;
+            if (vi * 16 < Cfg::A_BYTES) *reinterpret_cast<v4i*>(&lds_a[buf][vi * 16]) = areg[r];
+        }
+    };
+
+    v4i acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int kc = 0; kc < n_chunks; ++kc) {
+        const int buf = kc & 1;
+        if (kc + 1 < n_chunks) load_global(kc + 1);
+        v4i a[FM], b[FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+            a[i] = *reinterpret_cast<const v4i*>(&lds_a[buf][((wm * FM + i) * 64 + lane) * 16]);
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+            b[j] = *reinterpret_cast<const v4i*>(
+                &lds_b[buf][((lane >> 4) * TN + wn * (TN / WN) + j * 16 + (lane & 15)) * 16]);
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        if (kc + 1 < n_chunks) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------------
+    const int gq = lane >> 4;
+    const bool has_bias = ep.bias != nullptr;
+#pragma unroll
+    for (int ip = 0; ip < FM / 2; ++ip) {
+        const int tpair = (mt0 + wm * FM) / 2 + ip;
+        const int ch0 = 32 * tpair + 8 * gq;  // this lane's 8 consecutive output channels
+        if (ch0 >= g.K) continue;
+        float si[8], bi[8], so[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            si[e] = ep.scale_in[ch0 + e];
+            bi[e] = has_bias ? ep.bias[ch0 + e] : 0.f;
+            so[e] = ep.scale_out ? ep.scale_out[ch0 + e] : 1.f;
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const long gpo = tile_base + wn * (TN / WN) + j * 16 + (lane & 15);
+            if (gpo >= total_pix) continue;
+            const int n = (int)(gpo / OHW);
+            const int pix = (int)(gpo % OHW);
+            int a8[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a8[e] = acc[2 * ip][j][e];
+                a8[4 + e] = acc[2 * ip + 1][j][e];
+            }
+            epilogue_store8(out, ep, n, ch0, pix, g.K, OHW, a8, si, bi, so);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------------
+
+int igemm_padded_rows(int K) { return (K + 31) / 32 * 32; }
+int igemm_channel_groups(int C) { return (C + 63) / 64; }
+
+// physical GEMM row -> logical output channel (rows of a pair of 16-row tiles are interleaved in fours, so
+// that MFMA lane group q of the pair ends up with channels 32*pair + 8*q .. +7)
+int igemm_row_channel(int row) {
+    const int mt = row / 16, r = row % 16;
+    return 32 * (mt / 2) + 8 * (r / 4) + 4 * (mt % 2) + (r % 4);
+}
+
+size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw) {
+    return (size_t)kh * kw * igemm_channel_groups(C) * (igemm_padded_rows(K) / 16) * 1024;
+}
+
+// weight [K, C, kh, kw] int8 -> [k-chunk = (tap, channel group)][16-row tile][lane][16 bytes]
+void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst) {
+    const int mt16 = igemm_padded_rows(K) / 16, cgs = igemm_channel_groups(C);
+    size_t o = 0;
+    for (int tap = 0; tap < kh * kw; ++tap)
+        for (int cg = 0; cg < cgs; ++cg)
+            for (int mt = 0; mt < mt16; ++mt)
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int ch = igemm_row_channel(mt * 16 + (lane & 15));
+                    for (int b = 0; b < 16; ++b, ++o) {
+                        const int c = cg * 64 + (lane >> 4) * 16 + b;
+                        dst[o] = (ch < K && c < C) ? w[((size_t)ch * C + c) * kh * kw + tap] : 0;
+                    }
+                }
+}
+
+template <int TM, int TN, int WM, int WN>
+static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                               hipStream_t stream) {
+    const long total_pix = (long)g.N * g.OH * g.OW;
+    const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
+    const int mpad = igemm_padded_rows(g.K);
+    const int m_tiles = (mpad + TM - 1) / TM;
+    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN>), dim3(n_pix_tiles, m_tiles), dim3(256), 0, stream, x, wpk,
+                       out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
+    return hipGetLastError();
+}
+
+// tile choice: the widest row tile that does not pad M further, then the widest pixel tile that still
+// leaves at least two workgroups per compute unit
+void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
+    const int mpad = igemm_padded_rows(g.K);
+    int TM = 32;
+    if (mpad % 128 == 0) TM = 128;
+    else if (mpad % 64 == 0) TM = 64;
+    const long total_pix = (long)g.N * g.OH * g.OW;
+    const long m_tiles = mpad / TM;
+    int TN = 64;
+    if (((total_pix + 255) / 256) * m_tiles >= 512) TN = 256;
+    else if (((total_pix + 127) / 128) * m_tiles >= 512) TN = 128;
+    *tm = TM;
+    *tn = TN;
+}
+
+hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                          int tm, int tn, hipStream_t stream) {
+    if (tm == 0 || tn == 0) igemm_choose_tiles(g, &tm, &tn);
+    // a row tile must not reach past the padded weight rows
+    if (igemm_padded_rows(g.K) % tm != 0) return hipErrorInvalidValue;
+#define OHIP_IG(TM_, TN_, WM_, WN_) \
+    if (tm == TM_ && tn == TN_) return launch_igemm<TM_, TN_, WM_, WN_>(x, wpk, out, g, ep, stream);
+    OHIP_IG(128, 256, 2, 2)
+    OHIP_IG(128, 128, 2, 2)
+    OHIP_IG(128, 64, 4, 1)
+    OHIP_IG(64, 256, 2, 2)
+    OHIP_IG(64, 128, 2, 2)
+    OHIP_IG(64, 64, 2, 2)
+    OHIP_IG(32, 256, 1, 4)
+    OHIP_IG(32, 128, 1, 4)
+    OHIP_IG(32, 64, 1, 4)
+#undef OHIP_IG
+    return hipErrorInvalidValue;
+}
+
+}  // namespace ohip

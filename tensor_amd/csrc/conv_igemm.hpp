@@ -1,0 +1,38 @@
+// Host interface of the MFMA implicit-GEMM convolution (conv_igemm.hip) and the other kernel families.
+#pragma once
+#include "common.hpp"
+
+namespace ohip {
+
+// conv_igemm.hip
+int igemm_padded_rows(int K);
+int igemm_channel_groups(int C);
+int igemm_row_channel(int row);
+size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw);
+void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst);
+void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn);
+hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep, int tm,
+                          int tn, hipStream_t stream);
+
+// conv_direct.hip
+hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void* out, const ConvGeom& g,
+                           const Epilogue& ep, hipStream_t stream);
+
+// conv_dw.hip
+size_t dw_packed_weight_bytes(int C, int kh, int kw);
+void dw_pack_weights(const int8_t* w, int C, int kh, int kw, int32_t* dst);
+hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const ConvGeom& g, const Epilogue& ep,
+                       hipStream_t stream);
+
+// elementwise.hip
+hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,
+                        int n_scales, int round_mode, hipStream_t stream);
+hipError_t run_dequantize(const int32_t* src, int sp, float* dst, int dp, int N, int C, int HW, const float* scale,
+                          int n_scale, const float* bias, int n_bias, hipStream_t stream);
+hipError_t run_requantize(const int32_t* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scale_in,
+                          int n_scale_in, const float* scale_out, int n_scale_out, const float* bias, int n_bias,
+                          int act, float act_p0, int round_mode, hipStream_t stream);
+hipError_t run_repack(const void* src, int sp, void* dst, int dp, int elem_bytes, int N, int C, int HW,
+                      hipStream_t stream);
+
+}  // namespace ohip

@@ -1,0 +1,50 @@
+"""Helpers shared by the GPU parity tests: run one ConvolutionLayer-shaped problem through the C ABI."""
+import numpy as np
+
+from tensor_amd import capi
+
+ACT = {"": 0, "Relu": 1, "LRelu": 2, "Relu6": 3}
+
+
+def in_layout_for(x, C):
+    """The layout Net::convert_layout hands to the layer (Tensor/Net.cpp:388-405)."""
+    if x.dtype == np.int8:
+        return capi.I8_P8 if C % 8 == 0 else capi.I8
+    if C % 8 == 0:
+        return capi.F32_P8
+    if C % 4 == 0:
+        return capi.F32_P4
+    return capi.F32
+
+
+def host_scale_in(w_scales, in_scale):
+    """ConvolutionLayer::create_pipeline_int8 (Tensor/ConvolutionLayer.cpp:667-679) as the host does it."""
+    ws = np.asarray(w_scales, np.float32)
+    with np.errstate(divide="ignore"):
+        si = (np.float32(1.0) / (np.float32(in_scale) * ws)).astype(np.float32)
+    si[ws == 0] = 0
+    return si
+
+
+def run_conv(hip, oracle, x, wq, w_scales, in_scale, *, stride=1, pad=0, dil=1, groups=1, bias=None, top_scale=1.0,
+             out_kind=capi.OUT_I32, act=0, act_p0=0.0, out_layout=None, in_layout=None, tile=None):
+    """x: NCHW numpy (fp32 or int8). Returns the NCHW numpy result of the GPU layer."""
+    n, C, H, W = x.shape
+    K = wq.shape[0]
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(np.broadcast_to(w_scales, (K,)), in_scale), bias=bias,
+                    in_scale=float(in_scale), out_scale=[top_scale] if out_kind == capi.OUT_I8 else None,
+                    stride=(stride, stride), pad=(pad, pad), dil=(dil, dil), groups=groups, act=act, act_p0=act_p0,
+                    out_kind=out_kind, out_round=oracle.requantize_round_mode(C, K, groups, True),
+                    in_round=oracle.quantize_round_mode(C, True))
+    if tile is not None:
+        conv.set_tile(*tile)
+    in_layout = in_layout_for(x, C) if in_layout is None else in_layout
+    out_layout = conv.default_out_layout() if out_layout is None else out_layout
+    xd = hip.to_device(capi.pack_np(x, capi.layout_pack(in_layout)))
+    out = conv.forward(xd, in_layout, n, H, W, out_layout)
+    hip.torch.cuda.synchronize()
+    oh, ow = conv.out_hw(H, W)
+    kind = conv.kernel_kind(in_layout, n, H, W, out_layout)
+    res = capi.unpack_np(out.cpu().numpy(), capi.layout_pack(out_layout), (n, K, oh, ow))
+    conv.close()
+    return res, kind

@@ -1,0 +1,253 @@
+"""GPU parity tests proper: the HIP path, called through the C ABI, against (a) the golden vectors produced by
+the compiled reference and (b) the CPU oracle on seeded inputs. int32 accumulators and int8 outputs must be
+bit-exact; fp32 outputs within 1e-5 relative (they are in fact reproduced bitwise, which is asserted too)."""
+import numpy as np
+import pytest
+
+from cases import LAYER_CASES
+from gpu_util import ACT, run_conv
+from oracle.binding import ROUND_EXACT, ROUND_SSE
+from tensor_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+FP32_RTOL = 1e-5
+
+
+def assert_f32_close(got, want):
+    np.testing.assert_allclose(got, want, rtol=FP32_RTOL, atol=1e-30)
+
+
+def _g(golden, tag, key):
+    return golden.get(tag + "/" + key)
+
+
+@pytest.mark.parametrize("case", LAYER_CASES, ids=[c[0] for c in LAYER_CASES])
+def test_layer_against_reference_vectors(hip, oracle, golden, case):
+    name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params = case
+    x, wq = _g(golden, name, "x"), _g(golden, name, "wq")
+    common = dict(stride=s, pad=p, dil=d, groups=g, bias=_g(golden, name, "bias"),
+                  top_scale=float(_g(golden, name, "top_scale")), act=ACT[act],
+                  act_p0=float(act_params[0]) if act_params else 0.0)
+    ws, ins = _g(golden, name, "w_scales"), float(_g(golden, name, "in_scale"))
+    # raw accumulators (what otter::convolution returns)
+    acc, kind = run_conv(hip, oracle, x, wq, ws, ins, out_kind=capi.OUT_I32, **common)
+    np.testing.assert_array_equal(acc, _g(golden, name, "acc"))
+    # the layer output, in the reference's default packed layout and unpacked
+    want = _g(golden, name, "out")
+    kind_out = capi.OUT_I8 if i8_out else capi.OUT_F32
+    for out_layout in (None, capi.I8 if i8_out else capi.F32):
+        out, _ = run_conv(hip, oracle, x, wq, ws, ins, out_kind=kind_out, out_layout=out_layout, **common)
+        if i8_out:
+            np.testing.assert_array_equal(out, want)
+        else:
+            assert_f32_close(out, want)
+            np.testing.assert_array_equal(out.view(np.int32), want.view(np.int32))
+    # the fast kernels must be the ones that ran, not the scalar fallback
+    if C % 8 == 0 and (g == 1 or g == C == K):
+        assert kind in (1, 2, 3)
+
+
+def test_layer_unpacked_input_layouts(hip, oracle, golden):
+    """The same blob handed over unpacked (fp32 NCHW / int8 NCHW) gives the same answer."""
+    for case in LAYER_CASES[:3] + LAYER_CASES[14:16]:
+        name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params = case
+        x = _g(golden, name, "x")
+        out, _ = run_conv(hip, oracle, x, _g(golden, name, "wq"), _g(golden, name, "w_scales"),
+                          float(_g(golden, name, "in_scale")), stride=s, pad=p, dil=d, groups=g,
+                          bias=_g(golden, name, "bias"), top_scale=float(_g(golden, name, "top_scale")), act=ACT[act],
+                          out_kind=capi.OUT_I8 if i8_out else capi.OUT_F32,
+                          in_layout=capi.I8 if in_i8 else capi.F32)
+        want = _g(golden, name, "out")
+        if i8_out:
+            np.testing.assert_array_equal(out, want)
+        else:
+            assert_f32_close(out, want)
+
+
+# ---- standalone quantize / requantize / dequantize against the reference's fine-print vectors ----------
+
+@pytest.mark.parametrize("C,packing", [(8, True), (8, False), (4, True), (4, False), (3, True), (3, False)])
+def test_quantize_near_ties(hip, oracle, golden, C, packing):
+    tag = "quant_ties/C%d_pack%d" % (C, int(packing))
+    x, want = golden[tag + "/x"], golden[tag + "/q"]
+    # |x*scale| >= 2^31 is outside the supported domain (x86 integer-indefinite artefact)
+    ok = np.abs(x) < 2.0 ** 31
+    mode = oracle.quantize_round_mode(C, packing)
+    sp = (8 if C % 8 == 0 else 4 if C % 4 == 0 else 1) if packing else 1
+    dp = 8 if (packing and C % 8 == 0) else 1
+    src = hip.to_device(capi.pack_np(x, sp))
+    scales = hip.to_device(np.ones(1, np.float32))
+    q = hip.quantize(src, capi.layout_for(np.float32, sp), x.shape, scales, mode, capi.layout_for(np.int8, dp))
+    got = capi.unpack_np(q.cpu().numpy(), dp, x.shape)
+    np.testing.assert_array_equal(got[ok], want[ok])
+
+
+def test_quantize_per_channel(hip, golden):
+    x, ps = golden["quant_perchannel/x"], golden["quant_perchannel/scales"]
+    for sp in (1, 4, 8):
+        for dp in (1, 8):
+            q = hip.quantize(hip.to_device(capi.pack_np(x, sp)), capi.layout_for(np.float32, sp), x.shape,
+                             hip.to_device(ps), ROUND_SSE, capi.layout_for(np.int8, dp))
+            np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), dp, x.shape), golden["quant_perchannel/q"])
+
+
+@pytest.mark.parametrize("C", [8, 4, 6])
+@pytest.mark.parametrize("packing", [True, False])
+def test_requantize_exact_ties(hip, golden, C, packing):
+    for j in range(4):
+        tag = "requant_ties/C%d_pack%d_b%d" % (C, int(packing), j)
+        mode = ROUND_SSE if (packing and C % 4 == 0) else ROUND_EXACT
+        acc = golden[tag + "/acc"]
+        sp = 4 if (packing and C % 4 == 0) else 1
+        dp = 8 if (packing and C % 8 == 0) else 1
+        bias = golden.get(tag + "/bias")
+        q = hip.requantize(hip.to_device(capi.pack_np(acc, sp)), capi.layout_for(np.int32, sp), acc.shape,
+                           hip.to_device(golden[tag + "/scale_in"]), hip.to_device(golden[tag + "/scale_out"]),
+                           None if bias is None else hip.to_device(bias), 0, 0.0, mode, capi.layout_for(np.int8, dp))
+        np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), dp, acc.shape), golden[tag + "/q"])
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3])
+@pytest.mark.parametrize("C,packing", [(8, True), (12, True), (6, True), (8, False)])
+def test_requantize_random(hip, golden, act, C, packing):
+    tag = "requant_rand/act%d_C%d_pack%d" % (act, C, int(packing))
+    mode = ROUND_SSE if (packing and C % 4 == 0) else ROUND_EXACT
+    acc = golden[tag + "/acc"]
+    ap = golden.get(tag + "/act_params")
+    for sp in ((1, 4, 8) if C % 8 == 0 else (1, 4) if C % 4 == 0 else (1,)):
+        for dp in ((1, 8) if C % 8 == 0 else (1,)):
+            q = hip.requantize(hip.to_device(capi.pack_np(acc, sp)), capi.layout_for(np.int32, sp), acc.shape,
+                               hip.to_device(golden[tag + "/scale_in"]), hip.to_device(golden[tag + "/scale_out"]),
+                               hip.to_device(golden[tag + "/bias"]), act, float(ap[0]) if ap is not None else 0.0,
+                               mode, capi.layout_for(np.int8, dp))
+            np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), dp, acc.shape), golden[tag + "/q"])
+
+
+@pytest.mark.parametrize("C,packing", [(8, True), (4, True), (8, False)])
+def test_dequantize_bitwise(hip, golden, C, packing):
+    for j in (0, 1):
+        tag = "dequant/C%d_pack%d_b%d" % (C, int(packing), j)
+        acc, bias = golden[tag + "/acc"], golden.get(tag + "/bias")
+        for sp in ((1, 4, 8) if C % 8 == 0 else (1, 4)):
+            for dp in ((1, 4, 8) if C % 8 == 0 else (1, 4)):
+                y = hip.dequantize(hip.to_device(capi.pack_np(acc, sp)), capi.layout_for(np.int32, sp), acc.shape,
+                                   hip.to_device(golden[tag + "/scale"]),
+                                   None if bias is None else hip.to_device(bias), capi.layout_for(np.float32, dp))
+                got = capi.unpack_np(y.cpu().numpy(), dp, acc.shape)
+                assert_f32_close(got, golden[tag + "/y"])
+                np.testing.assert_array_equal(got.view(np.int32), golden[tag + "/y"].view(np.int32))
+
+
+def test_repack_roundtrip(hip):
+    rng = np.random.default_rng(3)
+    a = rng.integers(-100, 100, size=(2, 16, 5, 7)).astype(np.int8)
+    for sp in (1, 8):
+        for dp in (1, 8):
+            r = hip.repack(hip.to_device(capi.pack_np(a, sp)), capi.layout_for(np.int8, sp), a.shape,
+                           capi.layout_for(np.int8, dp))
+            np.testing.assert_array_equal(capi.unpack_np(r.cpu().numpy(), dp, a.shape), a)
+    f = rng.normal(size=(2, 16, 5, 7)).astype(np.float32)
+    for sp in (1, 4, 8):
+        for dp in (1, 4, 8):
+            r = hip.repack(hip.to_device(capi.pack_np(f, sp)), capi.layout_for(np.float32, sp), f.shape,
+                           capi.layout_for(np.float32, dp))
+            np.testing.assert_array_equal(capi.unpack_np(r.cpu().numpy(), dp, f.shape), f)
+
+
+# ---- seeded random shapes against the oracle: every MFMA tile shape, ragged pixel counts, odd channels ----
+
+def _rand_problem(rng, C, K, k, g, N, H, W, in_i8=True):
+    wq = rng.integers(-127, 128, size=(K, C // g, k, k)).astype(np.int8)
+    ws = rng.uniform(50, 400, K).astype(np.float32)
+    x = rng.integers(-127, 128, size=(N, C, H, W)).astype(np.int8) if in_i8 else \
+        rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
+    bias = rng.normal(0, 0.5, K).astype(np.float32)
+    return x, wq, ws, bias
+
+
+TILES = [(128, 256), (128, 128), (128, 64), (64, 256), (64, 128), (64, 64), (32, 256), (32, 128), (32, 64)]
+
+
+@pytest.mark.parametrize("tile", TILES, ids=["%dx%d" % t for t in TILES])
+def test_igemm_every_tile_shape(hip, oracle, tile):
+    rng = np.random.default_rng(tile[0] * 1000 + tile[1])
+    # K = 128 divides every row tile; 2 x 19 x 23 pixels leaves a ragged last pixel tile
+    for (C, K, k, s, p) in [(64, 128, 3, 1, 1), (24, 128, 1, 1, 0), (72, 128, 3, 2, 1)]:
+        x, wq, ws, bias = _rand_problem(rng, C, K, k, 1, 2, 19, 23)
+        in_scale = 31.75
+        want, acc_want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), bias=bias,
+                                                   top_scale=9.0, int8_out=True, act_type=1, want_acc=True)
+        acc, kind = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, out_kind=capi.OUT_I32, tile=tile)
+        assert kind == 1
+        np.testing.assert_array_equal(acc, acc_want)
+        out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, bias=bias, top_scale=9.0, act=1,
+                          out_kind=capi.OUT_I8, tile=tile)
+        np.testing.assert_array_equal(out, want)
+
+
+@pytest.mark.parametrize("C,K,k,s,p,d,g,N,H,W", [
+    (16, 24, 1, 1, 0, 1, 1, 3, 14, 14),     # MobileNetV2 project: K % 32 != 0
+    (96, 160, 1, 1, 0, 1, 1, 2, 7, 7),
+    (320, 1280, 1, 1, 0, 1, 1, 1, 7, 7),
+    (144, 24, 1, 1, 0, 1, 1, 2, 9, 9),
+    (8, 20, 3, 1, 1, 1, 1, 1, 9, 9),        # K % 8 != 0, K % 4 == 0 -> Int4 / Byte
+    (8, 10, 3, 2, 1, 1, 1, 2, 9, 7),        # K % 4 != 0 -> unpacked outputs
+    (32, 32, 3, 1, 2, 2, 1, 1, 11, 11),     # dilation
+    (16, 16, 3, 1, 1, 1, 2, 1, 8, 8),       # grouped, non-depthwise: scalar kernel
+    (6, 6, 3, 1, 1, 1, 6, 1, 8, 8),         # depthwise with C % 8 != 0: scalar kernel
+    (12, 8, 3, 1, 1, 1, 1, 1, 8, 8),        # C % 8 != 0
+    (64, 64, 3, 1, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s1, ragged strips
+    (64, 64, 3, 2, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s2
+    (16, 16, 7, 1, 3, 1, 16, 1, 12, 12),    # depthwise 7x7
+    (16, 16, 3, 1, 2, 2, 16, 1, 12, 12),    # depthwise dilated -> generic depthwise kernel
+    (128, 128, 3, 1, 1, 1, 1, 4, 56, 56),   # the c3 layer at reduced batch
+])
+def test_random_shapes_against_oracle(hip, oracle, C, K, k, s, p, d, g, N, H, W):
+    rng = np.random.default_rng(C * 7 + K * 3 + k + s + g)
+    x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W)
+    in_scale = 20.0
+    for int8_out, act in ((True, 3), (False, 1), (True, 2)):
+        want, acc_want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), dil=(d, d),
+                                                   groups=g, bias=bias, top_scale=11.0, int8_out=int8_out,
+                                                   act_type=act, act_params=[0.25], want_acc=True)
+        acc, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, dil=d, groups=g,
+                          out_kind=capi.OUT_I32)
+        np.testing.assert_array_equal(acc, acc_want)
+        out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, dil=d, groups=g, bias=bias,
+                          top_scale=11.0, act=act, act_p0=0.25,
+                          out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        if int8_out:
+            np.testing.assert_array_equal(out, want)
+        else:
+            assert_f32_close(out, want)
+
+
+def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
+    rng = np.random.default_rng(11)
+    for C in (3, 4, 8, 32):
+        x, wq, ws, bias = _rand_problem(rng, C, 16, 3, 1, 2, 9, 10, in_i8=False)
+        in_scale = np.float32(127) / np.abs(x).max()
+        want = oracle.conv_layer_forward(x, wq, ws, in_scale, pad=(1, 1), bias=bias, top_scale=15.0, int8_out=True,
+                                         act_type=1)
+        out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, pad=1, bias=bias, top_scale=15.0, act=1,
+                          out_kind=capi.OUT_I8)
+        np.testing.assert_array_equal(out, want)
+
+
+def test_error_codes(hip):
+    wq = np.zeros((8, 8, 3, 3), np.int8)
+    conv = hip.conv(wq=wq, scale_in=np.ones(8, np.float32), out_kind=capi.OUT_F32, pad=(1, 1))
+    x = hip.to_device(np.zeros(8 * 5 * 5, np.int8))
+    with pytest.raises(capi.HipError) as e:
+        conv.forward(x, capi.I8_P8, 1, 5, 5, out_layout=capi.I8_P8)  # element type does not match out_kind
+    assert e.value.code == -2
+    with pytest.raises(capi.HipError) as e:
+        conv.forward(x, capi.I32_P4, 1, 5, 5, out_layout=capi.F32_P4)  # int32 input
+    assert e.value.code == -2
+    with pytest.raises(capi.HipError) as e:
+        hip.conv(wq=np.zeros((9, 4, 3, 3), np.int8), scale_in=np.ones(9, np.float32), groups=2)  # K % groups != 0
+    assert e.value.code == -2
+    with pytest.raises(capi.HipError) as e:
+        hip.conv(wq=wq, scale_in=np.ones(8, np.float32), out_kind=capi.OUT_I8)  # int8 output without output scale
+    assert e.value.code == -2

@@ -1,0 +1,385 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 convolution path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c0|c4] [--no-cpu] [--no-also]
+
+Prints ONE JSON line. The headline workload is BASELINE.json configs[3] (the MFMA-bound case the metric's
+"int8 conv TOPS (% MFMA peak)" is quoted on): four chained int8-in/int8-out 3x3 convolutions 128->128 at
+56x56, batch 64, fused requantize+ReLU. One step = the four layers back to back on device-resident int8
+activations. The other single-GPU configurations (depthwise c1 at stride 1 and 2 with its HBM roofline, the
+1x1 GEMM c2, the single-image c0) are measured the same way and reported under "also".
+
+Timing: HIP events recorded on the stream the kernels are launched on (torch's current stream is handed to the
+C ABI as the launch stream), inputs resident in HBM before the timed region.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0    # MI355X HBM3E, GB/s
+
+
+def quantize_weights(wf):
+    K = wf.shape[0]
+    ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
+    wq = np.clip(np.round(wf * ws[:, None, None, None]), -127, 127).astype(np.int8)
+    return wq, ws
+
+
+def host_scale_in(ws, in_scale):
+    return (np.float32(1.0) / (np.float32(in_scale) * ws)).astype(np.float32)
+
+
+class Timer:
+    def __init__(self, torch):
+        self.torch = torch
+
+    def run(self, fn, steps, warmup):
+        t = self.torch
+        for _ in range(warmup):
+            fn()
+        t.cuda.synchronize()
+        e0, e1 = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+        wall0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        t.cuda.synchronize()
+        wall = (time.perf_counter() - wall0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall
+
+
+# ------------------------------------------------------------------------------------------------------
+# workloads
+# ------------------------------------------------------------------------------------------------------
+
+def build_c3(hip, capi, rng):
+    """configs[3]: 4 x (128->128 3x3 s1 p1) at 56x56, batch 64, int8 in / int8 out, requantize+ReLU. The output
+    scale of each layer is 127/max(activation) on a seeded calibration batch of 16, computed with the fp32-output
+    variant of the same GPU layer; the next layer's input scale is that output scale."""
+    torch = hip.torch
+    N, C, H, W, L = 64, 128, 56, 56, 4
+    x = rng.integers(-127, 128, size=(N, C, H, W), dtype=np.int8)
+    xc = rng.integers(-127, 128, size=(16, C, H, W), dtype=np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    cal = hip.to_device(capi.pack_np(xc, 8))
+    in_scale = np.float32(127.0)
+    layers, params = [], []
+    for l in range(L):
+        wq, ws = quantize_weights(rng.normal(0, 0.04, (C, C, 3, 3)).astype(np.float32))
+        bias = rng.normal(0, 0.01, C).astype(np.float32)
+        si = host_scale_in(ws, in_scale)
+        probe = hip.conv(wq=wq, scale_in=si, bias=bias, pad=(1, 1), act=1, out_kind=capi.OUT_F32)
+        amax = float(probe.forward(cal, capi.I8_P8, 16, H, W).abs().max().item())
+        probe.close()
+        out_scale = np.float32(127.0) / np.float32(amax)
+        conv = hip.conv(wq=wq, scale_in=si, bias=bias, out_scale=[out_scale], pad=(1, 1), act=1,
+                        out_kind=capi.OUT_I8, out_round=capi.ROUND_SSE)
+        cal = conv.forward(cal, capi.I8_P8, 16, H, W)
+        layers.append(conv)
+        params.append(dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale)))
+        in_scale = out_scale
+    bufs = [hip.empty(N * C * H * W, np.int8) for _ in range(2)]
+
+    def step():
+        src = xd
+        for l, conv in enumerate(layers):
+            dst = bufs[l & 1]
+            conv.forward(src, capi.I8_P8, N, H, W, capi.I8_P8, out=dst)
+            src = dst
+        return src
+
+    ops_layer = 2.0 * N * C * C * 9 * H * W
+    return dict(name="c3", step=step, ops=L * ops_layer, launches=L, dom_ops=ops_layer,
+                dom_bytes=2 * N * C * H * W + C * C * 9, bound="mfma",
+                workload="4 x int8 3x3 conv 128->128 s1 p1 @56x56, batch 64, int8 in/out, requantize+ReLU",
+                dom_kernel="conv 3x3 128->128 (MFMA implicit GEMM)",
+                dom_fn=lambda: layers[1].forward(bufs[0], capi.I8_P8, N, H, W, capi.I8_P8, out=bufs[1]),
+                x=x, params=params, shape=(N, C, H, W))
+
+
+def build_c1(hip, capi, rng, stride):
+    """configs[1]: depthwise 3x3 p1 on 8x256x112x112 fp32, bias, ReLU6, requantize to int8 with 127/6."""
+    N, C, H, W = 8, 256, 112, 112
+    x = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
+    wq, ws = quantize_weights(rng.normal(0, 0.1, (C, 1, 3, 3)).astype(np.float32))
+    bias = rng.normal(0, 0.01, C).astype(np.float32)
+    in_scale = np.float32(127) / np.abs(x).max()
+    out_scale = np.float32(127.0 / 6.0)
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale),
+                    out_scale=[out_scale], stride=(stride, stride), pad=(1, 1), groups=C, act=3,
+                    out_kind=capi.OUT_I8)
+    xd = hip.to_device(capi.pack_np(x, 8))          # Float8, what Net::convert_layout hands the layer
+    oh, ow = conv.out_hw(H, W)
+    xq = hip.empty(N * C * H * W, np.int8)
+    out = hip.empty(N * C * oh * ow, np.int8)
+    scale_dev = hip.to_device(np.array([in_scale], np.float32))
+
+    def step():
+        hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
+        conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out)
+        return out
+
+    in_b, out_b = N * C * H * W, N * C * oh * ow
+    return dict(name="c1s%d" % stride, step=step, ops=2.0 * N * C * 9 * oh * ow, launches=2,
+                bytes=5 * in_b + in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=in_b + out_b, bound="hbm",
+                workload="depthwise int8 3x3 s%d p1, 8x256x112x112 fp32 in -> quantize -> conv+bias+ReLU6+requantize "
+                         "-> int8" % stride,
+                dom_kernel="depthwise 3x3 s%d + requantize (int8 in -> int8 out)" % stride,
+                dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out),
+                aux=dict(kernel="quantize fp32 Float8 -> Byte8", bytes=5 * in_b,
+                         fn=lambda: hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8,
+                                                 dst=xq)),
+                x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
+                shape=(N, C, H, W), stride=stride)
+
+
+def build_c2(hip, capi, rng):
+    """configs[2]: 1x1 conv 256->512 on 32x256x28x28 (GEMM M=512, N=25088, K=256), bias, dequantize+ReLU, fp32."""
+    N, C, K, H, W = 32, 256, 512, 28, 28
+    x = rng.uniform(0, 1, (N, C, H, W)).astype(np.float32)
+    wq, ws = quantize_weights(rng.normal(0, 0.03, (K, C, 1, 1)).astype(np.float32))
+    bias = rng.normal(0, 0.01, K).astype(np.float32)
+    in_scale = np.float32(127) / np.abs(x).max()
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale), act=1,
+                    out_kind=capi.OUT_F32)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    xq = hip.empty(N * C * H * W, np.int8)
+    out = hip.empty(N * K * H * W, np.float32)
+    scale_dev = hip.to_device(np.array([in_scale], np.float32))
+
+    def step():
+        hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
+        conv.forward(xq, capi.I8_P8, N, H, W, capi.F32_P4, out=out)
+        return out
+
+    ops = 2.0 * N * K * C * H * W
+    return dict(name="c2", step=step, ops=ops, launches=2, dom_ops=ops,
+                dom_bytes=N * C * H * W + K * C + 4 * N * K * H * W, bound="hbm",
+                workload="int8 1x1 conv 256->512 @28x28 batch 32 (GEMM 512x25088x256), fp32 in -> quantize -> conv + "
+                         "bias + dequantize + ReLU -> fp32",
+                dom_kernel="conv 1x1 256->512 (MFMA implicit GEMM, fp32 out)",
+                dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.F32_P4, out=out),
+                x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale))], shape=(N, C, H, W))
+
+
+def build_c0(hip, capi, rng):
+    """configs[0]: one 3x3 s1 p1 conv 64->64 on 1x64x56x56 fp32, no bias, dequantize to fp32."""
+    N, C, K, H, W = 1, 64, 64, 56, 56
+    x = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
+    wq, ws = quantize_weights(rng.normal(0, 0.05, (K, C, 3, 3)).astype(np.float32))
+    in_scale = np.float32(127) / np.abs(x).max()
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), in_scale=float(in_scale), pad=(1, 1),
+                    out_kind=capi.OUT_F32)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    ws_buf = hip.empty(N * C * H * W, np.int8)
+    out = hip.empty(N * K * H * W, np.float32)
+
+    def step():
+        conv.forward(xd, capi.F32_P8, N, H, W, capi.F32_P4, out=out, workspace=ws_buf)
+        return out
+
+    ops = 2.0 * N * K * C * 9 * H * W
+    return dict(name="c0", step=step, ops=ops, launches=2, dom_ops=ops,
+                dom_bytes=N * C * H * W + K * C * 9 + 4 * N * K * H * W, bound="mfma",
+                workload="single int8 3x3 conv 64->64 s1 p1, 1x64x56x56 fp32 in -> fp32 out (latency-bound)",
+                dom_kernel="conv 3x3 64->64 (MFMA implicit GEMM, fp32 out)",
+                dom_fn=None, x=x, params=[dict(wq=wq, ws=ws, bias=None, in_scale=float(in_scale))],
+                shape=(N, C, H, W))
+
+
+# ------------------------------------------------------------------------------------------------------
+# CPU baseline: the reference itself (oracle/_ref, kind "reference") or the C restatement (kind "port")
+# ------------------------------------------------------------------------------------------------------
+
+def cpu_baseline(wl, budget_s=15.0):
+    from oracle import binding
+    name = wl["name"]
+    p = wl["params"]
+    N, C, H, W = wl["shape"]
+    x = wl["x"]
+    try:
+        R = binding.Ref() if binding.ref_available() else None
+    except OSError:
+        R = None
+    if name == "c3":
+        n_img = 4
+        xs = x[:n_img]
+        if R is not None:
+            t_total = 0.0
+            cur = xs
+            for l in range(4):
+                opts = {"type": "Convolution", "in_channels": C, "out_channels": C, "kernel": 3, "stride": 1,
+                        "padding": 1, "int8_scale_term": 102, "activation": "Relu"}
+                L = R.conv_layer(opts, (1, C, H, W), p[l]["wq"], p[l]["bias"], p[l]["ws"], p[l]["in_scale"],
+                                 p[l]["out_scale"], True)
+                cur, t = L.forward(cur, repeat=3)
+                L.close()
+                t_total += t
+            ops = 4 * 2.0 * n_img * C * C * 9 * H * W
+            return dict(value=ops / t_total / 1e12, unit="TOPS", cores=R.num_threads(), kind="reference",
+                        sample="%d of 64 images through the 4 layers, reference ConvolutionLayer::forward per image "
+                               "(weights pre-packed), min of 3" % n_img)
+        O = binding.Oracle()
+        t0 = time.perf_counter()
+        O.conv_layer_forward(xs[:1], p[0]["wq"], p[0]["ws"], p[0]["in_scale"], pad=(1, 1), bias=p[0]["bias"],
+                             top_scale=p[0]["out_scale"], int8_out=True, act_type=1)
+        t = time.perf_counter() - t0
+        return dict(value=2.0 * C * C * 9 * H * W / t / 1e12, unit="TOPS", cores=O.num_threads(), kind="port",
+                    sample="1 image, layer 1, scalar C restatement")
+    if name.startswith("c1"):
+        s = wl["stride"]
+        n_img = 2
+        oh = (H + 2 - 3) // s + 1
+        algo_bytes = n_img * C * (H * W * 5 + H * W + oh * oh)
+        if R is not None:
+            opts = {"type": "Convolution", "in_channels": C, "out_channels": C, "kernel": 3, "stride": s, "padding": 1,
+                    "groups": C, "int8_scale_term": 101, "activation": "Relu6"}
+            L = R.conv_layer(opts, (1, C, H, W), p[0]["wq"], p[0]["bias"], p[0]["ws"], p[0]["in_scale"],
+                             p[0]["out_scale"], True)
+            _, t = L.forward(x[:n_img], repeat=3, want_out=False)
+            L.close()
+            return dict(value=algo_bytes / t / 1e9, unit="GB/s", cores=R.num_threads(), kind="reference",
+                        sample="%d of 8 images, reference layer forward (quantize + depthwise + requantize), min of 3, "
+                               "algorithmic bytes" % n_img)
+        O = binding.Oracle()
+        t0 = time.perf_counter()
+        O.conv_layer_forward(x[:n_img], p[0]["wq"], p[0]["ws"], p[0]["in_scale"], stride=(s, s), pad=(1, 1), groups=C,
+                             bias=p[0]["bias"], top_scale=p[0]["out_scale"], int8_out=True, act_type=3)
+        t = time.perf_counter() - t0
+        return dict(value=algo_bytes / t / 1e9, unit="GB/s", cores=O.num_threads(), kind="port",
+                    sample="%d images, scalar C restatement" % n_img)
+    if name in ("c2", "c0"):
+        n_img = min(4, N)
+        K = p[0]["wq"].shape[0]
+        k = p[0]["wq"].shape[2]
+        ops = 2.0 * n_img * K * C * k * k * H * W
+        if R is not None:
+            opts = {"type": "Convolution", "in_channels": C, "out_channels": K, "kernel": k, "stride": 1,
+                    "padding": k // 2, "int8_scale_term": 2, "bias_term": "true" if p[0]["bias"] is not None else "false"}
+            if name == "c2":
+                opts["activation"] = "Relu"
+            L = R.conv_layer(opts, (1, C, H, W), p[0]["wq"], p[0]["bias"], p[0]["ws"], p[0]["in_scale"], 1.0, True)
+            _, t = L.forward(x[:n_img], repeat=5, want_out=False)
+            L.close()
+            return dict(value=ops / t / 1e12, unit="TOPS", cores=R.num_threads(), kind="reference",
+                        sample="%d images, reference layer forward, min of 5" % n_img)
+    return None
+
+
+def measure(wl, timer, steps, warmup, unit_main):
+    ms, wall_ms = timer.run(wl["step"], steps, warmup)
+    res = dict(workload=wl["workload"], ms_per_step=ms, wall_ms_per_step=wall_ms)
+    if wl["bound"] == "mfma" or unit_main == "TOPS":
+        res["tops"] = wl["ops"] / (ms * 1e-3) / 1e12
+    if "bytes" in wl:
+        res["gbs"] = wl["bytes"] / (ms * 1e-3) / 1e9
+    # dominant kernel alone, back to back
+    if wl.get("dom_fn") is not None:
+        kms, _ = timer.run(wl["dom_fn"], max(steps * 4, 50), 5)
+    else:
+        kms = ms
+    if wl["bound"] == "mfma":
+        ach = wl["dom_ops"] / (kms * 1e-3) / 1e12
+        res["roofline"] = dict(bound="mfma", achieved=ach, peak=PEAK_INT8_TOPS, unit="TOP/s", frac=ach / PEAK_INT8_TOPS,
+                               traffic=None, kernel=wl["dom_kernel"], kernel_ms=kms)
+    else:
+        ach = wl["dom_bytes"] / (kms * 1e-3) / 1e9
+        res["roofline"] = dict(bound="hbm", achieved=ach, peak=PEAK_HBM_GBS, unit="GB/s", frac=ach / PEAK_HBM_GBS,
+                               traffic=None, kernel=wl["dom_kernel"], kernel_ms=kms)
+        res["roofline"]["tops"] = wl["dom_ops"] / (kms * 1e-3) / 1e12
+    if "aux" in wl:
+        ams, _ = timer.run(wl["aux"]["fn"], max(steps * 4, 50), 5)
+        res["aux_kernel"] = dict(kernel=wl["aux"]["kernel"], kernel_ms=ams, gbs=wl["aux"]["bytes"] / (ams * 1e-3) / 1e9,
+                                 frac_hbm=wl["aux"]["bytes"] / (ams * 1e-3) / 1e9 / PEAK_HBM_GBS)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-also", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU only (batch sharding is described in DESIGN.md); "
+              "--gpus %d is not supported" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    if int(os.environ.get("WORLD_SIZE", "1")) > 1:
+        print("bench.py: one process, one GPU", file=sys.stderr)
+        sys.exit(2)
+
+    from tensor_amd import capi
+    hip = capi.Library(0)
+    timer = Timer(hip.torch)
+    builders = {"c3": lambda r: build_c3(hip, capi, r), "c1s1": lambda r: build_c1(hip, capi, r, 1),
+                "c1s2": lambda r: build_c1(hip, capi, r, 2), "c2": lambda r: build_c2(hip, capi, r),
+                "c0": lambda r: build_c0(hip, capi, r)}
+    try:
+        from tensor_amd import mobilenet  # noqa: F401
+        builders["c4"] = lambda r: mobilenet.build_bench(hip, capi, r)
+    except ImportError:
+        pass
+    if a.workload not in builders:
+        print("unknown workload %s (have %s)" % (a.workload, sorted(builders)), file=sys.stderr)
+        sys.exit(2)
+
+    wl = builders[a.workload](np.random.default_rng(0))
+    unit = "TOPS" if wl["bound"] == "mfma" else ("images/s" if wl["name"] == "c4" else "GB/s")
+    res = measure(wl, timer, a.steps, a.warmup, unit)
+    if wl["name"] == "c4":
+        value = wl["images"] / (res["ms_per_step"] * 1e-3)
+        metric = "MobileNetV2-style int8 net images/sec b64"
+    elif unit == "TOPS":
+        value = res["tops"]
+        metric = "int8 conv TOPS"
+    else:
+        value = res["gbs"]
+        metric = "depthwise int8 HBM GB/s (quantize + depthwise layer, algorithmic bytes)"
+    line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "int8 x int8 -> int32 (fp32 epilogue)", "data": "synthetic, seeded (numpy default_rng(0))",
+            "config": {"workload": wl["workload"], "launches_per_step": wl["launches"]},
+            "roofline": res["roofline"], "wall_ms_per_step": res["wall_ms_per_step"]}
+    if "aux_kernel" in res:
+        line["aux_kernel"] = res["aux_kernel"]
+    if not a.no_cpu:
+        try:
+            line["cpu_baseline"] = cpu_baseline(wl)
+        except Exception as e:  # the baseline is a reported figure, never the measured path
+            line["cpu_baseline"] = {"error": str(e)[:200]}
+    if not a.no_also:
+        also = []
+        for name in ("c1s1", "c1s2", "c2", "c0", "c4"):
+            if name == a.workload or name not in builders:
+                continue
+            w2 = builders[name](np.random.default_rng(0))
+            r2 = measure(w2, timer, max(10, a.steps // 2), a.warmup, "")
+            entry = dict(name=name, **r2)
+            if name == "c4":
+                entry["images_per_s"] = w2["images"] / (r2["ms_per_step"] * 1e-3)
+            if not a.no_cpu and name != "c4":
+                try:
+                    entry["cpu_baseline"] = cpu_baseline(w2)
+                except Exception as e:
+                    entry["cpu_baseline"] = {"error": str(e)[:200]}
+            also.append(entry)
+            del w2
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

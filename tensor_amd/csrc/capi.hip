@@ -53,7 +53,7 @@ struct otter_hip_conv {
     int8_t* w_igemm = nullptr;   // MFMA lane order            (groups == 1, C % 8 == 0)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
     float* scale_in = nullptr;   // [Kpad]
-    float* bias = nullptr;       // [Kpad] or null
+    float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
     float* scale_out = nullptr;  // [Kpad] or null
     float* in_scale = nullptr;   // [1]
     int force_tm = 0, force_tn = 0;
@@ -173,7 +173,8 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
         const size_t wcount = (size_t)K * (C / g) * maxk;
         if ((rc = upload<int8_t>(&h->w_raw, weight, wcount, wcount, 0))) break;
         if ((rc = upload<float>(&h->scale_in, scale_in, K, kpad, 0.f))) break;
-        if (bias && (rc = upload<float>(&h->bias, bias, K, kpad, 0.f))) break;
+        // no bias: -0.0f, so that fma(acc, scale, bias) == acc * scale bit for bit (sign of zero included)
+        if ((rc = upload<float>(&h->bias, bias, bias ? K : 0, kpad, -0.0f))) break;
         if (d.out_kind == OTTER_HIP_OUT_I8) {
             std::vector<float> so(K);
             for (int i = 0; i < K; ++i) so[i] = n_out_scale == 1 ? out_scale[0] : out_scale[i];
@@ -235,19 +236,34 @@ int otter_hip_conv_set_tile(otter_hip_conv_t* h, int tm, int tn) {
     return OTTER_HIP_OK;
 }
 
-static int pick_kernel(const otter_hip_conv* h, int int8_layout) {
+static ConvGeom make_geom(const otter_hip_conv_desc& d, int n, int in_h, int in_w) {
+    ConvGeom g;
+    g.N = n, g.C = d.in_channels, g.H = in_h, g.W = in_w, g.K = d.out_channels;
+    g.kh = d.kernel_h, g.kw = d.kernel_w, g.sh = d.stride_h, g.sw = d.stride_w, g.ph = d.pad_h, g.pw = d.pad_w;
+    g.dh = d.dilation_h, g.dw = d.dilation_w, g.groups = d.groups;
+    g.OH = conv_out_size(in_h, d.kernel_h, d.stride_h, d.pad_h, d.dilation_h);
+    g.OW = conv_out_size(in_w, d.kernel_w, d.stride_w, d.pad_w, d.dilation_w);
+    return g;
+}
+
+// 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS
+static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
-        if (h->w_igemm) return 1;
+        if (h->w_igemm) {
+            if (h->force_tm > 0) return 1;
+            if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g)) return 3;
+            return 1;
+        }
     }
     return 0;
 }
 
-int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int, int, int, int) {
+int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int) {
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
     if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
-    return pick_kernel(h, l);
+    return pick_kernel(h, l, make_geom(h->d, n, in_h, in_w));
 }
 
 int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
@@ -267,12 +283,7 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     if (d.out_channels % layout_pack(out_layout))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: output pack does not divide K");
 
-    ConvGeom g;
-    g.N = n, g.C = d.in_channels, g.H = in_h, g.W = in_w, g.K = d.out_channels;
-    g.kh = d.kernel_h, g.kw = d.kernel_w, g.sh = d.stride_h, g.sw = d.stride_w, g.ph = d.pad_h, g.pw = d.pad_w;
-    g.dh = d.dilation_h, g.dw = d.dilation_w, g.groups = d.groups;
-    g.OH = conv_out_size(in_h, d.kernel_h, d.stride_h, d.pad_h, d.dilation_h);
-    g.OW = conv_out_size(in_w, d.kernel_w, d.stride_w, d.pad_w, d.dilation_w);
+    const ConvGeom g = make_geom(d, n, in_h, in_w);
     if (g.OH < 1 || g.OW < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: empty output");
     if ((size_t)n * g.C * in_h * in_w >= (1ull << 31) || (size_t)n * g.K * g.OH * g.OW >= (1ull << 31))
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
@@ -295,9 +306,15 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     ep.scale_in = h->scale_in, ep.bias = h->bias, ep.scale_out = h->scale_out;
     ep.act = d.activation_type, ep.act_p0 = d.activation_param0, ep.round_mode = d.out_round_mode;
     ep.out_kind = d.out_kind, ep.out_layout = out_layout;
+    ep.act_lo = (d.activation_type == 1 || d.activation_type == 3) ? 0.f : -__builtin_inff();
+    ep.act_hi = d.activation_type == 3 ? 6.f : __builtin_inff();
+    ep.round_half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
 
     // (2)+(3)+(4) convolution with the fused epilogue
-    switch (pick_kernel(h, q_layout)) {
+    switch (pick_kernel(h, q_layout, g)) {
+    case 3:
+        OHIP_CHECK(run_conv3x3_halo(xq, h->w_igemm, out, g, ep, h->force_tm < 0 ? h->force_tn : 0, stream));
+        break;
     case 2:
         if ((long)n * (g.C / 8) > 65535) {
             // the plane index rides on grid.y: run the batch in slices

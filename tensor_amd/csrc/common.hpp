@@ -109,7 +109,22 @@ struct Epilogue {
     int round_mode;
     int out_kind;    // otter_hip_out_kind
     int out_layout;  // otter_hip_layout
+    // fast epilogues (activation none / ReLU / clip[0,6] as one clamp, rounding mode as one constant)
+    float act_lo, act_hi;  // v = min(max(v, act_lo), act_hi)
+    float round_half;      // 0.5f (ROUND_SSE) or 0.49999997f (ROUND_EXACT)
 };
+
+// which epilogue code a kernel instance carries
+enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2 };
+
+// The fast epilogues need: activation in {none, ReLU, clip}, and (I8_P8) int8 output in Byte8 with K % 8 == 0
+// or (F32_P4) fp32 output in Float4 with K % 4 == 0.
+__host__ inline int pick_epilogue(const Epilogue& ep, int K) {
+    const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3;
+    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0) return EPI_I8_P8;
+    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_F32 && ep.out_layout == OTTER_HIP_F32_P4 && K % 4 == 0) return EPI_F32_P4;
+    return EPI_GENERIC;
+}
 
 struct ConvGeom {
     int N, C, H, W;        // input
@@ -179,6 +194,82 @@ __device__ __forceinline__ void epilogue_store8(void* __restrict__ out, const Ep
                 if (ch0 + e < K) o[elem_offset(1, n, ch0 + e, pix, K, OHW)] = r8[e];
         }
     }
+}
+
+// Out-of-line copy of the generic tail: keeps the kernels that carry it small (it is the slow path anyway).
+__device__ __noinline__ void epilogue_store8_generic(void* __restrict__ out, const Epilogue* ep, int n, int ch0, int pix,
+                                                     int K, int OHW, int a0, int a1, int a2, int a3, int a4, int a5,
+                                                     int a6, int a7) {
+    const int a8[8] = {a0, a1, a2, a3, a4, a5, a6, a7};
+    float si[8], bi[8], so[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        si[e] = ep->scale_in[ch0 + e];
+        bi[e] = ep->bias ? ep->bias[ch0 + e] : 0.f;
+        so[e] = ep->scale_out ? ep->scale_out[ch0 + e] : 1.f;
+    }
+    epilogue_store8(out, *ep, n, ch0, pix, K, OHW, a8, si, bi, so);
+}
+
+// Per-lane epilogue constants of 8 consecutive channels for the fast paths. `bias` always points at an array
+// (filled with -0.0f when the layer has no bias: fma(a, s, -0.0f) == a * s bit for bit, sign of zero included).
+struct Epi8 {
+    float si[8], bi[8], so[8];
+};
+
+template <int EPI>
+__device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) {
+    const ohip_v4i* s = reinterpret_cast<const ohip_v4i*>(ep.scale_in + ch0);
+    const ohip_v4i* b = reinterpret_cast<const ohip_v4i*>(ep.bias + ch0);
+    ohip_v4i s0 = s[0], s1 = s[1], b0 = b[0], b1 = b[1];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        p.si[e] = __int_as_float(s0[e]);
+        p.si[4 + e] = __int_as_float(s1[e]);
+        p.bi[e] = __int_as_float(b0[e]);
+        p.bi[4 + e] = __int_as_float(b1[e]);
+    }
+    if constexpr (EPI == EPI_I8_P8) {
+        const ohip_v4i* o = reinterpret_cast<const ohip_v4i*>(ep.scale_out + ch0);
+        ohip_v4i o0 = o[0], o1 = o[1];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            p.so[e] = __int_as_float(o0[e]);
+            p.so[4 + e] = __int_as_float(o1[e]);
+        }
+    }
+}
+
+// requantize 8 channels and store one Byte8 element
+__device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const Epilogue& ep, const Epi8& p, size_t elem,
+                                                const int (&a8)[8]) {
+    int q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float v = __fmaf_rn((float)a8[e], p.si[e], p.bi[e]);
+        v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        v = __fmul_rn(v, p.so[e]);
+        float adj = __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
+        q[e] = min(max((int)adj, -127), 127);
+    }
+    ohip_v2i pk;
+    pk[0] = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | (q[3] << 24);
+    pk[1] = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | (q[7] << 24);
+    *reinterpret_cast<ohip_v2i*>(out + elem) = pk;
+}
+
+// dequantize (+clamp activation) 4 channels and store one Float4 element
+__device__ __forceinline__ void epi4_store_f32p4(float* __restrict__ out, const Epilogue& ep, const float* si,
+                                                 const float* bi, size_t elem, int a0, int a1, int a2, int a3) {
+    const int a[4] = {a0, a1, a2, a3};
+    ohip_v4i r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = __fmaf_rn((float)a[e], si[e], bi[e]);
+        v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        r[e] = __float_as_int(v);
+    }
+    *reinterpret_cast<ohip_v4i*>(out + elem) = r;
 }
 
 }  // namespace ohip

@@ -32,7 +32,7 @@ struct IgemmCfg {
     static_assert(TN % 64 == 0, "pixel tile");
 };
 
-template <int TM, int TN, int WM, int WN>
+template <int TM, int TN, int WM, int WN, int EPI>
 __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                          void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
                                                          int c_groups, int n_pix_tiles) {
@@ -148,33 +148,40 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     }
 
     // ---- epilogue -----------------------------------------------------------------------------------
+    // (no `continue` / early exits inside the unrolled loops: the accumulator array must stay in registers)
     const int gq = lane >> 4;
-    const bool has_bias = ep.bias != nullptr;
 #pragma unroll
     for (int ip = 0; ip < FM / 2; ++ip) {
         const int tpair = (mt0 + wm * FM) / 2 + ip;
         const int ch0 = 32 * tpair + 8 * gq;  // this lane's 8 consecutive output channels
-        if (ch0 >= g.K) continue;
-        float si[8], bi[8], so[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            si[e] = ep.scale_in[ch0 + e];
-            bi[e] = has_bias ? ep.bias[ch0 + e] : 0.f;
-            so[e] = ep.scale_out ? ep.scale_out[ch0 + e] : 1.f;
-        }
+        const bool ch_ok = ch0 < g.K;
+        Epi8 prm;
+        if constexpr (EPI != EPI_GENERIC) epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const long gpo = tile_base + wn * (TN / WN) + j * 16 + (lane & 15);
-            if (gpo >= total_pix) continue;
-            const int n = (int)(gpo / OHW);
-            const int pix = (int)(gpo % OHW);
             int a8[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 a8[e] = acc[2 * ip][j][e];
                 a8[4 + e] = acc[2 * ip + 1][j][e];
             }
-            epilogue_store8(out, ep, n, ch0, pix, g.K, OHW, a8, si, bi, so);
+            if (ch_ok && gpo < total_pix) {
+                const int n = (int)(gpo / OHW);
+                const int pix = (int)(gpo % OHW);
+                if constexpr (EPI == EPI_I8_P8) {
+                    epi8_store_i8p8((int8_t*)out, ep, prm, elem_offset(8, n, ch0, pix, g.K, OHW), a8);
+                } else if constexpr (EPI == EPI_F32_P4) {
+                    epi4_store_f32p4((float*)out, ep, prm.si, prm.bi, elem_offset(4, n, ch0, pix, g.K, OHW), a8[0],
+                                     a8[1], a8[2], a8[3]);
+                    if (ch0 + 4 < g.K)
+                        epi4_store_f32p4((float*)out, ep, prm.si + 4, prm.bi + 4,
+                                         elem_offset(4, n, ch0 + 4, pix, g.K, OHW), a8[4], a8[5], a8[6], a8[7]);
+                } else {
+                    epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
+                                            a8[6], a8[7]);
+                }
+            }
         }
     }
 }
@@ -213,16 +220,29 @@ void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* d
                 }
 }
 
-template <int TM, int TN, int WM, int WN>
-static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
-                               hipStream_t stream) {
+template <int TM, int TN, int WM, int WN, int EPI>
+static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                                 hipStream_t stream) {
     const long total_pix = (long)g.N * g.OH * g.OW;
     const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
     const int mpad = igemm_padded_rows(g.K);
     const int m_tiles = (mpad + TM - 1) / TM;
-    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN>), dim3(n_pix_tiles, m_tiles), dim3(256), 0, stream, x, wpk,
-                       out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
+    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI>), dim3(n_pix_tiles, m_tiles), dim3(256), 0, stream, x,
+                       wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
     return hipGetLastError();
+}
+
+template <int TM, int TN, int WM, int WN>
+static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                               hipStream_t stream) {
+    switch (pick_epilogue(ep, g.K)) {
+    case EPI_I8_P8:
+        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8>(x, wpk, out, g, ep, stream);
+    case EPI_F32_P4:
+        return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, stream);
+    default:
+        return launch_igemm_e<TM, TN, WM, WN, EPI_GENERIC>(x, wpk, out, g, ep, stream);
+    }
 }
 
 // tile choice: the widest row tile that does not pad M further, then the widest pixel tile that still

@@ -14,6 +14,11 @@ void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn);
 hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep, int tm,
                           int tn, hipStream_t stream);
 
+// conv3x3.hip
+bool conv3x3_halo_supported(const ConvGeom& g);
+hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                            int force_fn, hipStream_t stream);
+
 // conv_direct.hip
 hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void* out, const ConvGeom& g,
                            const Epilogue& ep, hipStream_t stream);

@@ -186,6 +186,29 @@ def test_igemm_every_tile_shape(hip, oracle, tile):
         np.testing.assert_array_equal(out, want)
 
 
+@pytest.mark.parametrize("fn", [4, 5, 6, 7, 8])
+def test_halo3x3_every_fragment_count(hip, oracle, fn):
+    """The 3x3 stride-1 LDS-halo MFMA kernel: wide (K > 64) and narrow wave layouts, padded channel counts,
+    pad 0 and 1, ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at once)."""
+    rng = np.random.default_rng(fn)
+    for (C, K, p, N, H, W) in [(128, 128, 1, 2, 19, 23), (64, 64, 1, 1, 56, 56), (72, 24, 0, 2, 11, 9),
+                               (16, 160, 1, 1, 7, 7), (320, 96, 1, 1, 14, 30)]:
+        x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
+        in_scale = 25.0
+        for int8_out in (True, False):
+            want, acc_want = oracle.conv_layer_forward(x, wq, ws, in_scale, pad=(p, p), bias=bias, top_scale=7.0,
+                                                       int8_out=int8_out, act_type=1, want_acc=True)
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, bias=bias, top_scale=7.0, act=1,
+                                 out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32, tile=(-1, fn))
+            assert kind == 3
+            if int8_out:
+                np.testing.assert_array_equal(out, want)
+            else:
+                assert_f32_close(out, want)
+        acc, _ = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, out_kind=capi.OUT_I32, tile=(-1, fn))
+        np.testing.assert_array_equal(acc, acc_want)
+
+
 @pytest.mark.parametrize("C,K,k,s,p,d,g,N,H,W", [
     (16, 24, 1, 1, 0, 1, 1, 3, 14, 14),     # MobileNetV2 project: K % 32 != 0
     (96, 160, 1, 1, 0, 1, 1, 2, 7, 7),

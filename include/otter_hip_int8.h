@@ -142,7 +142,7 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
 /* Tuning / test hook with no counterpart in the reference. (0, 0): automatic choice. tm > 0: force the generic
  * MFMA implicit-GEMM kernel with a tile of tm output channels x tn pixels (tm in {32,64,128}, tn in
  * {64,128,256}). tm < 0: keep the 3x3 halo kernel where it applies and force its pixel-fragment count to tn
- * (4..8, 0 = automatic). */
+ * (4..7, 0 = automatic). */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
 /* ------------------------------------------------------------------------------------------------ */

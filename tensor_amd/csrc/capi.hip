@@ -167,7 +167,7 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
     h->d = d;
     const int K = d.out_channels, C = d.in_channels, g = d.groups, maxk = d.kernel_h * d.kernel_w;
     h->depthwise = (C == g && g == K);
-    const int kpad = (K + 31) / 32 * 32;
+    const int kpad = igemm_padded_rows(K);  // the kernels read the per-channel arrays up to the padded row count
     int rc = OTTER_HIP_OK;
     do {
         const size_t wcount = (size_t)K * (C / g) * maxk;

@@ -115,13 +115,14 @@ struct Epilogue {
 };
 
 // which epilogue code a kernel instance carries
-enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2 };
+enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3 };
 
 // The fast epilogues need: activation in {none, ReLU, clip}, and (I8_P8) int8 output in Byte8 with K % 8 == 0
 // or (F32_P4) fp32 output in Float4 with K % 4 == 0.
 __host__ inline int pick_epilogue(const Epilogue& ep, int K) {
     const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3;
-    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0) return EPI_I8_P8;
+    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0)
+        return ep.act != 0 ? EPI_I8_P8_NONNEG : EPI_I8_P8;  // after ReLU / clip the value to round is never negative
     if (clamp_act && ep.out_kind == OTTER_HIP_OUT_F32 && ep.out_layout == OTTER_HIP_F32_P4 && K % 4 == 0) return EPI_F32_P4;
     return EPI_GENERIC;
 }
@@ -229,7 +230,7 @@ __device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) 
         p.bi[e] = __int_as_float(b0[e]);
         p.bi[4 + e] = __int_as_float(b1[e]);
     }
-    if constexpr (EPI == EPI_I8_P8) {
+    if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
         const ohip_v4i* o = reinterpret_cast<const ohip_v4i*>(ep.scale_out + ch0);
         ohip_v4i o0 = o[0], o1 = o[1];
 #pragma unroll
@@ -240,21 +241,38 @@ __device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) 
     }
 }
 
-// requantize 8 channels and store one Byte8 element
+// requantize 8 channels and store one Byte8 element. NONNEG: the activation clamp has a lower bound of 0, so the
+// value handed to the rounding step is >= 0: copysign(half, v) is just half and only the upper saturation can bind.
+// The median-of-three clamp differs from max/min only in the sign of a zero result, which the rounding discards.
+typedef short ohip_v2s __attribute__((ext_vector_type(2)));
+
+template <bool NONNEG>
 __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const Epilogue& ep, const Epi8& p, size_t elem,
                                                 const int (&a8)[8]) {
     int q[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float v = __fmaf_rn((float)a8[e], p.si[e], p.bi[e]);
-        v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        v = __builtin_amdgcn_fmed3f(v, ep.act_lo, ep.act_hi);
         v = __fmul_rn(v, p.so[e]);
-        float adj = __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
-        q[e] = min(max((int)adj, -127), 127);
+        float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
+        q[e] = (int)adj;  // toward zero, saturating
     }
     ohip_v2i pk;
-    pk[0] = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | (q[3] << 24);
-    pk[1] = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | (q[7] << 24);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        // two int32 -> two saturated int16 in one dword, clamp both halves at once, then gather the low bytes
+        ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h], q[4 * h + 1]));
+        ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h + 2], q[4 * h + 3]));
+        const ohip_v2s top = {127, 127}, bot = {-127, -127};
+        lo = __builtin_elementwise_min(lo, top);
+        hi = __builtin_elementwise_min(hi, top);
+        if (!NONNEG) {
+            lo = __builtin_elementwise_max(lo, bot);
+            hi = __builtin_elementwise_max(hi, bot);
+        }
+        pk[h] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
+    }
     *reinterpret_cast<ohip_v2i*>(out + elem) = pk;
 }
 

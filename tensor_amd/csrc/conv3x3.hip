@@ -72,55 +72,76 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
 
     for (int cb0 = 0; cb0 < c_groups * 64; cb0 += cb) {
         __syncthreads();  // everyone is done reading the previous channel block
+        // Stage the halo: one wave per (channel pair, row) line, lanes along the columns, so that the only
+        // divisions are wave-uniform (scalar) and a wave reads 2 x 512 contiguous bytes per line. Lines are taken
+        // in batches of SB with all loads of a batch issued before the first LDS write, so a batch costs one
+        // memory round trip.
         {
-            const int items = (cb / 16) * R * cols;
-            for (int idx = tid; idx < items; idx += 256) {
-                const int xc = idx % cols;
-                const int rr = idx / cols;
-                const int r = rr % R, j = rr / R;
-                const int iy = r_lo - g.ph + r, ix = xc - 1;
-                const int o0 = cb0 / 8 + 2 * j;
-                v2i lo = {0, 0}, hi = {0, 0};
-                if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W) {
-                    const int8_t* px = xn + ((size_t)iy * g.W + ix) * 8;
-                    if (o0 < C8) lo = *reinterpret_cast<const v2i*>(px + (size_t)o0 * g.H * g.W * 8);
-                    if (o0 + 1 < C8) hi = *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * g.H * g.W * 8);
+            constexpr int SB = 6;
+            const int lines = (cb / 16) * R;
+            for (int xc0 = 0; xc0 < cols; xc0 += 64) {
+                const int xc = xc0 + lane;
+                const int ix = xc - 1;
+                const bool col_ok = ix >= 0 && ix < g.W;
+                for (int l0 = wave; l0 < lines; l0 += 4 * SB) {
+                    v2i lo[SB], hi[SB];
+#pragma unroll
+                    for (int k = 0; k < SB; ++k) {
+                        const int line = min(l0 + 4 * k, lines - 1);
+                        const int j = line / R, r = line - j * R;
+                        const int iy = r_lo - g.ph + r;
+                        const int o0 = cb0 / 8 + 2 * j;
+                        const bool ok = col_ok && iy >= 0 && iy < g.H;
+                        const int8_t* px = xn + ((size_t)iy * g.W + ix) * 8;
+                        lo[k] = (ok && o0 < C8) ? *reinterpret_cast<const v2i*>(px + (size_t)o0 * g.H * g.W * 8) : v2i{0, 0};
+                        hi[k] = (ok && o0 + 1 < C8) ? *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * g.H * g.W * 8)
+                                                    : v2i{0, 0};
+                    }
+#pragma unroll
+                    for (int k = 0; k < SB; ++k) {
+                        const int line = l0 + 4 * k;
+                        const int j = line / R, r = line - j * R;
+                        if (line < lines && xc < cols)
+                            *reinterpret_cast<v4i*>(lds + (size_t)j * plane + ((size_t)r * cols + xc) * 16) =
+                                v4i{lo[k][0], lo[k][1], hi[k][0], hi[k][1]};
+                    }
                 }
-                *reinterpret_cast<v4i*>(&lds[(size_t)j * plane + (r * cols + xc) * 16]) = v4i{lo[0], lo[1], hi[0], hi[1]};
             }
         }
         __syncthreads();
 
-        const int nq = 9 * nck;
-        v4i a0[FM], a1[FM];
-        auto load_a = [&](int q, v4i (&a)[FM]) {
-            const int tap = q / nck, cc = q % nck;
-            const int8_t* p = wlane + (size_t)(tap * c_groups + cb0 / 64 + cc) * kc_stride;
+        // Main loop: no barrier, no branch. The nine taps are unrolled; weight fragments travel through a ring of
+        // three register stages and are requested two k-chunks (~0.4 us of MFMA work) before use. Every load is
+        // unconditional (the weight rows are padded to whole row blocks and the chunk index is clamped), so that
+        // the compiler can count outstanding loads and wait only for the oldest stage.
+        v4i ring[3][FM];
+        const int cg0 = cb0 / 64;
+        auto load_a = [&](int cc, int tap, v4i (&a)[FM]) {
+            const int8_t* p = wlane + (size_t)(tap * c_groups + cg0 + cc) * kc_stride;
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-                a[i] = (mt_base + i < m_tiles16) ? *reinterpret_cast<const v4i*>(p + i * 1024) : v4i{0, 0, 0, 0};
+            for (int i = 0; i < FM; ++i) a[i] = *reinterpret_cast<const v4i*>(p + i * 1024);
         };
-        auto compute = [&](int q, const v4i (&a)[FM]) {
-            const int tap = q / nck, cc = q % nck;
-            const int tapofs = ((tap / 3) * cols + tap % 3) * 16 + cc * 4 * plane;
-            v4i b[FN];
+        load_a(0, 0, ring[0]);
+        load_a(0, 1, ring[1]);
+        for (int cc = 0; cc < nck; ++cc) {
+            const int cc_next = min(cc + 1, nck - 1);
+            const int ccofs = cc * 4 * plane;
 #pragma unroll
-            for (int f = 0; f < FN; ++f) b[f] = *reinterpret_cast<const v4i*>(&lds[bofs[f] + tapofs]);
+            for (int tap = 0; tap < 9; ++tap) {
+                if (tap + 2 < 9) load_a(cc, tap + 2, ring[(tap + 2) % 3]);
+                else load_a(cc_next, tap + 2 - 9, ring[(tap + 2) % 3]);
+                const int tapofs = ((tap / 3) * cols + tap % 3) * 16 + ccofs;
+                v4i b[FN];
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+                for (int f = 0; f < FN; ++f) b[f] = *reinterpret_cast<const v4i*>(&lds[bofs[f] + tapofs]);
 #pragma unroll
-                for (int f = 0; f < FN; ++f)
-                    acc[i][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[f], acc[i][f], 0, 0, 0);
-        };
-        load_a(0, a0);
-        int q = 0;
-        for (; q + 1 < nq; q += 2) {
-            load_a(q + 1, a1);
-            compute(q, a0);
-            if (q + 2 < nq) load_a(q + 2, a0);
-            compute(q + 1, a1);
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int f = 0; f < FN; ++f)
+                        acc[i][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[tap % 3][i], b[f], acc[i][f], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);  // keep the prefetch distance: no hoisting of later taps' loads
+            }
         }
-        if (q < nq) compute(q, a0);
     }
 
     // ---- epilogue (no early exits inside the unrolled loops: the accumulators must stay in registers) -------
@@ -141,8 +162,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                 a8[4 + e] = acc[2 * ip + 1][f][e];
             }
             if (ch_ok && pix < OHW) {
-                if constexpr (EPI == EPI_I8_P8) {
-                    epi8_store_i8p8((int8_t*)out, ep, prm, elem_offset(8, n, ch0, pix, g.K, OHW), a8);
+                if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
+                    epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
+                                                             elem_offset(8, n, ch0, pix, g.K, OHW), a8);
                 } else if constexpr (EPI == EPI_F32_P4) {
                     epi4_store_f32p4((float*)out, ep, prm.si, prm.bi, elem_offset(4, n, ch0, pix, g.K, OHW), a8[0],
                                      a8[1], a8[2], a8[3]);
@@ -206,6 +228,8 @@ hipError_t launch_halo(const int8_t* x, const int8_t* wpk, void* out, const Conv
     switch (pick_epilogue(ep, g.K)) {
     case EPI_I8_P8:
         return launch_halo_e<FM, FN, WM, WN, EPI_I8_P8>(x, wpk, out, g, ep, pl, stream);
+    case EPI_I8_P8_NONNEG:
+        return launch_halo_e<FM, FN, WM, WN, EPI_I8_P8_NONNEG>(x, wpk, out, g, ep, pl, stream);
     case EPI_F32_P4:
         return launch_halo_e<FM, FN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, pl, stream);
     default:
@@ -222,7 +246,7 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
     const bool wide = igemm_padded_rows(g.K) > 64;
     const int m_blocks = wide ? (igemm_padded_rows(g.K) / 16 + 7) / 8 : 1;
     bool found = false;
-    for (int fn = 4; fn <= 8; ++fn) {
+    for (int fn = 4; fn <= 7; ++fn) {  // 8 fragments would spill at two waves per SIMD
         if (force_fn && fn != force_fn) continue;
         const int pt = (wide ? 32 : 64) * fn;
         HaloPlan p;
@@ -272,7 +296,6 @@ hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const
         OHIP_HALO(5)
         OHIP_HALO(6)
         OHIP_HALO(7)
-        OHIP_HALO(8)
     }
 #undef OHIP_HALO
     return hipErrorInvalidValue;

@@ -169,8 +169,9 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             if (ch_ok && gpo < total_pix) {
                 const int n = (int)(gpo / OHW);
                 const int pix = (int)(gpo % OHW);
-                if constexpr (EPI == EPI_I8_P8) {
-                    epi8_store_i8p8((int8_t*)out, ep, prm, elem_offset(8, n, ch0, pix, g.K, OHW), a8);
+                if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
+                    epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
+                                                             elem_offset(8, n, ch0, pix, g.K, OHW), a8);
                 } else if constexpr (EPI == EPI_F32_P4) {
                     epi4_store_f32p4((float*)out, ep, prm.si, prm.bi, elem_offset(4, n, ch0, pix, g.K, OHW), a8[0],
                                      a8[1], a8[2], a8[3]);
@@ -190,7 +191,8 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
 // host side
 // ---------------------------------------------------------------------------------------------------
 
-int igemm_padded_rows(int K) { return (K + 31) / 32 * 32; }
+// weight rows are padded so that every kernel's row block is whole: 32, 64, or a multiple of 128
+int igemm_padded_rows(int K) { return K <= 32 ? 32 : (K <= 64 ? 64 : (K + 127) / 128 * 128); }
 int igemm_channel_groups(int C) { return (C + 63) / 64; }
 
 // physical GEMM row -> logical output channel (rows of a pair of 16-row tiles are interleaved in fours, so
@@ -238,6 +240,8 @@ static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, co
     switch (pick_epilogue(ep, g.K)) {
     case EPI_I8_P8:
         return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8>(x, wpk, out, g, ep, stream);
+    case EPI_I8_P8_NONNEG:
+        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8_NONNEG>(x, wpk, out, g, ep, stream);
     case EPI_F32_P4:
         return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, stream);
     default:

@@ -35,7 +35,7 @@ __device__ __forceinline__ void mac8(int (&acc)[8], v2i px, const int* __restric
 }
 
 // 3x3, dilation 1, stride S (1 or 2): R output rows per lane with the input rows kept in registers.
-template <int S, int R>
+template <int S, int R, int EPI>
 __global__ void __launch_bounds__(256) conv_dw3x3_kernel(const int8_t* __restrict__ x, const int32_t* __restrict__ wmask,
                                                          void* __restrict__ out, ConvGeom g, Epilogue ep, int n_strips) {
     const int C8 = g.C / 8;
@@ -50,13 +50,13 @@ __global__ void __launch_bounds__(256) conv_dw3x3_kernel(const int8_t* __restric
     const int* wsrc = wmask + (size_t)o * 72;
 #pragma unroll
     for (int i = 0; i < 72; ++i) wm[i] = wsrc[i];
-    float si[8], bi[8], so[8];
-    const bool has_bias = ep.bias != nullptr;
+    // per-channel epilogue constants: wave-uniform (one channel octet per workgroup), so they sit in SGPRs
+    Epi8 prm;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        si[e] = ep.scale_in[o * 8 + e];
-        bi[e] = has_bias ? ep.bias[o * 8 + e] : 0.f;
-        so[e] = ep.scale_out ? ep.scale_out[o * 8 + e] : 1.f;
+        prm.si[e] = ep.scale_in[o * 8 + e];
+        prm.bi[e] = ep.bias[o * 8 + e];
+        prm.so[e] = ep.scale_out ? ep.scale_out[o * 8 + e] : 1.f;
     }
 
     const int8_t* xp = x + (size_t)plane * g.H * g.W * 8;
@@ -90,7 +90,111 @@ __global__ void __launch_bounds__(256) conv_dw3x3_kernel(const int8_t* __restric
         for (int u = 0; u < 3; ++u)
 #pragma unroll
             for (int v = 0; v < 3; ++v) mac8(acc, rows[r * S + u][v], &wm[(u * 3 + v) * 8]);
-        epilogue_store8(out, ep, n, o * 8, oy * g.OW + ox, g.K, OHW, acc, si, bi, so);
+        const int pix = oy * g.OW + ox;
+        if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
+            epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm, ((size_t)plane * OHW + pix) * 8, acc);
+        } else {
+            epilogue_store8(out, ep, n, o * 8, pix, g.K, OHW, acc, prm.si, prm.bi, prm.so);
+        }
+    }
+}
+
+// 3x3, int8 Byte8 out (the requantize epilogue): same strip walk, but the channel octet is processed as two
+// halves of four channels, one after the other. A half needs 36 weight words + 12 epilogue constants, which fit
+// the scalar register file; the whole octet (72 + 24) does not, and spilling them to VGPR lanes costs more VALU
+// work than the convolution itself. The first tap starts the accumulator (no zero-initialisation moves).
+template <int S, int R, bool NONNEG>
+__global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __restrict__ x, const int32_t* __restrict__ wmask,
+                                                            int8_t* __restrict__ out, ConvGeom g, Epilogue ep,
+                                                            int n_strips, int col_chunks) {
+    // A wave = 64 consecutive output columns of ONE strip, so "is this input row inside the image" is a scalar
+    // branch, not a per-lane exec mask (those masks would crowd the weights out of the scalar registers).
+    const int C8 = g.C / 8;
+    const int plane = blockIdx.y;
+    const int o = plane % C8;
+    const int chunk = blockIdx.x % col_chunks;
+    const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * 4 + (threadIdx.x >> 6));
+    const int ox = chunk * 64 + (threadIdx.x & 63);
+    if (strip >= n_strips || ox >= g.OW) return;
+
+    const int8_t* xp = x + (size_t)plane * g.H * g.W * 8;
+    const int ix0 = ox * S - g.pw;
+    // columns 0 and 2 of the window can fall off the image for the first / last output column only: read a clamped
+    // address and zero the value
+    const bool c0_ok = ix0 >= 0, c2_ok = ix0 + 2 < g.W, c1_ok = ix0 + 1 < g.W;
+    const int ixc0 = max(ix0, 0), ixc1 = min(ix0 + 1, g.W - 1), ixc2 = min(ix0 + 2, g.W - 1);
+    const int oy0 = strip * R;
+    const int OHW = g.OH * g.OW;
+
+    constexpr int NROWS = (R - 1) * S + 3;  // input rows a strip touches
+    v2i rows[NROWS][3];
+    const int iy_base = oy0 * S - g.ph;
+#pragma unroll
+    for (int r = 0; r < NROWS; ++r) {
+        const int iy = iy_base + r;
+        if (iy >= 0 && iy < g.H) {  // wave-uniform
+            const int8_t* rp = xp + (size_t)iy * g.W * 8;
+            const v2i a = *reinterpret_cast<const v2i*>(rp + (size_t)ixc0 * 8);
+            const v2i b = *reinterpret_cast<const v2i*>(rp + (size_t)ixc1 * 8);
+            const v2i c = *reinterpret_cast<const v2i*>(rp + (size_t)ixc2 * 8);
+            rows[r][0] = c0_ok ? a : v2i{0, 0};
+            rows[r][1] = c1_ok ? b : v2i{0, 0};
+            rows[r][2] = c2_ok ? c : v2i{0, 0};
+        } else {
+            rows[r][0] = rows[r][1] = rows[r][2] = v2i{0, 0};
+        }
+    }
+
+    int packed[2][R];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        int wm[9][4];
+        float si[4], bi[4], so[4];
+        const int* wsrc = wmask + (size_t)o * 72 + h * 4;
+#pragma unroll
+        for (int k = 0; k < 9; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wm[k][e] = wsrc[k * 8 + e];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            si[e] = ep.scale_in[o * 8 + h * 4 + e];
+            bi[e] = ep.bias[o * 8 + h * 4 + e];
+            so[e] = ep.scale_out[o * 8 + h * 4 + e];
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int q[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                int acc = __builtin_amdgcn_sdot4(rows[r * S][0][h], wm[0][e], 0, false);
+#pragma unroll
+                for (int k = 1; k < 9; ++k) acc = __builtin_amdgcn_sdot4(rows[r * S + k / 3][k % 3][h], wm[k][e], acc, false);
+                float v = __fmaf_rn((float)acc, si[e], bi[e]);
+                v = __builtin_amdgcn_fmed3f(v, ep.act_lo, ep.act_hi);
+                v = __fmul_rn(v, so[e]);
+                const float adj =
+                    NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
+                q[e] = (int)adj;
+            }
+            ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[0], q[1]));
+            ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[2], q[3]));
+            const ohip_v2s top = {127, 127}, bot = {-127, -127};
+            lo = __builtin_elementwise_min(lo, top);
+            hi = __builtin_elementwise_min(hi, top);
+            if (!NONNEG) {
+                lo = __builtin_elementwise_max(lo, bot);
+                hi = __builtin_elementwise_max(hi, bot);
+            }
+            packed[h][r] =
+                (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // the second half's scalars are fetched after the first half is done
+    }
+    int8_t* op = out + (size_t)plane * OHW * 8;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int oy = oy0 + r;
+        if (oy < g.OH) *reinterpret_cast<v2i*>(op + ((size_t)oy * g.OW + ox) * 8) = v2i{packed[0][r], packed[1][r]};
     }
 }
 
@@ -141,12 +245,26 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
         const int R = g.sh == 1 ? R1 : R2;
         const int n_strips = (g.OH + R - 1) / R;
         const int blocks = (n_strips * g.OW + 255) / 256;
-        if (g.sh == 1)
-            hipLaunchKernelGGL((conv_dw3x3_kernel<1, R1>), dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g,
-                               ep, n_strips);
-        else
-            hipLaunchKernelGGL((conv_dw3x3_kernel<2, R2>), dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g,
-                               ep, n_strips);
+        const int epi = pick_epilogue(ep, g.K);
+#define OHIP_DW(S_, R_, E_) \
+    hipLaunchKernelGGL((conv_dw3x3_kernel<S_, R_, E_>), dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g, ep, \
+                       n_strips)
+        const int col_chunks = (g.OW + 63) / 64;
+        const int blocks8 = col_chunks * ((n_strips + 3) / 4);
+#define OHIP_DW8(S_, R_, N_) \
+    hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, planes), dim3(256), 0, stream, x, wmask, \
+                       (int8_t*)out, g, ep, n_strips, col_chunks)
+        if (g.sh == 1) {
+            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(1, R1, true);
+            else if (epi == EPI_I8_P8) OHIP_DW8(1, R1, false);
+            else OHIP_DW(1, R1, EPI_GENERIC);
+        } else {
+            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(2, R2, true);
+            else if (epi == EPI_I8_P8) OHIP_DW8(2, R2, false);
+            else OHIP_DW(2, R2, EPI_GENERIC);
+        }
+#undef OHIP_DW
+#undef OHIP_DW8
     } else {
         const int blocks = (g.OH * g.OW + 255) / 256;
         hipLaunchKernelGGL(conv_dw_generic_kernel, dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g, ep);

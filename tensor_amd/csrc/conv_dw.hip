@@ -27,6 +27,14 @@ void dw_pack_weights(const int8_t* w, int C, int kh, int kw, int32_t* dst) {
             }
 }
 
+// first tap: the three-operand form with a literal zero accumulator (the compiler would otherwise emit a zeroing
+// move plus the accumulate-in-place form for every output)
+__device__ __forceinline__ int dot4_first(int x, int w) {
+    int r;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(x), "s"(w));
+    return r;
+}
+
 __device__ __forceinline__ void mac8(int (&acc)[8], v2i px, const int* __restrict__ wm) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) acc[e] = __builtin_amdgcn_sdot4(px[0], wm[e], acc[e], false);
@@ -113,7 +121,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
     const int plane = blockIdx.y;
     const int o = plane % C8;
     const int chunk = blockIdx.x % col_chunks;
-    const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * 4 + (threadIdx.x >> 6));
+    const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * (blockDim.x >> 6) + (threadIdx.x >> 6));
     const int ox = chunk * 64 + (threadIdx.x & 63);
     if (strip >= n_strips || ox >= g.OW) return;
 
@@ -121,8 +129,9 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
     const int ix0 = ox * S - g.pw;
     // columns 0 and 2 of the window can fall off the image for the first / last output column only: read a clamped
     // address and zero the value
-    const bool c0_ok = ix0 >= 0, c2_ok = ix0 + 2 < g.W, c1_ok = ix0 + 1 < g.W;
-    const int ixc0 = max(ix0, 0), ixc1 = min(ix0 + 1, g.W - 1), ixc2 = min(ix0 + 2, g.W - 1);
+    // (the middle column is always inside: pad <= 1 is checked on the host)
+    const bool c0_ok = ix0 >= 0, c2_ok = ix0 + 2 < g.W;
+    const int ixc0 = max(ix0, 0), ixc1 = ix0 + 1, ixc2 = min(ix0 + 2, g.W - 1);
     const int oy0 = strip * R;
     const int OHW = g.OH * g.OW;
 
@@ -138,7 +147,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
             const v2i b = *reinterpret_cast<const v2i*>(rp + (size_t)ixc1 * 8);
             const v2i c = *reinterpret_cast<const v2i*>(rp + (size_t)ixc2 * 8);
             rows[r][0] = c0_ok ? a : v2i{0, 0};
-            rows[r][1] = c1_ok ? b : v2i{0, 0};
+            rows[r][1] = b;
             rows[r][2] = c2_ok ? c : v2i{0, 0};
         } else {
             rows[r][0] = rows[r][1] = rows[r][2] = v2i{0, 0};
@@ -158,7 +167,8 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             si[e] = ep.scale_in[o * 8 + h * 4 + e];
-            bi[e] = ep.bias[o * 8 + h * 4 + e];
+            // the bias lives in a vector register: fma(acc, scale, bias) may name only one scalar operand
+            asm volatile("v_mov_b32 %0, %1" : "=v"(bi[e]) : "s"(ep.bias[o * 8 + h * 4 + e]));
             so[e] = ep.scale_out[o * 8 + h * 4 + e];
         }
 #pragma unroll
@@ -166,7 +176,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
             int q[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                int acc = __builtin_amdgcn_sdot4(rows[r * S][0][h], wm[0][e], 0, false);
+                int acc = dot4_first(rows[r * S][0][h], wm[0][e]);
 #pragma unroll
                 for (int k = 1; k < 9; ++k) acc = __builtin_amdgcn_sdot4(rows[r * S + k / 3][k % 3][h], wm[k][e], acc, false);
                 float v = __fmaf_rn((float)acc, si[e], bi[e]);
@@ -245,14 +255,17 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
         const int R = g.sh == 1 ? R1 : R2;
         const int n_strips = (g.OH + R - 1) / R;
         const int blocks = (n_strips * g.OW + 255) / 256;
-        const int epi = pick_epilogue(ep, g.K);
+        int epi = pick_epilogue(ep, g.K);
+        if (g.pw > 1 || g.ph > 1) epi = EPI_GENERIC;  // the fast kernel assumes the window's middle column is inside
 #define OHIP_DW(S_, R_, E_) \
     hipLaunchKernelGGL((conv_dw3x3_kernel<S_, R_, E_>), dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g, ep, \
                        n_strips)
+        // one wave per (strip, 64-column chunk); waves per workgroup chosen so that no wave is born idle
         const int col_chunks = (g.OW + 63) / 64;
-        const int blocks8 = col_chunks * ((n_strips + 3) / 4);
+        const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
+        const int blocks8 = col_chunks * (n_strips / wpb);
 #define OHIP_DW8(S_, R_, N_) \
-    hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, planes), dim3(256), 0, stream, x, wmask, \
+    hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, planes), dim3(64 * wpb), 0, stream, x, wmask, \
                        (int8_t*)out, g, ep, n_strips, col_chunks)
         if (g.sh == 1) {
             if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(1, R1, true);

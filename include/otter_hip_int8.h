@@ -171,6 +171,27 @@ int otter_hip_requantize(const int32_t* src, int src_layout, int n, int c, int h
 int otter_hip_repack(const void* src, int src_layout, int n, int c, int h, int w, void* dst, int dst_layout,
                      void* stream);
 
+/* ------------------------------------------------------------------------------------------------ */
+/* fp32 glue between the int8 layers of a network (all pointers are device pointers)                */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* EltwiseLayer::forward, operation sum (Tensor/EltwiseLayer.cpp:48-80): out = a + b over `count` floats of two
+ * blobs in the same layout. */
+int otter_hip_eltwise_add(const float* a, const float* b, float* out, size_t count, void* stream);
+
+/* ReluLayer / LReluLayer / Relu6Layer / SigmoidLayer::forward_inplace (Tensor/ReluLayer.cpp, LReluLayer.cpp:45-,
+ * Relu6Layer.cpp:29-100) on a device blob; activation_type as in otter_hip_conv_desc. */
+int otter_hip_activation(float* x, size_t count, int activation_type, float activation_param0, void* stream);
+
+/* Global average pooling to [N, C] (unpacked). The reference registry has no average-pooling layer
+ * (Tensor/LayerDeclaration.hpp:42-68); this is the fp32 mean over H*W that the MobileNetV2-style network needs. */
+int otter_hip_global_avgpool(const float* src, int src_layout, int n, int c, int h, int w, float* dst, void* stream);
+
+/* InnerProductLayer::forward, fp32 (Tensor/InnerProductLayer.cpp:176-): y[n][o] = sum_i x[n][i]*weight[o][i] + bias[o].
+ * bias may be NULL. */
+int otter_hip_inner_product(const float* x, int n, int in_features, const float* weight, const float* bias,
+                            int out_features, float* y, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

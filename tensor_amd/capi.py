@@ -65,7 +65,9 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_stream_destroy", "otter_hip_stream_synchronize", "otter_hip_conv_create",
            "otter_hip_conv_destroy", "otter_hip_conv_output_shape", "otter_hip_conv_default_out_layout",
            "otter_hip_conv_workspace_bytes", "otter_hip_conv_forward", "otter_hip_conv_kernel_kind",
-           "otter_hip_quantize", "otter_hip_dequantize", "otter_hip_requantize", "otter_hip_repack"]
+           "otter_hip_quantize", "otter_hip_dequantize", "otter_hip_requantize", "otter_hip_repack",
+           "otter_hip_conv_set_tile", "otter_hip_eltwise_add", "otter_hip_activation", "otter_hip_global_avgpool",
+           "otter_hip_inner_product"]
 
 
 def load_cdll():

@@ -409,4 +409,37 @@ int otter_hip_repack(const void* src, int src_layout, int n, int c, int h, int w
     return OTTER_HIP_OK;
 }
 
+// -----------------------------------------------------------------------------------------------------
+// fp32 glue between the int8 layers of a network
+// -----------------------------------------------------------------------------------------------------
+
+int otter_hip_eltwise_add(const float* a, const float* b, float* out, size_t count, void* stream) {
+    if (!a || !b || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_eltwise_add: null");
+    OHIP_CHECK(run_eltwise_add(a, b, out, count, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_activation(float* x, size_t count, int activation_type, float activation_param0, void* stream) {
+    if (!x) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_activation: null");
+    if (activation_type < 0 || activation_type > 4)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_activation: activation type not supported");
+    OHIP_CHECK(run_activation(x, count, activation_type, activation_param0, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_global_avgpool(const float* src, int src_layout, int n, int c, int h, int w, float* dst, void* stream) {
+    if (!src || !dst) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_global_avgpool: null");
+    if (!valid_layout(src_layout) || layout_elem(src_layout) != 0 || c % layout_pack(src_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_global_avgpool: bad layout");
+    OHIP_CHECK(run_global_avgpool(src, layout_pack(src_layout), n, c, h * w, dst, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_inner_product(const float* x, int n, int in_features, const float* weight, const float* bias,
+                            int out_features, float* y, void* stream) {
+    if (!x || !weight || !y) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_inner_product: null");
+    OHIP_CHECK(run_inner_product(x, weight, bias, y, n, in_features, out_features, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
 }  // extern "C"

@@ -1,0 +1,1071 @@
+// Implementation of the host-side mirror of Otter's Layer / ConvolutionLayer / Net interface over the C ABI.
+#include "otter_hip.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <random>
+#include <sstream>
+
+#include "../../include/otter_hip_int8.h"
+
+namespace otter {
+
+namespace {
+
+void hip_check(int rc, const char* what) {
+    if (rc != 0) throw Error(std::string(what) + ": " + otter_hip_last_error());
+}
+
+std::string trim(std::string s) {
+    s.erase(std::remove_if(s.begin(), s.end(), [](unsigned char c) { return c == ' '; }), s.end());
+    return s;
+}
+
+std::vector<std::string> split_list(const std::string& s) {
+    std::vector<std::string> out;
+    std::stringstream ss(s);
+    std::string item;
+    while (std::getline(ss, item, ',')) {
+        item = trim(item);
+        if (!item.empty()) out.push_back(item);
+    }
+    return out;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------
+// dtypes
+// ---------------------------------------------------------------------------------------------------
+int elempack_of(ScalarType t) {
+    switch (t) {
+    case ScalarType::Float4:
+    case ScalarType::Int4:
+        return 4;
+    case ScalarType::Float8:
+    case ScalarType::Byte8:
+    case ScalarType::Int8:
+        return 8;
+    default:
+        return 1;
+    }
+}
+
+ScalarType base_of(ScalarType t) {
+    switch (t) {
+    case ScalarType::Float:
+    case ScalarType::Float4:
+    case ScalarType::Float8:
+        return ScalarType::Float;
+    case ScalarType::Byte:
+    case ScalarType::Byte8:
+        return ScalarType::Byte;
+    case ScalarType::Int:
+    case ScalarType::Int4:
+    case ScalarType::Int8:
+        return ScalarType::Int;
+    default:
+        return ScalarType::Undefined;
+    }
+}
+
+size_t elemsize_of(ScalarType t) { return (base_of(t) == ScalarType::Byte ? 1 : 4) * (size_t)elempack_of(t); }
+
+ScalarType scalar_type_of(ScalarType base, int p) {
+    base = base_of(base);
+    if (base == ScalarType::Float) return p == 8 ? ScalarType::Float8 : (p == 4 ? ScalarType::Float4 : ScalarType::Float);
+    if (base == ScalarType::Byte) return p == 8 ? ScalarType::Byte8 : ScalarType::Byte;
+    if (base == ScalarType::Int) return p == 8 ? ScalarType::Int8 : (p == 4 ? ScalarType::Int4 : ScalarType::Int);
+    return ScalarType::Undefined;
+}
+
+int hip_layout_of(ScalarType t) {
+    switch (t) {
+    case ScalarType::Float: return OTTER_HIP_F32;
+    case ScalarType::Float4: return OTTER_HIP_F32_P4;
+    case ScalarType::Float8: return OTTER_HIP_F32_P8;
+    case ScalarType::Byte: return OTTER_HIP_I8;
+    case ScalarType::Byte8: return OTTER_HIP_I8_P8;
+    case ScalarType::Int: return OTTER_HIP_I32;
+    case ScalarType::Int4: return OTTER_HIP_I32_P4;
+    case ScalarType::Int8: return OTTER_HIP_I32_P8;
+    default: return -1;
+    }
+}
+
+static ScalarType scalar_type_of_layout(int layout) {
+    static const ScalarType map[] = {ScalarType::Float, ScalarType::Float4, ScalarType::Float8, ScalarType::Byte,
+                                     ScalarType::Byte8, ScalarType::Int,    ScalarType::Int4,   ScalarType::Int8};
+    return map[layout];
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Tensor
+// ---------------------------------------------------------------------------------------------------
+// Device blobs are recycled through a size-keyed free list (the role CPUCachingAllocator plays in the reference,
+// Tensor/CPUCachingAllocator.hpp): a network asks for the same sizes on every pass, and hipFree would synchronise
+// the device each time. All work of this layer is issued on one stream, so a recycled buffer is never still in use.
+namespace {
+struct DevicePool {
+    std::mutex mu;
+    std::multimap<size_t, void*> free_list;
+    void* get(size_t bytes) {
+        {
+            std::lock_guard<std::mutex> g(mu);
+            auto it = free_list.find(bytes);
+            if (it != free_list.end()) {
+                void* p = it->second;
+                free_list.erase(it);
+                return p;
+            }
+        }
+        void* p = nullptr;
+        if (otter_hip_malloc(&p, bytes) != 0) {
+            release_all();
+            hip_check(otter_hip_malloc(&p, bytes), "device allocation");
+        }
+        return p;
+    }
+    void put(size_t bytes, void* p) {
+        std::lock_guard<std::mutex> g(mu);
+        free_list.emplace(bytes, p);
+    }
+    void release_all() {
+        std::lock_guard<std::mutex> g(mu);
+        for (auto& kv : free_list) otter_hip_free(kv.second);
+        free_list.clear();
+    }
+};
+DevicePool& pool() {
+    static DevicePool* p = new DevicePool();
+    return *p;
+}
+}  // namespace
+
+void device_cache_clear() { pool().release_all(); }
+
+struct Tensor::Storage {
+    void* host = nullptr;
+    void* dev = nullptr;
+    size_t bytes = 0;
+    bool host_valid = false, dev_valid = false;
+    ~Storage() {
+        std::free(host);
+        if (dev) pool().put(bytes, dev);
+    }
+};
+
+int64_t Tensor::numel() const {
+    int64_t n = 1;
+    for (auto s : sizes_) n *= s;
+    return sizes_.empty() ? 0 : n;
+}
+
+Tensor Tensor::empty(const std::vector<int64_t>& sizes, ScalarType dtype) {
+    Tensor t;
+    t.sizes_ = sizes;
+    t.dtype_ = dtype;
+    t.st_ = std::make_shared<Storage>();
+    t.st_->bytes = t.nbytes();
+    t.st_->host = std::malloc(t.st_->bytes ? t.st_->bytes : 1);
+    if (!t.st_->host) throw Error("Tensor::empty: host allocation failed");
+    t.st_->host_valid = true;
+    return t;
+}
+
+Tensor Tensor::empty_device(const std::vector<int64_t>& sizes, ScalarType dtype) {
+    Tensor t;
+    t.sizes_ = sizes;
+    t.dtype_ = dtype;
+    t.st_ = std::make_shared<Storage>();
+    t.st_->bytes = t.nbytes();
+    t.st_->dev = pool().get(t.st_->bytes);
+    t.st_->dev_valid = true;
+    return t;
+}
+
+Tensor Tensor::from_blob(const void* data, const std::vector<int64_t>& sizes, ScalarType dtype) {
+    Tensor t = empty(sizes, dtype);
+    std::memcpy(t.st_->host, data, t.st_->bytes);
+    return t;
+}
+
+const void* Tensor::data_ptr() const {
+    OTTER_CHECK(defined(), "data_ptr of an undefined tensor");
+    Storage& s = *st_;
+    if (!s.host) {
+        s.host = std::malloc(s.bytes ? s.bytes : 1);
+        if (!s.host) throw Error("Tensor: host allocation failed");
+    }
+    if (!s.host_valid) {
+        OTTER_CHECK(s.dev_valid, "tensor has no valid copy");
+        hip_check(otter_hip_memcpy_d2h(s.host, s.dev, s.bytes, nullptr), "download");
+        hip_check(otter_hip_stream_synchronize(nullptr), "download");
+        s.host_valid = true;
+    }
+    return s.host;
+}
+
+void* Tensor::data_ptr() {
+    void* p = const_cast<void*>(static_cast<const Tensor*>(this)->data_ptr());
+    st_->dev_valid = false;  // the caller may write through the pointer
+    return p;
+}
+
+void* Tensor::device_ptr() const {
+    OTTER_CHECK(defined(), "device_ptr of an undefined tensor");
+    Storage& s = *st_;
+    if (!s.dev) s.dev = pool().get(s.bytes);
+    if (!s.dev_valid) {
+        OTTER_CHECK(s.host_valid, "tensor has no valid copy");
+        hip_check(otter_hip_memcpy_h2d(s.dev, s.host, s.bytes, nullptr), "upload");
+        s.dev_valid = true;
+    }
+    return s.dev;
+}
+
+bool Tensor::on_device() const { return st_ && st_->dev_valid; }
+
+void Tensor::mark_device_written() {
+    st_->dev_valid = true;
+    st_->host_valid = false;
+}
+
+Tensor Tensor::view(const std::vector<int64_t>& sizes) const {
+    Tensor t = *this;
+    int64_t n = 1, neg = -1;
+    std::vector<int64_t> s = sizes;
+    for (size_t i = 0; i < s.size(); ++i) {
+        if (s[i] < 0) neg = (int64_t)i;
+        else n *= s[i];
+    }
+    if (neg >= 0) s[neg] = numel() / n;
+    t.sizes_ = s;
+    OTTER_CHECK(t.numel() == numel(), "view: size mismatch");
+    return t;
+}
+
+Tensor Tensor::packing(int p) const {
+    OTTER_CHECK(defined() && dim() == 4, "packing: 4-d tensor expected");
+    const int p0 = elempack();
+    if (p == p0) return *this;
+    const int64_t N = sizes_[0], C = sizes_[1] * p0, H = sizes_[2], W = sizes_[3];
+    OTTER_CHECK(C % p == 0, "packing: elempack does not divide the channel count");
+    const ScalarType dt = scalar_type_of(dtype_, p);
+    OTTER_CHECK(dt != ScalarType::Undefined && elempack_of(dt) == p, "packing: no such packed dtype");
+    if (on_device()) {  // keep it on the device
+        Tensor out = empty_device({N, C / p, H, W}, dt);
+        hip_check(otter_hip_repack(device_ptr(), hip_layout_of(dtype_), (int)N, (int)C, (int)H, (int)W, out.device_ptr(),
+                                   hip_layout_of(dt), nullptr),
+                  "packing");
+        return out;
+    }
+    Tensor out = empty({N, C / p, H, W}, dt);
+    const size_t eb = base_of(dtype_) == ScalarType::Byte ? 1 : 4;
+    const char* s = static_cast<const char*>(data_ptr());
+    char* d = static_cast<char*>(out.st_->host);
+    const int64_t HW = H * W;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int64_t i = 0; i < HW; ++i)
+                std::memcpy(d + ((((n * (C / p) + c / p) * HW + i) * p) + c % p) * eb,
+                            s + ((((n * (C / p0) + c / p0) * HW + i) * p0) + c % p0) * eb, eb);
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// ParamDict / options
+// ---------------------------------------------------------------------------------------------------
+int ParamDict::get(int id, int def) const {
+    auto it = params_.find(id);
+    return it == params_.end() || it->second.type != 1 ? def : it->second.i;
+}
+float ParamDict::get(int id, float def) const {
+    auto it = params_.find(id);
+    return it == params_.end() || it->second.type != 2 ? def : it->second.f;
+}
+Tensor ParamDict::get(int id, const Tensor& def) const {
+    auto it = params_.find(id);
+    return it == params_.end() || it->second.type != 3 ? def : it->second.t;
+}
+void ParamDict::set(int id, int i) {
+    params_[id].type = 1;
+    params_[id].i = i;
+}
+void ParamDict::set(int id, float f) {
+    params_[id].type = 2;
+    params_[id].f = f;
+}
+void ParamDict::set(int id, const Tensor& t) {
+    params_[id].type = 3;
+    params_[id].t = t;
+}
+void ParamDict::clear() { params_.clear(); }
+
+bool opt_find(const LayerOption& o, const std::string& k) { return o.find(k) != o.end(); }
+int opt_find_int(const LayerOption& o, const std::string& k, int def) {
+    auto it = o.find(k);
+    return it == o.end() ? def : std::atoi(it->second.c_str());
+}
+float opt_find_float(const LayerOption& o, const std::string& k, float def) {
+    auto it = o.find(k);
+    return it == o.end() ? def : (float)std::atof(it->second.c_str());
+}
+std::string opt_find_string(const LayerOption& o, const std::string& k, const std::string& def) {
+    auto it = o.find(k);
+    return it == o.end() ? def : it->second;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Layer base + registry
+// ---------------------------------------------------------------------------------------------------
+int Layer::parse_param(LayerOption&, ParamDict&) { return 0; }
+int Layer::compute_output_shape(ParamDict&) {
+    top_shapes = bottom_shapes;
+    return 0;
+}
+int Layer::load_param(const ParamDict&) { return 0; }
+int Layer::init_model() { return 0; }
+int Layer::load_model(const Initializer&) { return 0; }
+int Layer::create_pipeline(const NetOption&) { return 0; }
+int Layer::forward(const Tensor& bottom, Tensor& top, const NetOption& opt) const {
+    if (!support_inplace) return -1;
+    top = bottom;
+    return forward_inplace(top, opt);
+}
+int Layer::forward(const std::vector<Tensor>& bottoms, std::vector<Tensor>& tops, const NetOption& opt) const {
+    if (!support_inplace) return -1;
+    tops = bottoms;
+    for (auto& t : tops) {
+        int rc = forward_inplace(t, opt);
+        if (rc) return rc;
+    }
+    return 0;
+}
+int Layer::forward_inplace(Tensor&, const NetOption&) const { return -1; }
+
+static std::map<std::string, LayerRegistry::Creator>& registry() {
+    static auto* r = new std::map<std::string, LayerRegistry::Creator>();
+    return *r;
+}
+void LayerRegistry::AddCreator(const std::string& type, Creator creator) { registry()[type] = creator; }
+Layer* LayerRegistry::CreateLayer(const std::string& type) {
+    auto it = registry().find(type);
+    return it == registry().end() ? nullptr : it->second();
+}
+std::vector<std::string> LayerRegistry::TypeList() {
+    std::vector<std::string> v;
+    for (auto& kv : registry()) v.push_back(kv.first);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// ConvolutionLayer
+// ---------------------------------------------------------------------------------------------------
+ConvolutionLayer::ConvolutionLayer() {
+    one_blob_only = true;
+    support_inplace = false;
+    support_packing = true;
+}
+
+ConvolutionLayer::~ConvolutionLayer() {
+    if (handle_) otter_hip_conv_destroy(handle_);
+}
+
+// option keys and defaults of Tensor/ConvolutionLayer.cpp:58-156
+int ConvolutionLayer::parse_param(LayerOption& option, ParamDict& pd) {
+    pd.clear();
+    auto pair = [&](const char* hk, const char* wk, const char* k, int def, int lo, int& h, int& w) {
+        h = opt_find_int(option, hk, -1);
+        w = opt_find_int(option, wk, -1);
+        const int both = opt_find_int(option, k, def);
+        if (h < lo) h = both;
+        if (w < lo) w = both;
+    };
+    int kh, kw, sh, sw, ph, pw, dh, dw, oph, opw;
+    pair("kernel_h", "kernel_w", "kernel", 3, 1, kh, kw);
+    pair("stride_h", "stride_w", "stride", 1, 1, sh, sw);
+    pair("padding_h", "padding_w", "padding", 0, 0, ph, pw);
+    pair("dilation_h", "dilation_w", "dilation", 1, 1, dh, dw);
+    pair("output_padding_h", "output_padding_w", "output_padding", 0, 0, oph, opw);
+    int bias = opt_find(option, "batchnorm") ? 0 : 1;
+    if (opt_find(option, "bias_term")) bias = option["bias_term"] == "false" ? 0 : 1;
+    const std::string act = opt_find_string(option, "activation", "");
+    int act_type = act == "Relu" ? 1 : act == "LRelu" ? 2 : act == "Relu6" ? 3 : act == "Sigmoid" ? 4 : 0;
+    Tensor act_params;
+    if (opt_find(option, "activation_params")) {
+        auto items = split_list(option["activation_params"]);
+        act_params = Tensor::empty({(int64_t)items.size()}, ScalarType::Float);
+        for (size_t i = 0; i < items.size(); ++i) act_params.data_ptr<float>()[i] = (float)std::atof(items[i].c_str());
+    }
+    if (opt_find(option, "batchnorm")) act_type = 0;
+    pd.set((int)ConvParam::In_channels, opt_find_int(option, "in_channels", 1));
+    pd.set((int)ConvParam::Out_channels, opt_find_int(option, "out_channels", 1));
+    pd.set((int)ConvParam::Kernel_height, kh);
+    pd.set((int)ConvParam::Kernel_width, kw);
+    pd.set((int)ConvParam::Stride_height, sh);
+    pd.set((int)ConvParam::Stride_width, sw);
+    pd.set((int)ConvParam::Padding_height, ph);
+    pd.set((int)ConvParam::Padding_width, pw);
+    pd.set((int)ConvParam::Dilation_height, dh);
+    pd.set((int)ConvParam::Dilation_width, dw);
+    pd.set((int)ConvParam::Output_padding_height, oph);
+    pd.set((int)ConvParam::Output_padding_width, opw);
+    pd.set((int)ConvParam::Group, opt_find_int(option, "groups", 1));
+    pd.set((int)ConvParam::Bias_term, bias);
+    pd.set((int)ConvParam::Int8_scale_term, opt_find_int(option, "int8_scale_term", 0));
+    pd.set((int)ConvParam::Activation_type, act_type);
+    pd.set((int)ConvParam::Activation_params, act_params);
+    return 0;
+}
+
+// Tensor/ConvolutionLayer.cpp:158-183
+int ConvolutionLayer::compute_output_shape(ParamDict& pd) {
+    OTTER_CHECK(!bottom_shapes.empty() && bottom_shapes[0].size() == 4, "Convolution: 4-d bottom shape expected");
+    const auto& in = bottom_shapes[0];
+    const int K = pd.get((int)ConvParam::Out_channels, 1);
+    const int kh = pd.get((int)ConvParam::Kernel_height, 3), kw = pd.get((int)ConvParam::Kernel_width, 3);
+    const int sh = pd.get((int)ConvParam::Stride_height, 1), sw = pd.get((int)ConvParam::Stride_width, 1);
+    const int ph = pd.get((int)ConvParam::Padding_height, 0), pw = pd.get((int)ConvParam::Padding_width, 0);
+    const int dh = pd.get((int)ConvParam::Dilation_height, 1), dw = pd.get((int)ConvParam::Dilation_width, 1);
+    const int g = pd.get((int)ConvParam::Group, 1);
+    const int64_t ow = (in[3] + 2 * pw - dw * (kw - 1) - 1) / sw + 1;
+    const int64_t oh = (in[2] + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
+    pd.set((int)ConvParam::In_channels, (int)in[1]);
+    pd.set((int)ConvParam::Weight_data_size, (int)(in[1] / g * kh * kw * K));
+    top_shapes = {{in[0], K, oh, ow}};
+    return 0;
+}
+
+int ConvolutionLayer::load_param(const ParamDict& pd) {
+    in_channels = pd.get((int)ConvParam::In_channels, 1);
+    out_channels = pd.get((int)ConvParam::Out_channels, 1);
+    kernel_height = pd.get((int)ConvParam::Kernel_height, 3);
+    kernel_width = pd.get((int)ConvParam::Kernel_width, 3);
+    stride_height = pd.get((int)ConvParam::Stride_height, 1);
+    stride_width = pd.get((int)ConvParam::Stride_width, 1);
+    padding_height = pd.get((int)ConvParam::Padding_height, 0);
+    padding_width = pd.get((int)ConvParam::Padding_width, 0);
+    dilation_height = pd.get((int)ConvParam::Dilation_height, 1);
+    dilation_width = pd.get((int)ConvParam::Dilation_width, 1);
+    output_padding_height = pd.get((int)ConvParam::Output_padding_height, 0);
+    output_padding_width = pd.get((int)ConvParam::Output_padding_width, 0);
+    groups = pd.get((int)ConvParam::Group, 1);
+    bias_term = pd.get((int)ConvParam::Bias_term, 0);
+    weight_data_size = pd.get((int)ConvParam::Weight_data_size, 0);
+    int8_scale_term = pd.get((int)ConvParam::Int8_scale_term, 0);
+    activation_type = pd.get((int)ConvParam::Activation_type, 0);
+    activation_params = pd.get((int)ConvParam::Activation_params, Tensor());
+    return 0;
+}
+
+// random int8 model (the "no weight file" mode of Tensor/ConvolutionLayer.cpp:208-243; signed weights here)
+int ConvolutionLayer::init_model() {
+    if (!int8_scale_term) return -1;  // fp32 convolutions are not part of this path
+    std::mt19937 rng(1234u + (unsigned)out_channels * 31u + (unsigned)in_channels);
+    const int64_t per = (int64_t)(in_channels / groups) * kernel_height * kernel_width;
+    weight_data = Tensor::empty({out_channels, in_channels / groups, kernel_height, kernel_width}, ScalarType::Byte);
+    int8_t* w = weight_data.data_ptr<int8_t>();
+    std::uniform_int_distribution<int> wd(-127, 127);
+    for (int64_t i = 0; i < per * out_channels; ++i) w[i] = (int8_t)wd(rng);
+    std::uniform_real_distribution<float> ud(0.f, 1.f);
+    if (bias_term) {
+        bias_data = Tensor::empty({out_channels}, ScalarType::Float);
+        for (int i = 0; i < out_channels; ++i) bias_data.data_ptr<float>()[i] = ud(rng);
+    }
+    const bool dw = in_channels == groups && groups == out_channels;
+    weight_data_int8_scales = Tensor::empty({out_channels}, ScalarType::Float);
+    for (int i = 0; i < out_channels; ++i) weight_data_int8_scales.data_ptr<float>()[i] = 50.f + 200.f * ud(rng);
+    const int nb = dw ? groups : 1;
+    bottom_blob_int8_scales = Tensor::empty({nb}, ScalarType::Float);
+    const float bs = 10.f + 50.f * ud(rng);
+    for (int i = 0; i < nb; ++i) bottom_blob_int8_scales.data_ptr<float>()[i] = bs;
+    if (int8_scale_term > 100) {
+        top_blob_int8_scales = Tensor::empty({nb}, ScalarType::Float);
+        const float ts = 5.f + 20.f * ud(rng);
+        for (int i = 0; i < nb; ++i) top_blob_int8_scales.data_ptr<float>()[i] = ts;
+    }
+    return 0;
+}
+
+// order of the ncnn weight stream: Tensor/ConvolutionLayer.cpp:245-296
+int ConvolutionLayer::load_model(const Initializer& in) {
+    weight_data = in.load({out_channels, in_channels / groups, kernel_height, kernel_width}, 0);
+    if (bias_term) bias_data = in.load({out_channels}, 1);
+    const bool dw = in_channels == groups && groups == out_channels;
+    auto replicate = [&](const Tensor& one, int n) {
+        Tensor t = Tensor::empty({n}, ScalarType::Float);
+        for (int i = 0; i < n; ++i) t.data_ptr<float>()[i] = one.data_ptr<float>()[0];
+        return t;
+    };
+    if (dw) {
+        if (int8_scale_term == 1 || int8_scale_term == 101) {
+            weight_data_int8_scales = in.load({groups}, 1);
+            bottom_blob_int8_scales = replicate(in.load({1}, 1), groups);
+        } else if (int8_scale_term == 2 || int8_scale_term == 102) {
+            weight_data_int8_scales = replicate(in.load({1}, 1), groups);
+            bottom_blob_int8_scales = replicate(in.load({1}, 1), groups);
+        }
+        if (int8_scale_term > 100) top_blob_int8_scales = replicate(in.load({1}, 1), groups);
+    } else {
+        if (int8_scale_term) {
+            weight_data_int8_scales = in.load({out_channels}, 1);
+            bottom_blob_int8_scales = in.load({1}, 1);
+        }
+        if (int8_scale_term > 100) top_blob_int8_scales = in.load({1}, 1);
+    }
+    return 0;
+}
+
+int ConvolutionLayer::create_pipeline(const NetOption& opt) {
+    if (weight_data.defined() && weight_data.scalar_type() == ScalarType::Byte) return create_pipeline_int8(opt);
+    return -1;  // fp32 convolution: outside the accelerated path
+}
+
+// Tensor/ConvolutionLayer.cpp:666-752: scale_in on the host (true division), weights re-laid-out once
+int ConvolutionLayer::create_pipeline_int8(const NetOption& opt) {
+    OTTER_CHECK(weight_data_int8_scales.defined() && bottom_blob_int8_scales.defined(),
+                "Convolution: int8 scales missing");
+    scale_in_data = Tensor::empty({out_channels}, ScalarType::Float);
+    const float* ws = weight_data_int8_scales.data_ptr<float>();
+    const float in_scale = bottom_blob_int8_scales.data_ptr<float>()[0];
+    for (int p = 0; p < out_channels; ++p)
+        scale_in_data.data_ptr<float>()[p] = ws[p] == 0 ? 0.f : 1.f / (in_scale * ws[p]);
+
+    otter_hip_conv_desc d;
+    d.in_channels = in_channels, d.out_channels = out_channels;
+    d.kernel_h = kernel_height, d.kernel_w = kernel_width, d.stride_h = stride_height, d.stride_w = stride_width;
+    d.pad_h = padding_height, d.pad_w = padding_width, d.dilation_h = dilation_height, d.dilation_w = dilation_width;
+    d.groups = groups, d.activation_type = activation_type;
+    d.activation_param0 = activation_params.defined() ? activation_params.data_ptr<float>()[0] : 0.1f;
+    d.out_kind = int8_scale_term > 100 ? OTTER_HIP_OUT_I8 : OTTER_HIP_OUT_F32;
+    // which rounding primitive the reference's routing ends in (Tensor/QuantizeX86.cpp:402,1177-1179,1729)
+    const bool pk = opt.use_packing_layout;
+    const bool dw8 = in_channels == groups && groups == out_channels && in_channels % 8 == 0;
+    d.in_round_mode = (pk && in_channels % 8 == 0) ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT;
+    d.out_round_mode = (pk && (dw8 || out_channels % 4 == 0)) ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT;
+    if (handle_) {
+        otter_hip_conv_destroy(handle_);
+        handle_ = nullptr;
+    }
+    const float* top = top_blob_int8_scales.defined() ? top_blob_int8_scales.data_ptr<float>() : nullptr;
+    if (d.out_kind == OTTER_HIP_OUT_I8 && !top) return -1;
+    return otter_hip_conv_create(&d, weight_data.data_ptr<int8_t>(), scale_in_data.data_ptr<float>(),
+                                 bias_term && bias_data.defined() ? bias_data.data_ptr<float>() : nullptr, in_scale, top,
+                                 top ? 1 : 0, &handle_);
+}
+
+int ConvolutionLayer::forward(const Tensor& bottom, Tensor& top, const NetOption& opt) const {
+    if (int8_scale_term) return forward_int8(bottom, top, opt);
+    return -1;
+}
+
+// Tensor/ConvolutionLayer.cpp:754-847, whole batch in one launch
+int ConvolutionLayer::forward_int8(const Tensor& bottom, Tensor& top, const NetOption& opt) const {
+    if (!handle_ || !bottom.defined() || bottom.dim() != 4) return -1;
+    const int in_layout = hip_layout_of(bottom.scalar_type());
+    if (in_layout < 0 || base_of(bottom.scalar_type()) == ScalarType::Int) return -1;
+    const int N = (int)bottom.size(0), H = (int)bottom.size(2), W = (int)bottom.size(3);
+    if (bottom.channels() != in_channels) return -1;
+    int oh = 0, ow = 0;
+    if (otter_hip_conv_output_shape(handle_, H, W, &oh, &ow)) return -1;
+    int out_layout = otter_hip_conv_default_out_layout(handle_);
+    if (!opt.use_packing_layout)
+        out_layout = int8_scale_term > 100 ? OTTER_HIP_I8 : OTTER_HIP_F32;
+    if (force_out_layout >= 0) out_layout = force_out_layout;
+    const ScalarType odt = scalar_type_of_layout(out_layout);
+    try {
+        top = Tensor::empty_device({N, out_channels / elempack_of(odt), oh, ow}, odt);
+        Tensor ws;
+        const size_t ws_bytes = otter_hip_conv_workspace_bytes(handle_, in_layout, N, H, W);
+        if (ws_bytes) ws = Tensor::empty_device({(int64_t)ws_bytes}, ScalarType::Byte);
+        const int rc = otter_hip_conv_forward(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
+                                              ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
+        if (rc) return rc;
+        top.mark_device_written();
+    } catch (const Error&) {
+        return -100;
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// functional API
+// ---------------------------------------------------------------------------------------------------
+static Tensor to_device_f32(const Tensor& t) { return t; }
+
+Tensor quantize_to_int8(const Tensor& src, const Tensor& scale_data, bool pack) {
+    OTTER_CHECK(src.defined() && src.dim() == 4 && base_of(src.scalar_type()) == ScalarType::Float,
+                "quantize_to_int8: 4-d fp32 tensor expected");
+    const int64_t N = src.size(0), C = src.channels(), H = src.size(2), W = src.size(3);
+    // Tensor/QuantizeX86.cpp:47-58,402,554: only a packed source becomes Byte8
+    const bool to8 = pack && src.elempack() > 1 && C % 8 == 0;
+    const ScalarType odt = to8 ? ScalarType::Byte8 : ScalarType::Byte;
+    Tensor out = Tensor::empty_device({N, C / elempack_of(odt), H, W}, odt);
+    Tensor scales = to_device_f32(scale_data);
+    hip_check(otter_hip_quantize((const float*)src.device_ptr(), hip_layout_of(src.scalar_type()), (int)N, (int)C, (int)H,
+                                 (int)W, (const float*)scales.device_ptr(), (int)scales.numel(),
+                                 to8 ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT, (int8_t*)out.device_ptr(),
+                                 hip_layout_of(odt), nullptr),
+              "quantize_to_int8");
+    out.mark_device_written();
+    return out;
+}
+
+Tensor dequantize_from_int32(const Tensor& src, const Tensor& scale_data, const Tensor& bias_data, bool) {
+    OTTER_CHECK(src.defined() && src.dim() == 4 && base_of(src.scalar_type()) == ScalarType::Int,
+                "dequantize_from_int32: 4-d int32 tensor expected");
+    const int64_t N = src.size(0), C = src.channels(), H = src.size(2), W = src.size(3);
+    const ScalarType odt = scalar_type_of(ScalarType::Float, src.elempack());  // Int4 -> Float4, Int8 -> Float8
+    Tensor out = Tensor::empty_device({N, C / elempack_of(odt), H, W}, odt);
+    const bool has_bias = bias_data.defined() && bias_data.numel() > 0;
+    hip_check(otter_hip_dequantize((const int32_t*)src.device_ptr(), hip_layout_of(src.scalar_type()), (int)N, (int)C,
+                                   (int)H, (int)W, (const float*)scale_data.device_ptr(), (int)scale_data.numel(),
+                                   has_bias ? (const float*)bias_data.device_ptr() : nullptr,
+                                   has_bias ? (int)bias_data.numel() : 0, (float*)out.device_ptr(), hip_layout_of(odt),
+                                   nullptr),
+              "dequantize_from_int32");
+    out.mark_device_written();
+    return out;
+}
+
+Tensor requantize_from_int32_to_int8(const Tensor& src, const Tensor& scale_in, const Tensor& scale_out,
+                                     const Tensor& bias, int act, const Tensor& act_params, bool pack) {
+    OTTER_CHECK(src.defined() && src.dim() == 4 && base_of(src.scalar_type()) == ScalarType::Int,
+                "requantize_from_int32_to_int8: 4-d int32 tensor expected");
+    const int64_t N = src.size(0), C = src.channels(), H = src.size(2), W = src.size(3);
+    // Tensor/QuantizeX86.cpp:1177-1179,1729: elempack 4/8 source -> SIMD rounding, Byte8 when C % 8 == 0
+    const bool packed_src = src.elempack() > 1;
+    const ScalarType odt = (pack && packed_src && C % 8 == 0) ? ScalarType::Byte8 : ScalarType::Byte;
+    Tensor out = Tensor::empty_device({N, C / elempack_of(odt), H, W}, odt);
+    const bool has_bias = bias.defined() && bias.numel() > 0;
+    hip_check(otter_hip_requantize((const int32_t*)src.device_ptr(), hip_layout_of(src.scalar_type()), (int)N, (int)C,
+                                   (int)H, (int)W, (const float*)scale_in.device_ptr(), (int)scale_in.numel(),
+                                   (const float*)scale_out.device_ptr(), (int)scale_out.numel(),
+                                   has_bias ? (const float*)bias.device_ptr() : nullptr, has_bias ? (int)bias.numel() : 0,
+                                   act, act_params.defined() ? act_params.data_ptr<float>()[0] : 0.1f,
+                                   packed_src ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT, (int8_t*)out.device_ptr(),
+                                   hip_layout_of(odt), nullptr),
+              "requantize_from_int32_to_int8");
+    out.mark_device_written();
+    return out;
+}
+
+Tensor convolution(const Tensor& input, const Tensor& weight, const Tensor&, const Tensor&, const std::vector<int>& stride,
+                   const std::vector<int>& padding, const std::vector<int>& dilation, bool transposed,
+                   const std::vector<int>&, int64_t groups, bool packed, const Tensor&, const Tensor&) {
+    OTTER_CHECK(!transposed, "convolution: transposed convolution is not part of the int8 path");
+    OTTER_CHECK(input.defined() && input.dim() == 4 && base_of(input.scalar_type()) == ScalarType::Byte,
+                "convolution: int8 input expected");
+    OTTER_CHECK(weight.defined() && weight.dim() == 4 && weight.scalar_type() == ScalarType::Byte,
+                "convolution: int8 weight [K, C/g, kh, kw] expected");
+    const int K = (int)weight.size(0), C = (int)input.channels();
+    OTTER_CHECK(weight.size(1) * groups == C, "convolution: expected input channels == weight channels * groups");
+    otter_hip_conv_desc d;
+    d.in_channels = C, d.out_channels = K, d.kernel_h = (int)weight.size(2), d.kernel_w = (int)weight.size(3);
+    d.stride_h = stride[0], d.stride_w = stride[stride.size() > 1 ? 1 : 0];
+    d.pad_h = padding[0], d.pad_w = padding[padding.size() > 1 ? 1 : 0];
+    d.dilation_h = dilation[0], d.dilation_w = dilation[dilation.size() > 1 ? 1 : 0];
+    d.groups = (int)groups, d.activation_type = 0, d.activation_param0 = 0.f, d.out_kind = OTTER_HIP_OUT_I32;
+    d.out_round_mode = d.in_round_mode = OTTER_HIP_ROUND_SSE;
+    std::vector<float> ones((size_t)K, 1.f);
+    otter_hip_conv* h = nullptr;
+    hip_check(otter_hip_conv_create(&d, weight.data_ptr<int8_t>(), ones.data(), nullptr, 1.f, nullptr, 0, &h), "convolution");
+    int layout = packed ? otter_hip_conv_default_out_layout(h) : OTTER_HIP_I32;
+    int oh = 0, ow = 0;
+    const int N = (int)input.size(0), H = (int)input.size(2), W = (int)input.size(3);
+    int rc = otter_hip_conv_output_shape(h, H, W, &oh, &ow);
+    Tensor out;
+    if (!rc) {
+        const ScalarType odt = scalar_type_of_layout(layout);
+        out = Tensor::empty_device({N, K / elempack_of(odt), oh, ow}, odt);
+        rc = otter_hip_conv_forward(h, input.device_ptr(), hip_layout_of(input.scalar_type()), N, H, W, out.device_ptr(),
+                                    layout, nullptr, 0, nullptr);
+        if (!rc) out.mark_device_written();
+    }
+    otter_hip_conv_destroy(h);
+    hip_check(rc, "convolution");
+    return out;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// glue layers
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+class InputLayer : public Layer {
+public:
+    InputLayer() { one_blob_only = true; }
+    int parse_param(LayerOption& o, ParamDict& pd) override {  // Tensor/InputLayer.cpp:21-25
+        pd.set(0, opt_find_int(o, "batchsize", 1));
+        pd.set(1, opt_find_int(o, "channel", 1));
+        pd.set(2, opt_find_int(o, "height", 1));
+        pd.set(3, opt_find_int(o, "width", 1));
+        return 0;
+    }
+    int compute_output_shape(ParamDict& pd) override {
+        top_shapes = {{pd.get(0, 1), pd.get(1, 1), pd.get(2, 1), pd.get(3, 1)}};
+        return 0;
+    }
+    std::string type() const override { return "Input"; }
+};
+
+class ActivationLayer : public Layer {
+public:
+    explicit ActivationLayer(int act, const char* name) : act_(act), name_(name) {
+        one_blob_only = true;
+        support_inplace = true;
+        support_packing = true;
+    }
+    int parse_param(LayerOption& o, ParamDict& pd) override {
+        pd.set(0, opt_find_float(o, "alpha", 0.1f));
+        return 0;
+    }
+    int load_param(const ParamDict& pd) override {
+        slope_ = pd.get(0, 0.1f);
+        return 0;
+    }
+    // writes a fresh blob: the input may be shared with another consumer through a Split layer
+    int forward_inplace(Tensor& t, const NetOption&) const override {
+        if (!t.defined() || base_of(t.scalar_type()) != ScalarType::Float || t.dim() != 4) return -1;
+        Tensor out = Tensor::empty_device(t.sizes(), t.scalar_type());
+        const int l = hip_layout_of(t.scalar_type());
+        if (otter_hip_repack(t.device_ptr(), l, (int)t.size(0), (int)t.channels(), (int)t.size(2), (int)t.size(3),
+                             out.device_ptr(), l, nullptr))
+            return -1;
+        if (otter_hip_activation((float*)out.device_ptr(), (size_t)out.numel() * out.elempack(), act_, slope_, nullptr))
+            return -1;
+        out.mark_device_written();
+        t = out;
+        return 0;
+    }
+    std::string type() const override { return name_; }
+
+private:
+    int act_;
+    float slope_ = 0.1f;
+    const char* name_;
+};
+
+class EltwiseLayer : public Layer {  // Tensor/EltwiseLayer.cpp: operation "Sum"
+public:
+    EltwiseLayer() { support_packing = true; }
+    int parse_param(LayerOption& o, ParamDict&) override {
+        return opt_find_string(o, "eltwise_type", "Sum") == "Sum" ? 0 : -1;
+    }
+    int compute_output_shape(ParamDict&) override {
+        top_shapes = {bottom_shapes[0]};
+        return 0;
+    }
+    int forward(const std::vector<Tensor>& b, std::vector<Tensor>& tops, const NetOption&) const override {
+        if (b.size() < 2) return -1;
+        Tensor acc = b[0];
+        for (size_t i = 1; i < b.size(); ++i) {
+            if (base_of(b[i].scalar_type()) != ScalarType::Float || b[i].channels() != acc.channels()) return -1;
+            Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
+            Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
+            if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
+                                      (size_t)acc.numel() * acc.elempack(), nullptr))
+                return -1;
+            out.mark_device_written();
+            acc = out;
+        }
+        tops.assign(1, acc);
+        return 0;
+    }
+    std::string type() const override { return "Eltwise"; }
+};
+
+class SplitLayer : public Layer {  // Tensor/SplitLayer.cpp: every top shares the bottom blob
+public:
+    int compute_output_shape(ParamDict&) override {
+        top_shapes.assign(tops.size(), bottom_shapes[0]);
+        return 0;
+    }
+    int forward(const std::vector<Tensor>& b, std::vector<Tensor>& t, const NetOption&) const override {
+        t.assign(tops.size(), b[0]);
+        return 0;
+    }
+    std::string type() const override { return "Split"; }
+};
+
+class GlobalAvgPoolLayer : public Layer {
+public:
+    GlobalAvgPoolLayer() {
+        one_blob_only = true;
+        support_packing = true;
+    }
+    int compute_output_shape(ParamDict&) override {
+        top_shapes = {{bottom_shapes[0][0], bottom_shapes[0][1], 1, 1}};
+        return 0;
+    }
+    int forward(const Tensor& b, Tensor& top, const NetOption&) const override {
+        if (base_of(b.scalar_type()) != ScalarType::Float || b.dim() != 4) return -1;
+        top = Tensor::empty_device({b.size(0), b.channels(), 1, 1}, ScalarType::Float);
+        if (otter_hip_global_avgpool((const float*)b.device_ptr(), hip_layout_of(b.scalar_type()), (int)b.size(0),
+                                     (int)b.channels(), (int)b.size(2), (int)b.size(3), (float*)top.device_ptr(), nullptr))
+            return -1;
+        top.mark_device_written();
+        return 0;
+    }
+    std::string type() const override { return "GlobalAvgPool"; }
+};
+
+}  // namespace
+
+// Tensor/InnerProductLayer.cpp (fp32 only in the reference as well)
+InnerProductLayer::InnerProductLayer() { one_blob_only = true; }
+int InnerProductLayer::parse_param(LayerOption& o, ParamDict& pd) {
+    pd.set(0, opt_find_int(o, "out_features", 0));
+    int bias = 1;
+    if (opt_find(o, "bias_term")) bias = o["bias_term"] == "false" ? 0 : 1;
+    pd.set(1, bias);
+    return 0;
+}
+int InnerProductLayer::compute_output_shape(ParamDict& pd) {
+    const auto& in = bottom_shapes[0];
+    in_features = (int)(in[1] * in[2] * in[3]);
+    pd.set(2, in_features);
+    top_shapes = {{in[0], pd.get(0, 0), 1, 1}};
+    return 0;
+}
+int InnerProductLayer::load_param(const ParamDict& pd) {
+    out_features = pd.get(0, 0);
+    bias_term = pd.get(1, 1);
+    in_features = pd.get(2, in_features);
+    return 0;
+}
+int InnerProductLayer::init_model() {
+    std::mt19937 rng(99u + (unsigned)out_features);
+    std::normal_distribution<float> nd(0.f, std::sqrt(2.f / (float)in_features));
+    weight_data = Tensor::empty({out_features, in_features}, ScalarType::Float);
+    for (int64_t i = 0; i < weight_data.numel(); ++i) weight_data.data_ptr<float>()[i] = nd(rng);
+    if (bias_term) {
+        bias_data = Tensor::empty({out_features}, ScalarType::Float);
+        for (int i = 0; i < out_features; ++i) bias_data.data_ptr<float>()[i] = 0.01f * nd(rng);
+    }
+    return 0;
+}
+int InnerProductLayer::load_model(const Initializer& in) {
+    weight_data = in.load({out_features, in_features}, 0);
+    if (bias_term) bias_data = in.load({out_features}, 1);
+    return 0;
+}
+int InnerProductLayer::forward(const Tensor& b, Tensor& top, const NetOption&) const {
+    if (!weight_data.defined() || b.scalar_type() != ScalarType::Float) return -1;
+    const int N = (int)b.size(0);
+    if (b.numel() != (int64_t)N * in_features) return -1;
+    top = Tensor::empty_device({N, out_features, 1, 1}, ScalarType::Float);
+    if (otter_hip_inner_product((const float*)b.device_ptr(), N, in_features, (const float*)weight_data.device_ptr(),
+                                bias_term ? (const float*)bias_data.device_ptr() : nullptr, out_features,
+                                (float*)top.device_ptr(), nullptr))
+        return -1;
+    top.mark_device_written();
+    return 0;
+}
+
+void register_hip_layers() {
+    LayerRegistry::AddCreator("Input", []() -> Layer* { return new InputLayer(); });
+    LayerRegistry::AddCreator("Convolution", []() -> Layer* { return new ConvolutionLayer(); });
+    LayerRegistry::AddCreator("Relu", []() -> Layer* { return new ActivationLayer(1, "Relu"); });
+    LayerRegistry::AddCreator("LRelu", []() -> Layer* { return new ActivationLayer(2, "LRelu"); });
+    LayerRegistry::AddCreator("Relu6", []() -> Layer* { return new ActivationLayer(3, "Relu6"); });
+    LayerRegistry::AddCreator("Eltwise", []() -> Layer* { return new EltwiseLayer(); });
+    LayerRegistry::AddCreator("Split", []() -> Layer* { return new SplitLayer(); });
+    LayerRegistry::AddCreator("InnerProduct", []() -> Layer* { return new InnerProductLayer(); });
+    LayerRegistry::AddCreator("GlobalAvgPool", []() -> Layer* { return new GlobalAvgPoolLayer(); });
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Net / Extractor
+// ---------------------------------------------------------------------------------------------------
+Net::Net() {
+    static bool once = (register_hip_layers(), true);
+    (void)once;
+}
+
+Net::~Net() {
+    for (Layer* l : layers_) delete l;
+}
+
+// Tensor/Net.cpp:40-80 (the automatic batch-norm / activation companions do not apply to int8 layers)
+void Net::addLayer(LayerOption option) {
+    if (!opt_find(option, "name")) option["name"] = std::to_string(layer_options_.size());
+    if (!opt_find(option, "output")) option["output"] = option["name"];
+    layer_options_.push_back(option);
+}
+
+// Tensor/Net.cpp:82-172: default input = previous layer's first output; a blob with several consumers gets an
+// automatic Split layer
+void Net::graph_construct() {
+    for (size_t i = 0; i < layer_options_.size(); ++i) {
+        LayerOption& l = layer_options_[i];
+        if (i > 0 && !opt_find(l, "input") && l["type"] != "Input")
+            l["input"] = split_list(layer_options_[i - 1]["output"])[0];
+    }
+    // consumers per blob name
+    for (size_t i = 0; i < layer_options_.size(); ++i) {
+        std::map<std::string, std::vector<size_t>> users;
+        const auto outs = split_list(layer_options_[i]["output"]);
+        for (size_t j = 0; j < layer_options_.size(); ++j) {
+            if (layer_options_[j]["type"] == "Input") continue;
+            for (const auto& in : split_list(layer_options_[j]["input"]))
+                for (const auto& o : outs)
+                    if (in == o) users[o].push_back(j);
+        }
+        size_t inserted = 0;
+        for (auto& kv : users) {
+            if (kv.second.size() < 2) continue;
+            LayerOption sp;
+            sp["type"] = "Split";
+            sp["name"] = "auto_sp_" + std::to_string(i) + "_" + kv.first;
+            sp["input"] = kv.first;
+            std::string outs_s;
+            for (size_t k = 0; k < kv.second.size(); ++k) {
+                const std::string nn = "asp_" + kv.first + "_" + std::to_string(k);
+                outs_s += (k ? "," : "") + nn;
+                // rewrite that consumer's input list (a consumer using the blob twice gets two split outputs)
+                size_t idx = kv.second[k] + (kv.second[k] > i ? inserted : 0);
+                auto ins = split_list(layer_options_[idx]["input"]);
+                for (auto& s : ins)
+                    if (s == kv.first) {
+                        s = nn;
+                        break;
+                    }
+                std::string joined;
+                for (size_t q = 0; q < ins.size(); ++q) joined += (q ? "," : "") + ins[q];
+                layer_options_[idx]["input"] = joined;
+            }
+            sp["output"] = outs_s;
+            layer_options_.insert(layer_options_.begin() + i + 1 + inserted, sp);
+            ++inserted;
+        }
+        i += inserted;
+    }
+}
+
+void Net::compile(CompileMode mode) {
+    graph_construct();
+    std::map<std::string, int> blob_index;
+    for (auto& lo : layer_options_) {
+        Layer* layer = LayerRegistry::CreateLayer(lo["type"]);
+        OTTER_CHECK(layer != nullptr, "Unknown layer type: " + lo["type"]);
+        layer->name = lo["name"];
+        const int li = (int)layers_.size();
+        if (lo["type"] != "Input")
+            for (const auto& in : split_list(lo["input"])) {
+                auto it = blob_index.find(in);
+                OTTER_CHECK(it != blob_index.end(), "layer " + layer->name + ": unknown input blob " + in);
+                layer->bottoms.push_back(it->second);
+                blobs_[it->second].consumers.push_back(li);
+                const Layer* prod = layers_[blobs_[it->second].producer];
+                size_t k = 0;
+                while (prod->tops[k] != it->second) ++k;
+                layer->bottom_shapes.push_back(prod->top_shapes[k]);
+            }
+        for (const auto& out : split_list(lo["output"])) {
+            Blob b;
+            b.name = out;
+            b.producer = li;
+            blob_index[out] = (int)blobs_.size();
+            layer->tops.push_back((int)blobs_.size());
+            blobs_.push_back(b);
+        }
+        ParamDict pd;
+        OTTER_CHECK(layer->parse_param(lo, pd) == 0, "layer " + layer->name + ": parse_param failed");
+        OTTER_CHECK(layer->compute_output_shape(pd) == 0, "layer " + layer->name + ": compute_output_shape failed");
+        OTTER_CHECK(layer->load_param(pd) == 0, "layer " + layer->name + ": load_param failed");
+        if (mode == CompileMode::Initial) {
+            layer->init_model();
+            layer->create_pipeline(option);
+        }
+        layers_.push_back(layer);
+    }
+}
+
+// Tensor/Net.cpp:538-611: every layer reads its tensors from the stream in order, then builds its pipeline
+int Net::load_weight(const Initializer& initializer) {
+    for (Layer* l : layers_) {
+        int rc = l->load_model(initializer);
+        if (rc) return rc;
+        rc = l->create_pipeline(option);
+        if (rc && l->type() == "Convolution") return rc;
+    }
+    return 0;
+}
+
+int Net::find_blob_index_by_name(const std::string& name) const {
+    for (size_t i = 0; i < blobs_.size(); ++i)
+        if (blobs_[i].name == name) return (int)i;
+    return -1;
+}
+
+Layer* Net::layer_by_name(const std::string& name) const {
+    for (Layer* l : layers_)
+        if (l->name == name) return l;
+    return nullptr;
+}
+
+// Tensor/Net.cpp:350-505: lazy, recursive, memoised in the extractor's blob table
+int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt) const {
+    const Layer* layer = layers_[li];
+    for (int b : layer->bottoms)
+        if (!blobs[b].defined()) {
+            int rc = forward_layer(blobs_[b].producer, blobs, opt);
+            if (rc) return rc;
+        }
+    if (layer->type() == "Input") return blobs[layer->tops[0]].defined() ? 0 : -1;
+    if (layer->one_blob_only) {
+        Tensor bottom = blobs[layer->bottoms[0]];
+        Tensor top;
+        int rc;
+        if (layer->support_inplace) {
+            // an in-place layer may only overwrite its input when nobody else reads that blob
+            top = bottom;
+            rc = layer->forward_inplace(top, opt);
+        } else {
+            rc = layer->forward(bottom, top, opt);
+        }
+        if (rc) return rc;
+        blobs[layer->tops[0]] = top;
+    } else {
+        std::vector<Tensor> bottoms, tops;
+        for (int b : layer->bottoms) bottoms.push_back(blobs[b]);
+        int rc = layer->forward(bottoms, tops, opt);
+        if (rc) return rc;
+        for (size_t k = 0; k < layer->tops.size(); ++k) blobs[layer->tops[k]] = tops[k];
+    }
+    if (opt.lightmode)  // Tensor/Net.cpp:449-451: the inputs are not needed any more
+        for (int b : layer->bottoms)
+            if (blobs_[b].consumers.size() == 1) blobs[b] = Tensor();
+    return 0;
+}
+
+Extractor Net::create_extractor() const { return Extractor(this, blobs_.size()); }
+
+Extractor::Extractor(const Net* net, size_t blob_count) : option(net->option), net_(net), blob_tensors_(blob_count) {}
+
+void Extractor::clear() { blob_tensors_.assign(blob_tensors_.size(), Tensor()); }
+
+int Extractor::input(const std::string& name, const Tensor& in) {
+    const int i = net_->find_blob_index_by_name(name);
+    if (i < 0) return -1;
+    blob_tensors_[i] = in;
+    return 0;
+}
+
+int Extractor::extract(const std::string& name, Tensor& feat, int type) {
+    const int i = net_->find_blob_index_by_name(name);
+    if (i < 0) return -1;
+    int ret = 0;
+    if (!blob_tensors_[i].defined()) ret = net_->forward_layer(net_->blobs_[i].producer, blob_tensors_, option);
+    if (ret) return ret;
+    feat = blob_tensors_[i];
+    if (option.use_packing_layout && type == 0 && feat.dim() == 4 && feat.elempack() != 1) feat = feat.packing(1);
+    return 0;
+}
+
+}  // namespace otter

@@ -1,0 +1,283 @@
+// Host side of the MI355X int8 convolution path: the part of Otter's C++ interface that the path lives behind
+// (Tensor handle with the packed dtypes, NetOption, ParamDict, Layer, LayerRegistry, ConvolutionLayer, the
+// functional quantize / convolution entry points, Net / Extractor), re-implemented over the C ABI in
+// include/otter_hip_int8.h. Names, option keys, argument meaning and int return codes are the reference's, so that
+// code written against Otter's Layer / Net API drives the GPU path unchanged; everything outside the int8
+// convolution path (fp32 convolutions, detection heads, image I/O ...) is not here.
+//
+// Activations may live on the host, on the device, or both: a Tensor produced by a GPU layer stays on the device
+// until somebody asks for its host pointer, so consecutive layers of a Net chain without host round trips.
+#pragma once
+
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+struct otter_hip_conv;
+
+namespace otter {
+
+// Tensor/Exception.hpp:88-91
+struct Error : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+#define OTTER_CHECK(cond, msg)                     \
+    do {                                           \
+        if (!(cond)) throw ::otter::Error(msg);    \
+    } while (0)
+
+// the dtypes of the int8 path (Tensor/ScalarType.hpp:45-74): element type x elempack
+enum class ScalarType { Undefined, Float, Float4, Float8, Byte, Byte8, Int, Int4, Int8 };
+
+int elempack_of(ScalarType t);
+size_t elemsize_of(ScalarType t);          // bytes of one packed element
+ScalarType scalar_type_of(ScalarType base, int elempack);  // get_update_scalarType
+ScalarType base_of(ScalarType t);          // Float / Byte / Int
+int hip_layout_of(ScalarType t);           // otter_hip_layout
+
+class Tensor {
+public:
+    Tensor() = default;
+    static Tensor empty(const std::vector<int64_t>& sizes, ScalarType dtype);        // host storage
+    static Tensor empty_device(const std::vector<int64_t>& sizes, ScalarType dtype); // device storage only
+    static Tensor from_blob(const void* data, const std::vector<int64_t>& sizes, ScalarType dtype);  // copies
+
+    bool defined() const { return (bool)st_; }
+    int64_t dim() const { return (int64_t)sizes_.size(); }
+    int64_t size(int i) const { return sizes_[i]; }
+    const std::vector<int64_t>& sizes() const { return sizes_; }
+    ScalarType scalar_type() const { return dtype_; }
+    int elempack() const { return elempack_of(dtype_); }
+    int64_t numel() const;          // packed elements
+    size_t nbytes() const { return (size_t)numel() * elemsize_of(dtype_); }
+    int64_t channels() const { return dim() == 4 ? sizes_[1] * elempack() : 0; }  // logical C
+
+    // Tensor::packing (Tensor/Tensor.cpp:29-35): [N,C/p,H,W] with elempack p -> elempack `p`
+    Tensor packing(int p) const;
+    Tensor view(const std::vector<int64_t>& sizes) const;
+
+    void* data_ptr();               // host pointer; downloads first if the fresh copy is on the device
+    const void* data_ptr() const;
+    template <typename T>
+    T* data_ptr() { return static_cast<T*>(data_ptr()); }
+    template <typename T>
+    const T* data_ptr() const { return static_cast<const T*>(data_ptr()); }
+
+    void* device_ptr() const;       // device pointer; uploads first if the fresh copy is on the host
+    bool on_device() const;         // a valid device copy exists
+    void mark_device_written();     // the device copy is now the fresh one
+
+private:
+    struct Storage;
+    std::shared_ptr<Storage> st_;
+    std::vector<int64_t> sizes_;
+    ScalarType dtype_ = ScalarType::Undefined;
+};
+
+// Tensor/NetOption.hpp
+class NetOption {
+public:
+    bool lightmode = true;
+    bool train = false;
+    bool use_non_lib_optimize = true;
+    bool use_packing_layout = true;
+    bool use_fp16_storage = true;
+    int openmp_blocktime = 20;
+};
+enum class CompileMode { Inference, Initial };
+
+// Tensor/ParamDict.hpp
+class ParamDict {
+public:
+    int get(int id, int def) const;
+    float get(int id, float def) const;
+    Tensor get(int id, const Tensor& def) const;
+    void set(int id, int i);
+    void set(int id, float f);
+    void set(int id, const Tensor& t);
+    void clear();
+
+private:
+    struct Entry {
+        int type = 0;
+        int i = 0;
+        float f = 0;
+        Tensor t;
+    };
+    std::map<int, Entry> params_;
+};
+
+using LayerOption = std::unordered_map<std::string, std::string>;
+#define OUTPUT_SHAPE_HINT 30
+bool opt_find(const LayerOption& o, const std::string& k);
+int opt_find_int(const LayerOption& o, const std::string& k, int def);
+float opt_find_float(const LayerOption& o, const std::string& k, float def);
+std::string opt_find_string(const LayerOption& o, const std::string& k, const std::string& def);
+
+// Weight source of load_model (Tensor/Initializer.hpp): hands out consecutive tensors of a weight stream.
+// type 0 = weight (may be int8), 1 = fp32 vector.
+class Initializer {
+public:
+    virtual ~Initializer() = default;
+    virtual Tensor load(const std::vector<int64_t>& shape, int type) const = 0;
+};
+
+// Tensor/Layer.hpp:23-62
+class Layer {
+public:
+    Layer() = default;
+    virtual ~Layer() = default;
+    virtual int parse_param(LayerOption& option, ParamDict& pd);
+    virtual int compute_output_shape(ParamDict& pd);
+    virtual int load_param(const ParamDict& pd);
+    virtual int init_model();
+    virtual int load_model(const Initializer& initializer);
+    virtual int create_pipeline(const NetOption& opt);
+    virtual std::string type() const { return "Undefined"; }
+
+    // 0 success; -1 not supported; -100 allocation failure (Tensor/Layer.cpp:50-59)
+    virtual int forward(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const;
+    virtual int forward(const std::vector<Tensor>& bottom_blobs, std::vector<Tensor>& top_blobs,
+                        const NetOption& opt) const;
+    virtual int forward_inplace(Tensor& bottom_blob, const NetOption& opt) const;
+
+    bool support_inplace = false;
+    bool one_blob_only = false;
+    bool support_packing = false;
+    std::vector<int> bottoms, tops;
+    std::vector<std::vector<int64_t>> bottom_shapes, top_shapes;  // logical [N,C,H,W]
+    std::string name;
+};
+
+// Tensor/LayerRegistry.hpp:17-85: string-keyed factory; a later AddCreator overrides an earlier one
+class LayerRegistry {
+public:
+    typedef Layer* (*Creator)();
+    static void AddCreator(const std::string& type, Creator creator);
+    static Layer* CreateLayer(const std::string& type);   // nullptr for an unknown type
+    static std::vector<std::string> TypeList();
+};
+// registers the GPU layers of this library under the reference's type strings
+// ("Input", "Convolution", "Relu", "Relu6", "LRelu", "Eltwise", "Split", "InnerProduct", "GlobalAvgPool")
+void register_hip_layers();
+
+// Tensor/ConvolutionLayer.hpp:15-99 -- same public members, same option keys; int8 path on the GPU
+enum class ConvParam : int {
+    In_channels, Out_channels, Kernel_height, Kernel_width, Stride_height, Stride_width, Padding_height, Padding_width,
+    Dilation_height, Dilation_width, Output_padding_height, Output_padding_width, Group, Bias_term, Weight_data_size,
+    Int8_scale_term, Activation_type, Activation_params
+};
+
+class ConvolutionLayer : public Layer {
+public:
+    ConvolutionLayer();
+    ~ConvolutionLayer() override;
+    int parse_param(LayerOption& option, ParamDict& pd) override;
+    int compute_output_shape(ParamDict& pd) override;
+    int load_param(const ParamDict& pd) override;
+    int init_model() override;
+    int load_model(const Initializer& initializer) override;
+    int create_pipeline(const NetOption& opt) override;
+    int forward(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const override;
+    std::string type() const override { return "Convolution"; }
+
+    int in_channels = 1, out_channels = 1, kernel_height = 3, kernel_width = 3, stride_height = 1, stride_width = 1;
+    int padding_height = 0, padding_width = 0, dilation_height = 1, dilation_width = 1;
+    int output_padding_height = 0, output_padding_width = 0, groups = 1, bias_term = 0, int8_scale_term = 0;
+    int weight_data_size = 0, activation_type = 0;
+    Tensor activation_params;
+    Tensor weight_data, bias_data;
+    Tensor weight_data_int8_scales, bottom_blob_int8_scales, top_blob_int8_scales, scale_in_data;
+    // when set, forward() produces fp32 even if int8_scale_term > 100 is absent etc.; -1 = the reference's rule
+    int force_out_layout = -1;
+
+private:
+    int create_pipeline_int8(const NetOption& opt);
+    int forward_int8(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const;
+    otter_hip_conv* handle_ = nullptr;
+};
+
+// Tensor/InnerProductLayer.hpp (fp32; the reference has no int8 inner product either)
+class InnerProductLayer : public Layer {
+public:
+    InnerProductLayer();
+    int parse_param(LayerOption& option, ParamDict& pd) override;
+    int compute_output_shape(ParamDict& pd) override;
+    int load_param(const ParamDict& pd) override;
+    int init_model() override;
+    int load_model(const Initializer& initializer) override;
+    int forward(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const override;
+    std::string type() const override { return "InnerProduct"; }
+    int in_features = 0, out_features = 0, bias_term = 1;
+    Tensor weight_data, bias_data;
+};
+
+// returns every cached device blob to the driver
+void device_cache_clear();
+
+// Functional entry points (Tensor/Quantize.hpp:15-19, Tensor/Convolution.hpp:17-30), int8 path only.
+Tensor quantize_to_int8(const Tensor& src, const Tensor& scale_data, bool pack = false);
+Tensor dequantize_from_int32(const Tensor& src, const Tensor& scale_data, const Tensor& bias_data, bool pack = false);
+Tensor requantize_from_int32_to_int8(const Tensor& src, const Tensor& scale_in_data, const Tensor& scale_out_data,
+                                     const Tensor& bias_data, int activation_type, const Tensor& activation_params,
+                                     bool pack = false);
+// int8 input + int8 weight [K, C/g, kh, kw] -> int32 accumulators (Int4 when packed and K % 4 == 0, Int8-packed for
+// depthwise with C % 8 == 0, else Int)
+Tensor convolution(const Tensor& input, const Tensor& weight, const Tensor& weight_o, const Tensor& bias,
+                   const std::vector<int>& stride, const std::vector<int>& padding, const std::vector<int>& dilation,
+                   bool transposed, const std::vector<int>& output_padding, int64_t groups, bool packed = true,
+                   const Tensor& input_int8_scales = Tensor(), const Tensor& weight_int8_scales = Tensor());
+
+// Tensor/Net.hpp:22-114 (subset: graph build, lazy forward, extractor)
+class Extractor;
+class Net {
+    friend class Extractor;
+
+public:
+    Net();
+    ~Net();
+    void addLayer(LayerOption option);
+    void compile(CompileMode mode = CompileMode::Initial);
+    int load_weight(const Initializer& initializer);
+    Extractor create_extractor() const;
+    int find_blob_index_by_name(const std::string& name) const;
+    Layer* layer_by_name(const std::string& name) const;
+    size_t layer_count() const { return layers_.size(); }
+    NetOption option;
+
+private:
+    void graph_construct();
+    int forward_layer(int layer_index, std::vector<Tensor>& blobs, const NetOption& opt) const;
+    struct Blob {
+        std::string name;
+        int producer = -1;
+        std::vector<int> consumers;
+    };
+    std::vector<Layer*> layers_;
+    std::vector<Blob> blobs_;
+    std::vector<LayerOption> layer_options_;
+};
+
+class Extractor {
+    friend class Net;
+
+public:
+    void clear();
+    void set_lightmode(bool lightmode) { option.lightmode = lightmode; }
+    int input(const std::string& blob_name, const Tensor& in);
+    // type 0: unpacked (elempack 1) host-visible result, as the reference; type 1: whatever layout the layer left
+    int extract(const std::string& blob_name, Tensor& feat, int type);
+    NetOption option;
+
+private:
+    Extractor(const Net* net, size_t blob_count);
+    const Net* net_;
+    std::vector<Tensor> blob_tensors_;
+};
+
+}  // namespace otter

@@ -1,0 +1,126 @@
+"""The C++ host layer (tensor_amd/host): Otter's ConvolutionLayer / Net interface driving the GPU path.
+CPU: the library loads and exports its facade. GPU: networks built with the reference's option keys reproduce the
+oracle's layer-by-layer result bit for bit (int8) / within 1e-5 (fp32)."""
+import numpy as np
+import pytest
+
+from tensor_amd import hostnet
+
+
+def test_host_library_exports():
+    lib = hostnet.load_cdll()
+    for name in hostnet.EXPORTS:
+        assert hasattr(lib, name), name
+
+
+def _qweights(rng, K, Cg, k):
+    wf = rng.normal(0, 0.05, (K, Cg, k, k)).astype(np.float32)
+    ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
+    return np.clip(np.round(wf * ws[:, None, None, None]), -127, 127).astype(np.int8), ws
+
+
+@pytest.mark.gpu
+def test_net_chain_int8_activations_flow_between_layers(oracle):
+    """Input -> 3x3 conv (102, Relu) -> depthwise 3x3 s2 (101, Relu6) -> 1x1 conv (2): the chain the reference runs
+    as Byte8 -> Byte8 -> Float4."""
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, (2, 16, 20, 20)).astype(np.float32)
+    w1, s1 = _qweights(rng, 16, 16, 3)
+    w2, s2 = _qweights(rng, 16, 1, 3)
+    w3, s3 = _qweights(rng, 8, 16, 1)
+    b1, b2, b3 = (rng.normal(0, 0.1, n).astype(np.float32) for n in (16, 16, 8))
+    in1 = np.float32(127) / np.abs(x).max()
+    t1, t2 = np.float32(21.0), np.float32(127.0 / 6.0)
+    net = hostnet.Net()
+    net.add_layer(type="Input", name="data", batchsize=2, channel=16, height=20, width=20)
+    net.add_layer(type="Convolution", name="c1", out_channels=16, kernel=3, padding=1, int8_scale_term=102,
+                  activation="Relu")
+    net.add_layer(type="Convolution", name="c2", out_channels=16, kernel=3, stride=2, padding=1, groups=16,
+                  int8_scale_term=101, activation="Relu6")
+    net.add_layer(type="Convolution", name="c3", out_channels=8, kernel=1, int8_scale_term=2)
+    net.compile()
+    net.set_conv("c1", w1, b1, s1, in1, t1)
+    net.set_conv("c2", w2, b2, s2, t1, t2)
+    net.set_conv("c3", w3, b3, s3, t2)
+    np.testing.assert_array_equal(net.scale_in("c1", 16).view(np.int32), oracle.scale_in(s1, in1).view(np.int32))
+    y1 = oracle.conv_layer_forward(x, w1, s1, in1, pad=(1, 1), bias=b1, top_scale=t1, int8_out=True, act_type=1)
+    y2 = oracle.conv_layer_forward(y1, w2, s2, t1, stride=(2, 2), pad=(1, 1), groups=16, bias=b2, top_scale=t2,
+                                   int8_out=True, act_type=3)
+    y3 = oracle.conv_layer_forward(y2, w3, s3, t2, bias=b3)
+    np.testing.assert_array_equal(net.run("data", x, "c1"), y1)
+    np.testing.assert_array_equal(net.run("data", x, "c2"), y2)
+    np.testing.assert_allclose(net.run("data", x, "c3"), y3, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.gpu
+def test_net_residual_block_with_auto_split(oracle):
+    """A MobileNetV2-style inverted residual: the block input feeds the expand conv AND the element-wise add, so the
+    graph builder must insert a Split; the project conv feeds the add, so it stays fp32."""
+    rng = np.random.default_rng(6)
+    C, E = 16, 96
+    x = rng.uniform(0, 1, (2, C, 14, 14)).astype(np.float32)
+    we, se = _qweights(rng, E, C, 1)
+    wd, sd = _qweights(rng, E, 1, 3)
+    wp, sp = _qweights(rng, C, E, 1)
+    be, bd, bp = (rng.normal(0, 0.1, n).astype(np.float32) for n in (E, E, C))
+    in_e = np.float32(127) / np.abs(x).max()
+    te = td = np.float32(127.0 / 6.0)
+    net = hostnet.Net()
+    net.add_layer(type="Input", name="data", batchsize=2, channel=C, height=14, width=14)
+    net.add_layer(type="Convolution", name="expand", input="data", out_channels=E, kernel=1, int8_scale_term=102,
+                  activation="Relu6")
+    net.add_layer(type="Convolution", name="dw", out_channels=E, kernel=3, padding=1, groups=E, int8_scale_term=101,
+                  activation="Relu6")
+    net.add_layer(type="Convolution", name="project", out_channels=C, kernel=1, int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="add", input="data,project")
+    net.add_layer(type="GlobalAvgPool", name="pool")
+    net.add_layer(type="InnerProduct", name="fc", out_features=10)
+    net.compile()
+    net.set_conv("expand", we, be, se, in_e, te)
+    net.set_conv("dw", wd, bd, sd, te, td)
+    net.set_conv("project", wp, bp, sp, td)
+    wfc = rng.normal(0, 0.1, (10, C)).astype(np.float32)
+    bfc = rng.normal(0, 0.1, 10).astype(np.float32)
+    net.set_inner_product("fc", wfc, bfc)
+    y = oracle.conv_layer_forward(x, we, se, in_e, bias=be, top_scale=te, int8_out=True, act_type=3)
+    y = oracle.conv_layer_forward(y, wd, sd, te, pad=(1, 1), groups=E, bias=bd, top_scale=td, int8_out=True, act_type=3)
+    y = oracle.conv_layer_forward(y, wp, sp, td, bias=bp)
+    s = y + x
+    np.testing.assert_allclose(net.run("data", x, "add"), s, rtol=1e-5, atol=1e-30)
+    want = oracle.inner_product(oracle.global_avgpool(s), wfc, bfc)
+    got = net.run("data", x, "fc").reshape(2, 10)
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_functional_api_matches_oracle(oracle):
+    rng = np.random.default_rng(8)
+    for (C, K, k, s, p, g, i8) in [(16, 16, 3, 1, 1, 1, True), (32, 32, 3, 2, 1, 32, True), (8, 12, 1, 1, 0, 1, False)]:
+        x = rng.uniform(-1, 1, (2, C, 11, 9)).astype(np.float32)
+        wq, ws = _qweights(rng, K, C // g, k)
+        bias = rng.normal(0, 0.2, K).astype(np.float32)
+        in_scale = np.float32(127) / np.abs(x).max()
+        want, acc_want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), groups=g, bias=bias,
+                                                   top_scale=13.0, int8_out=i8, act_type=1 if i8 else 0, want_acc=True)
+        acc, out = hostnet.functional_chain(x, in_scale, wq, oracle.scale_in(ws, in_scale), bias, stride=s, pad=p,
+                                            groups=g, int8_out=i8, top_scale=13.0, act=1 if i8 else 0)
+        np.testing.assert_array_equal(acc, acc_want)
+        if i8:
+            np.testing.assert_array_equal(out, want)
+        else:
+            np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.gpu
+def test_error_conventions():
+    net = hostnet.Net()
+    net.add_layer(type="Input", name="data", batchsize=1, channel=8, height=4, width=4)
+    net.add_layer(type="NoSuchLayer", name="bad")
+    with pytest.raises(hostnet.HostError):
+        net.compile()
+    net2 = hostnet.Net()
+    net2.add_layer(type="Input", name="data", batchsize=1, channel=8, height=4, width=4)
+    net2.add_layer(type="Convolution", name="c", out_channels=8, kernel=3, padding=1, int8_scale_term=2)
+    net2.compile()
+    with pytest.raises(hostnet.HostError):  # pipeline never built: forward returns the reference's -1
+        net2.run("data", np.zeros((1, 8, 4, 4), np.float32), "c")

@@ -1,0 +1,37 @@
+"""MobileNetV2-style int8 network through the C++ host layer against the CPU oracle, at reduced resolution."""
+import numpy as np
+import pytest
+
+from tensor_amd import capi, hostnet, mobilenet
+
+
+def test_description_matches_the_configuration():
+    layers = mobilenet.describe()
+    convs = [l for l in layers if l["kind"] == "conv"]
+    assert len(convs) == 52 and sum(l["kind"] == "add" for l in layers) == 10
+    # 299.49 MMAC of convolution + 1.28 MMAC inner product per 224x224 image
+    assert abs(mobilenet.conv_macs_per_image(layers, 224) - 300.77e6) < 0.05e6
+    # a convolution writes int8 exactly when no element-wise add (or the pooling) consumes its output
+    feeds_add = {l["a"] for l in layers if l["kind"] == "add"} | {l["b"] for l in layers if l["kind"] == "add"}
+    for l in convs:
+        assert l["int8_out"] == (l["name"] not in feeds_add and l["name"] != "head")
+
+
+@pytest.mark.gpu
+def test_network_matches_oracle_layer_by_layer(hip, oracle):
+    rng = np.random.default_rng(0)
+    hw, batch = 64, 2
+    layers = mobilenet.describe(num_classes=50)
+    params = mobilenet.init_weights(layers, rng)
+    mobilenet.calibrate(hip, capi, layers, params, rng.uniform(0, 1, (4, 3, hw, hw)).astype(np.float32))
+    net = mobilenet.build_net(hostnet, layers, params, batch, hw, num_classes=50)
+    x = rng.uniform(0, 1, (batch, 3, hw, hw)).astype(np.float32)
+    want = mobilenet.oracle_forward(oracle, layers, params, x)
+    for name in ("stem", "b0_project", "b1_dw", "b2_add", "b5_project", "b9_add", "b16_project", "head"):
+        got = net.run("data", x, name)
+        if got.dtype == np.int8:
+            np.testing.assert_array_equal(got, want[name], err_msg=name)
+        else:
+            np.testing.assert_allclose(got, want[name], rtol=1e-5, atol=1e-30, err_msg=name)
+    got = net.run("data", x, "fc").reshape(batch, -1)
+    np.testing.assert_allclose(got, want["fc"], rtol=1e-4, atol=1e-5)

@@ -56,6 +56,7 @@ struct otter_hip_conv {
     float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
     float* scale_out = nullptr;  // [Kpad] or null
     float* in_scale = nullptr;   // [1]
+    int c_pad = 0;               // > 0: C is not a multiple of 8; the MFMA path runs on C zero-padded to c_pad
     int force_tm = 0, force_tn = 0;
 };
 
@@ -189,6 +190,17 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
             igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
             if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
+        } else if (g == 1) {
+            // C % 8 != 0 (e.g. an RGB stem): zero-pad the input channels to the next octet, weights included
+            const int cp = (C + 7) / 8 * 8;
+            std::vector<int8_t> wpad((size_t)K * cp * maxk, 0);
+            for (int k = 0; k < K; ++k)
+                for (int c = 0; c < C; ++c)
+                    std::memcpy(&wpad[((size_t)k * cp + c) * maxk], &weight[((size_t)k * C + c) * maxk], maxk);
+            std::vector<int8_t> wp(igemm_packed_weight_bytes(K, cp, d.kernel_h, d.kernel_w));
+            igemm_pack_weights(wpad.data(), K, cp, d.kernel_h, d.kernel_w, wp.data());
+            if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
+            h->c_pad = cp;
         }
     } while (0);
     if (rc != OTTER_HIP_OK) {
@@ -224,7 +236,9 @@ int otter_hip_conv_default_out_layout(const otter_hip_conv_t* h) {
 }
 
 size_t otter_hip_conv_workspace_bytes(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w) {
-    if (!h || !valid_layout(in_layout) || layout_elem(in_layout) != 0) return 0;
+    if (!h || !valid_layout(in_layout)) return 0;
+    if (h->c_pad) return (size_t)n * h->c_pad * in_h * in_w;  // the zero-padded Byte8 copy, fp32 or int8 input alike
+    if (layout_elem(in_layout) != 0) return 0;
     return (size_t)n * h->d.in_channels * in_h * in_w;
 }
 
@@ -263,7 +277,9 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, 
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
     if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
-    return pick_kernel(h, l, make_geom(h->d, n, in_h, in_w));
+    ConvGeom g = make_geom(h->d, n, in_h, in_w);
+    if (h->c_pad) l = OTTER_HIP_I8_P8, g.C = h->c_pad;
+    return pick_kernel(h, l, g);
 }
 
 int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
@@ -283,7 +299,7 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     if (d.out_channels % layout_pack(out_layout))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: output pack does not divide K");
 
-    const ConvGeom g = make_geom(d, n, in_h, in_w);
+    ConvGeom g = make_geom(d, n, in_h, in_w);
     if (g.OH < 1 || g.OW < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: empty output");
     if ((size_t)n * g.C * in_h * in_w >= (1ull << 31) || (size_t)n * g.K * g.OH * g.OW >= (1ull << 31))
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
@@ -292,7 +308,18 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     // (1) quantize_to_int8 when the blob is not int8 yet (Tensor/ConvolutionLayer.cpp:770-775)
     const int8_t* xq = (const int8_t*)in;
     int q_layout = in_layout;
-    if (layout_elem(in_layout) == 0) {
+    if (h->c_pad) {
+        // (quantize and) zero-pad the channels into a Byte8 copy; the MFMA kernels then see C = c_pad
+        const size_t need = (size_t)n * h->c_pad * in_h * in_w;
+        if (!workspace || workspace_bytes < need)
+            return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: this layer needs the workspace reported by "
+                                               "otter_hip_conv_workspace_bytes");
+        OHIP_CHECK(run_pad_pack8(in, layout_elem(in_layout) == 0, layout_pack(in_layout), (int8_t*)workspace, n, g.C,
+                                 h->c_pad, in_h * in_w, h->in_scale, d.in_round_mode, stream));
+        xq = (const int8_t*)workspace;
+        q_layout = OTTER_HIP_I8_P8;
+        g.C = h->c_pad;
+    } else if (layout_elem(in_layout) == 0) {
         const size_t need = (size_t)n * g.C * in_h * in_w;
         if (!workspace || workspace_bytes < need)
             return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: fp32 input needs a workspace of N*C*H*W bytes");

@@ -32,6 +32,8 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
 // elementwise.hip
 hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,
                         int n_scales, int round_mode, hipStream_t stream);
+hipError_t run_pad_pack8(const void* src, bool src_is_float, int sp, int8_t* dst, int N, int C, int Cp, int HW,
+                         const float* scale, int round_mode, hipStream_t stream);
 hipError_t run_dequantize(const int32_t* src, int sp, float* dst, int dp, int N, int C, int HW, const float* scale,
                           int n_scale, const float* bias, int n_bias, hipStream_t stream);
 hipError_t run_requantize(const int32_t* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scale_in,

@@ -156,6 +156,50 @@ hipError_t dispatch_ew(const TI* src, int sp, TO* dst, int dp, int N, int C, int
     return hipErrorInvalidValue;
 }
 
+// [N, C, HW] in any pack dividing C (fp32, quantized on the way, or int8) -> Byte8 with the channel count padded with
+// zeros to Cp = a multiple of 8: lets a convolution whose C is not a multiple of 8 (an RGB stem) use the MFMA path.
+template <typename T>
+__global__ void __launch_bounds__(256) pad_pack8_kernel(const T* __restrict__ src, int sp, int8_t* __restrict__ dst, int N,
+                                                        int C, int Cp, int HW, const float* __restrict__ scale,
+                                                        int round_mode) {
+    const size_t total = (size_t)N * (Cp / 8) * HW;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int pix = (int)(idx % HW);
+    const size_t r = idx / HW;
+    const int o = (int)(r % (Cp / 8));
+    const int n = (int)(r / (Cp / 8));
+    int q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int c = o * 8 + e;
+        q[e] = 0;
+        if (c < C) {
+            const T v = src[elem_offset(sp, n, c, pix, C, HW)];
+            if constexpr (sizeof(T) == 4) q[e] = float2int8_rt(__fmul_rn((float)v, scale[0]), round_mode);
+            else q[e] = (int)v;
+        }
+    }
+    ohip_v2i pk;
+    pk[0] = (q[0] & 0xff) | ((q[1] & 0xff) << 8) | ((q[2] & 0xff) << 16) | (q[3] << 24);
+    pk[1] = (q[4] & 0xff) | ((q[5] & 0xff) << 8) | ((q[6] & 0xff) << 16) | (q[7] << 24);
+    reinterpret_cast<ohip_v2i*>(dst)[idx] = pk;
+}
+
+hipError_t run_pad_pack8(const void* src, bool src_is_float, int sp, int8_t* dst, int N, int C, int Cp, int HW,
+                         const float* scale, int round_mode, hipStream_t stream) {
+    const size_t total = (size_t)N * (Cp / 8) * HW;
+    if (total == 0) return hipSuccess;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (src_is_float)
+        hipLaunchKernelGGL(pad_pack8_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)src, sp, dst, N, C, Cp,
+                           HW, scale, round_mode);
+    else
+        hipLaunchKernelGGL(pad_pack8_kernel<int8_t>, dim3(blocks), dim3(256), 0, stream, (const int8_t*)src, sp, dst, N, C,
+                           Cp, HW, scale, round_mode);
+    return hipGetLastError();
+}
+
 hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,
                         int n_scales, int round_mode, hipStream_t stream) {
     QuantOp op{scales, n_scales, round_mode};

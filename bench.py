@@ -197,6 +197,17 @@ def build_c0(hip, capi, rng):
                 shape=(N, C, H, W))
 
 
+def build_copy(hip, capi, rng):
+    """Calibration workload for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain device copy of 256 MiB."""
+    torch = hip.torch
+    n = 256 << 20
+    src = torch.zeros(n, dtype=torch.int8, device=hip.device)
+    dst = torch.empty_like(src)
+    return dict(name="copy", step=lambda: dst.copy_(src), ops=0.0, launches=1, bytes=2 * n, dom_ops=0.0, dom_bytes=2 * n,
+                bound="hbm", workload="device-to-device copy of 256 MiB (counter calibration)", dom_kernel="copy",
+                dom_fn=None, x=None, params=[], shape=(n,))
+
+
 # ------------------------------------------------------------------------------------------------------
 # CPU baseline: the reference itself (oracle/_ref, kind "reference") or the C restatement (kind "port")
 # ------------------------------------------------------------------------------------------------------
@@ -258,6 +269,8 @@ def cpu_baseline(wl, budget_s=15.0):
         t = time.perf_counter() - t0
         return dict(value=algo_bytes / t / 1e9, unit="GB/s", cores=O.num_threads(), kind="port",
                     sample="%d images, scalar C restatement" % n_img)
+    if name == "copy":
+        return None
     if name in ("c2", "c0"):
         n_img = min(4, N)
         K = p[0]["wq"].shape[0]
@@ -276,6 +289,16 @@ def cpu_baseline(wl, budget_s=15.0):
     return None
 
 
+def measured_traffic(name):
+    """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 --pmc summary
+    (profiles/hbm_traffic.json: FETCH_SIZE / WRITE_SIZE scaled by a copy-kernel calibration); None if not profiled."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f).get(name, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        return None
+
+
 def measure(wl, timer, steps, warmup, unit_main):
     ms, wall_ms = timer.run(wl["step"], steps, warmup)
     res = dict(workload=wl["workload"], ms_per_step=ms, wall_ms_per_step=wall_ms)
@@ -291,11 +314,11 @@ def measure(wl, timer, steps, warmup, unit_main):
     if wl["bound"] == "mfma":
         ach = wl["dom_ops"] / (kms * 1e-3) / 1e12
         res["roofline"] = dict(bound="mfma", achieved=ach, peak=PEAK_INT8_TOPS, unit="TOP/s", frac=ach / PEAK_INT8_TOPS,
-                               traffic=None, kernel=wl["dom_kernel"], kernel_ms=kms)
+                               traffic=measured_traffic(wl["name"]), kernel=wl["dom_kernel"], kernel_ms=kms)
     else:
         ach = wl["dom_bytes"] / (kms * 1e-3) / 1e9
         res["roofline"] = dict(bound="hbm", achieved=ach, peak=PEAK_HBM_GBS, unit="GB/s", frac=ach / PEAK_HBM_GBS,
-                               traffic=None, kernel=wl["dom_kernel"], kernel_ms=kms)
+                               traffic=measured_traffic(wl["name"]), kernel=wl["dom_kernel"], kernel_ms=kms)
         res["roofline"]["tops"] = wl["dom_ops"] / (kms * 1e-3) / 1e12
     if "aux" in wl:
         ams, _ = timer.run(wl["aux"]["fn"], max(steps * 4, 50), 5)
@@ -326,7 +349,7 @@ def main():
     timer = Timer(hip.torch)
     builders = {"c3": lambda r: build_c3(hip, capi, r), "c1s1": lambda r: build_c1(hip, capi, r, 1),
                 "c1s2": lambda r: build_c1(hip, capi, r, 2), "c2": lambda r: build_c2(hip, capi, r),
-                "c0": lambda r: build_c0(hip, capi, r)}
+                "c0": lambda r: build_c0(hip, capi, r), "copy": lambda r: build_copy(hip, capi, r)}
     try:
         from tensor_amd import mobilenet  # noqa: F401
         builders["c4"] = lambda r: mobilenet.build_bench(hip, capi, r)

@@ -7,6 +7,8 @@
 // strip and reused from registers for the rows below it.
 // The multiply-accumulate uses v_dot4_i32_i8 against a weight word that holds the tap weight in the byte of
 // its channel and zeros elsewhere: one instruction per (tap, channel) with no byte unpacking of the input.
+#include <algorithm>
+
 #include "common.hpp"
 #include "conv_igemm.hpp"
 
@@ -114,24 +116,33 @@ __global__ void __launch_bounds__(256) conv_dw3x3_kernel(const int8_t* __restric
 template <int S, int R, bool NONNEG>
 __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __restrict__ x, const int32_t* __restrict__ wmask,
                                                             int8_t* __restrict__ out, ConvGeom g, Epilogue ep,
-                                                            int n_strips, int col_chunks) {
+                                                            int n_strips, int col_chunks, int ipw) {
     // A wave = 64 consecutive output columns of ONE strip, so "is this input row inside the image" is a scalar
     // branch, not a per-lane exec mask (those masks would crowd the weights out of the scalar registers).
+    // Images narrower than half a wave put `ipw` images side by side in the wave instead (same channel octet, same
+    // strip, consecutive images): the weights and the row test stay wave-uniform and the lanes stay busy.
     const int C8 = g.C / 8;
-    const int plane = blockIdx.y;
-    const int o = plane % C8;
+    const int o = blockIdx.y % C8;
+    const int n0 = (blockIdx.y / C8) * ipw;
     const int chunk = blockIdx.x % col_chunks;
     const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    const int ox = chunk * 64 + (threadIdx.x & 63);
-    if (strip >= n_strips || ox >= g.OW) return;
+    const int lane = threadIdx.x & 63;
+    int di = 0, ox = chunk * 64 + lane;
+    if (ipw > 1) {
+        di = lane / g.OW;
+        ox = lane - di * g.OW;
+    }
+    if (strip >= n_strips || ox >= g.OW || di >= ipw || n0 + di >= g.N) return;
 
-    const int8_t* xp = x + (size_t)plane * g.H * g.W * 8;
+    // scalar base of the wave's first image + a 32-bit lane offset (the host keeps ipw image strides below 2^31)
+    const int8_t* xp = x + ((size_t)n0 * C8 + o) * g.H * g.W * 8;
+    const unsigned in_img = (unsigned)di * (unsigned)(C8 * g.H * g.W * 8);
     const int ix0 = ox * S - g.pw;
     // columns 0 and 2 of the window can fall off the image for the first / last output column only: read a clamped
     // address and zero the value
     // (the middle column is always inside: pad <= 1 is checked on the host)
     const bool c0_ok = ix0 >= 0, c2_ok = ix0 + 2 < g.W;
-    const int ixc0 = max(ix0, 0), ixc1 = ix0 + 1, ixc2 = min(ix0 + 2, g.W - 1);
+    const unsigned ixc0 = in_img + max(ix0, 0) * 8, ixc1 = in_img + (ix0 + 1) * 8, ixc2 = in_img + min(ix0 + 2, g.W - 1) * 8;
     const int oy0 = strip * R;
     const int OHW = g.OH * g.OW;
 
@@ -143,9 +154,9 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
         const int iy = iy_base + r;
         if (iy >= 0 && iy < g.H) {  // wave-uniform
             const int8_t* rp = xp + (size_t)iy * g.W * 8;
-            const v2i a = *reinterpret_cast<const v2i*>(rp + (size_t)ixc0 * 8);
-            const v2i b = *reinterpret_cast<const v2i*>(rp + (size_t)ixc1 * 8);
-            const v2i c = *reinterpret_cast<const v2i*>(rp + (size_t)ixc2 * 8);
+            const v2i a = *reinterpret_cast<const v2i*>(rp + ixc0);
+            const v2i b = *reinterpret_cast<const v2i*>(rp + ixc1);
+            const v2i c = *reinterpret_cast<const v2i*>(rp + ixc2);
             rows[r][0] = c0_ok ? a : v2i{0, 0};
             rows[r][1] = b;
             rows[r][2] = c2_ok ? c : v2i{0, 0};
@@ -200,11 +211,12 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
         }
         __builtin_amdgcn_sched_barrier(0);  // the second half's scalars are fetched after the first half is done
     }
-    int8_t* op = out + (size_t)plane * OHW * 8;
+    int8_t* op = out + ((size_t)n0 * C8 + o) * OHW * 8;
+    const unsigned out_lane = (unsigned)di * (unsigned)(C8 * OHW * 8) + (unsigned)ox * 8;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int oy = oy0 + r;
-        if (oy < g.OH) *reinterpret_cast<v2i*>(op + ((size_t)oy * g.OW + ox) * 8) = v2i{packed[0][r], packed[1][r]};
+        if (oy < g.OH) *reinterpret_cast<v2i*>(op + (size_t)oy * g.OW * 8 + out_lane) = v2i{packed[0][r], packed[1][r]};
     }
 }
 
@@ -264,9 +276,17 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
         const int col_chunks = (g.OW + 63) / 64;
         const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
         const int blocks8 = col_chunks * (n_strips / wpb);
+        // narrow images: several images of the same channel octet share a wave (lane offsets stay below 2^31)
+        int ipw = 1;
+        if (g.OW <= 32) {
+            ipw = std::min(64 / g.OW, g.N);
+            const size_t img = (size_t)g.C * std::max(g.H * g.W, g.OH * g.OW);
+            while (ipw > 1 && img * ipw >= ((size_t)1 << 31)) --ipw;
+        }
+        const int groups8 = ((g.N + ipw - 1) / ipw) * (g.C / 8);
 #define OHIP_DW8(S_, R_, N_) \
-    hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, planes), dim3(64 * wpb), 0, stream, x, wmask, \
-                       (int8_t*)out, g, ep, n_strips, col_chunks)
+    hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, groups8), dim3(64 * wpb), 0, stream, x, wmask, \
+                       (int8_t*)out, g, ep, n_strips, col_chunks, ipw)
         if (g.sh == 1) {
             if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(1, R1, true);
             else if (epi == EPI_I8_P8) OHIP_DW8(1, R1, false);

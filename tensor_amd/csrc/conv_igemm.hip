@@ -249,18 +249,32 @@ static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, co
     }
 }
 
-// tile choice: the widest row tile that does not pad M further, then the widest pixel tile that still
-// leaves at least two workgroups per compute unit
+// tile choice. Long reductions (3x3 and larger over many channels) are MFMA-bound: the widest row tile that does not
+// pad M further, then the widest pixel tile that still leaves two workgroups per compute unit. Short reductions
+// (pointwise layers, at most 16 k-chunks) are bound by latency and HBM: there the 128x256 tile's register count costs
+// more occupancy than its reuse saves, and the tiles below were the fastest ones measured on MI355X over the pointwise
+// shapes of a MobileNetV2 at batch 64 and 256->512 at 28x28.
 void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
     const int mpad = igemm_padded_rows(g.K);
-    int TM = 32;
-    if (mpad % 128 == 0) TM = 128;
-    else if (mpad % 64 == 0) TM = 64;
     const long total_pix = (long)g.N * g.OH * g.OW;
-    const long m_tiles = mpad / TM;
-    int TN = 64;
-    if (((total_pix + 255) / 256) * m_tiles >= 512) TN = 256;
-    else if (((total_pix + 127) / 128) * m_tiles >= 512) TN = 128;
+    const int n_chunks = g.kh * g.kw * igemm_channel_groups(g.C);
+    auto wgs = [&](int TM, int TN) { return ((total_pix + TN - 1) / TN) * (mpad / TM); };
+    int TM = 32, TN = 64;
+    if (n_chunks > 16) {
+        if (mpad % 128 == 0) TM = 128;
+        else if (mpad % 64 == 0) TM = 64;
+        if (wgs(TM, 256) >= 512) TN = 256;
+        else if (wgs(TM, 128) >= 512) TN = 128;
+    } else if (mpad >= 512 && mpad % 128 == 0) {
+        TM = 128;
+    } else if (mpad >= 64) {
+        TM = 64;
+        if (wgs(64, 256) >= 2048) TN = 256;
+        else if (wgs(64, 128) >= 1024) TN = 128;
+    } else {
+        if (wgs(32, 256) >= 2048) TN = 256;
+        else if (wgs(32, 128) >= 256) TN = 128;
+    }
     *tm = TM;
     *tn = TN;
 }

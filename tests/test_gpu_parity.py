@@ -222,6 +222,11 @@ def test_halo3x3_every_fragment_count(hip, oracle, fn):
     (12, 8, 3, 1, 1, 1, 1, 1, 8, 8),        # C % 8 != 0
     (64, 64, 3, 1, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s1, ragged strips
     (64, 64, 3, 2, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s2
+    (16, 16, 3, 1, 1, 1, 16, 11, 7, 7),     # depthwise, narrow image: 9 images share a wave, ragged last group
+    (24, 24, 3, 1, 1, 1, 24, 5, 14, 14),    # 4 images per wave
+    (16, 16, 3, 2, 1, 1, 16, 5, 28, 28),    # stride 2 to 14 columns: 4 images per wave
+    (8, 8, 3, 1, 1, 1, 8, 3, 9, 32),        # 2 images per wave, full wave
+    (8, 8, 3, 1, 0, 1, 8, 3, 9, 33),        # 33 columns: one image per wave again; pad 0
     (16, 16, 7, 1, 3, 1, 16, 1, 12, 12),    # depthwise 7x7
     (16, 16, 3, 1, 2, 2, 16, 1, 12, 12),    # depthwise dilated -> generic depthwise kernel
     (128, 128, 3, 1, 1, 1, 1, 4, 56, 56),   # the c3 layer at reduced batch

@@ -360,7 +360,7 @@ def main():
         sys.exit(2)
 
     wl = builders[a.workload](np.random.default_rng(0))
-    unit = "TOPS" if wl["bound"] == "mfma" else ("images/s" if wl["name"] == "c4" else "GB/s")
+    unit = "images/s" if wl["name"] == "c4" else ("GB/s" if "bytes" in wl else "TOPS")
     res = measure(wl, timer, a.steps, a.warmup, unit)
     if wl["name"] == "c4":
         value = wl["images"] / (res["ms_per_step"] * 1e-3)

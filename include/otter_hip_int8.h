@@ -142,7 +142,9 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
 /* Tuning / test hook with no counterpart in the reference. (0, 0): automatic choice. tm > 0: force the generic
  * MFMA implicit-GEMM kernel with a tile of tm output channels x tn pixels (tm in {32,64,128}, tn in
  * {64,128,256}). tm < 0: keep the 3x3 halo kernel where it applies and force its pixel-fragment count to tn
- * (4..7, 0 = automatic). */
+ * (4..7, 0 = automatic). tm == -2 on a depthwise 3x3 layer: force the matrix-core kernel's strip height to tn
+ * steps of 8 / stride output rows (0 = automatic). tm == -3: use the vector-ALU depthwise kernels instead, with a
+ * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
 /* ------------------------------------------------------------------------------------------------ */

@@ -52,6 +52,7 @@ struct otter_hip_conv {
     int8_t* w_raw = nullptr;     // [K, C/g, kh, kw]           (direct kernel)
     int8_t* w_igemm = nullptr;   // MFMA lane order            (groups == 1, C % 8 == 0)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
+    int8_t* w_dw_mfma = nullptr; // block-diagonal MFMA operands (depthwise 3x3, C % 8 == 0)
     float* scale_in = nullptr;   // [Kpad]
     float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
     float* scale_out = nullptr;  // [Kpad] or null
@@ -138,6 +139,7 @@ int otter_hip_conv_destroy(otter_hip_conv_t* h) {
     (void)hipFree(h->w_raw);
     (void)hipFree(h->w_igemm);
     (void)hipFree(h->w_dw);
+    (void)hipFree(h->w_dw_mfma);
     (void)hipFree(h->scale_in);
     (void)hipFree(h->bias);
     (void)hipFree(h->scale_out);
@@ -186,6 +188,11 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             std::vector<int32_t> wm(dw_packed_weight_bytes(C, d.kernel_h, d.kernel_w) / sizeof(int32_t));
             dw_pack_weights(weight, C, d.kernel_h, d.kernel_w, wm.data());
             if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
+            if (d.kernel_h == 3 && d.kernel_w == 3) {
+                std::vector<int8_t> wa(dw_mfma_weight_bytes(C));
+                dw_mfma_pack_weights(weight, C, wa.data());
+                if ((rc = upload<int8_t>(&h->w_dw_mfma, wa.data(), wa.size(), wa.size(), 0))) break;
+            }
         } else if (g == 1 && C % 8 == 0) {
             std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
             igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
@@ -342,22 +349,24 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     case 3:
         OHIP_CHECK(run_conv3x3_halo(xq, h->w_igemm, out, g, ep, h->force_tm < 0 ? h->force_tn : 0, stream));
         break;
-    case 2:
-        if ((long)n * (g.C / 8) > 65535) {
-            // the plane index rides on grid.y: run the batch in slices
-            const int per = 65535 / (g.C / 8);
-            if (per < 1) return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: too many channels");
-            for (int b = 0; b < n; b += per) {
-                ConvGeom gs = g;
-                gs.N = (n - b < per) ? n - b : per;
-                const size_t in_off = (size_t)b * g.C * in_h * in_w;
-                const size_t out_off = (size_t)b * g.K * g.OH * g.OW * layout_elem_bytes(out_layout);
-                OHIP_CHECK(run_conv_dw(xq + in_off, h->w_dw, (char*)out + out_off, gs, ep, stream));
-            }
-        } else {
-            OHIP_CHECK(run_conv_dw(xq, h->w_dw, out, g, ep, stream));
+    case 2: {
+        // set_tile(-2, s): force the strip height; set_tile(-3, s): same, on the vector-ALU kernels
+        const int dw_shift = (h->force_tm == -2 || h->force_tm == -3) ? h->force_tn : -1;
+        const int epi = pick_epilogue(ep, g.K);
+        const bool mfma = h->w_dw_mfma && h->force_tm != -3 && dw_mfma_applicable(g, ep, epi);
+        // the (image group, channel group) index rides on grid.y: run a very large batch in slices
+        const int per = 32768 / (g.C / 8);
+        if (per < 1) return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: too many channels");
+        for (int b = 0; b < n; b += per) {
+            ConvGeom gs = g;
+            gs.N = (n - b < per) ? n - b : per;
+            const int8_t* xs = xq + (size_t)b * g.C * in_h * in_w;
+            void* os = (char*)out + (size_t)b * g.K * g.OH * g.OW * layout_elem_bytes(out_layout);
+            if (mfma) OHIP_CHECK(run_conv_dw_mfma(xs, h->w_dw_mfma, os, gs, ep, epi, dw_shift, stream));
+            else OHIP_CHECK(run_conv_dw(xs, h->w_dw, os, gs, ep, dw_shift, stream));
         }
         break;
+    }
     case 1:
         OHIP_CHECK(run_conv_igemm(xq, h->w_igemm, out, g, ep, h->force_tm, h->force_tn, stream));
         break;

@@ -257,7 +257,7 @@ __global__ void __launch_bounds__(256) conv_dw_generic_kernel(const int8_t* __re
 }
 
 hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const ConvGeom& g, const Epilogue& ep,
-                       hipStream_t stream) {
+                       int strip_shift, hipStream_t stream) {
     const int planes = g.N * (g.C / 8);
     if (planes == 0 || g.OH * g.OW == 0) return hipSuccess;
     if (planes > 65535) return hipErrorInvalidValue;  // grid.y limit; the caller splits the batch
@@ -272,11 +272,8 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
 #define OHIP_DW(S_, R_, E_) \
     hipLaunchKernelGGL((conv_dw3x3_kernel<S_, R_, E_>), dim3(blocks, planes), dim3(256), 0, stream, x, wmask, out, g, ep, \
                        n_strips)
-        // one wave per (strip, 64-column chunk); waves per workgroup chosen so that no wave is born idle
-        const int col_chunks = (g.OW + 63) / 64;
-        const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
-        const int blocks8 = col_chunks * (n_strips / wpb);
         // narrow images: several images of the same channel octet share a wave (lane offsets stay below 2^31)
+        const int col_chunks = (g.OW + 63) / 64;
         int ipw = 1;
         if (g.OW <= 32) {
             ipw = std::min(64 / g.OW, g.N);
@@ -284,18 +281,35 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
             while (ipw > 1 && img * ipw >= ((size_t)1 << 31)) --ipw;
         }
         const int groups8 = ((g.N + ipw - 1) / ipw) * (g.C / 8);
+        // rows per strip: the tallest strip (most reuse of input rows, fewest scalar loads per output) that still gives
+        // every SIMD four waves; a small layer is latency-bound and wants many short waves instead
+        int shift = 0;  // strip height = R >> shift
+        if (strip_shift >= 0) shift = std::min(strip_shift, 2);
+        else while (shift < 2 && (long)col_chunks * ((g.OH + (R >> shift) - 1) / (R >> shift)) * groups8 < 4096) ++shift;
+        const int Rs = R >> shift;
+        const int strips8 = (g.OH + Rs - 1) / Rs;
+        // one wave per (strip, 64-column chunk); waves per workgroup chosen so that no wave is born idle
+        const int wpb = strips8 % 4 == 0 ? 4 : (strips8 % 2 == 0 ? 2 : 1);
+        const int blocks8 = col_chunks * (strips8 / wpb);
 #define OHIP_DW8(S_, R_, N_) \
     hipLaunchKernelGGL((conv_dw3x3_i8_kernel<S_, R_, N_>), dim3(blocks8, groups8), dim3(64 * wpb), 0, stream, x, wmask, \
-                       (int8_t*)out, g, ep, n_strips, col_chunks, ipw)
+                       (int8_t*)out, g, ep, strips8, col_chunks, ipw)
+#define OHIP_DW8_R(S_, RMAX_, N_)                  \
+    do {                                           \
+        if (shift == 0) OHIP_DW8(S_, RMAX_, N_);   \
+        else if (shift == 1) OHIP_DW8(S_, RMAX_ / 2, N_); \
+        else OHIP_DW8(S_, RMAX_ / 4, N_);          \
+    } while (0)
         if (g.sh == 1) {
-            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(1, R1, true);
-            else if (epi == EPI_I8_P8) OHIP_DW8(1, R1, false);
+            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8_R(1, R1, true);
+            else if (epi == EPI_I8_P8) OHIP_DW8_R(1, R1, false);
             else OHIP_DW(1, R1, EPI_GENERIC);
         } else {
-            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8(2, R2, true);
-            else if (epi == EPI_I8_P8) OHIP_DW8(2, R2, false);
+            if (epi == EPI_I8_P8_NONNEG) OHIP_DW8_R(2, R2, true);
+            else if (epi == EPI_I8_P8) OHIP_DW8_R(2, R2, false);
             else OHIP_DW(2, R2, EPI_GENERIC);
         }
+#undef OHIP_DW8_R
 #undef OHIP_DW
 #undef OHIP_DW8
     } else {

@@ -24,10 +24,15 @@ hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void*
                            const Epilogue& ep, hipStream_t stream);
 
 // conv_dw.hip
+size_t dw_mfma_weight_bytes(int C);
+void dw_mfma_pack_weights(const int8_t* w, int C, int8_t* dst);
+bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi);
+hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
+                            int strip_shift, hipStream_t stream);
 size_t dw_packed_weight_bytes(int C, int kh, int kw);
 void dw_pack_weights(const int8_t* w, int C, int kh, int kw, int32_t* dst);
 hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const ConvGeom& g, const Epilogue& ep,
-                       hipStream_t stream);
+                       int strip_shift, hipStream_t stream);
 
 // elementwise.hip
 hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,

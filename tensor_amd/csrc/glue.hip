@@ -24,31 +24,86 @@ __global__ void __launch_bounds__(256) activation_kernel(float* __restrict__ x, 
     if (i < n) x[i] = activate(x[i], act, p0);
 }
 
-// mean over H*W per (n, c); input in any fp32 layout, output [N, C] unpacked. One wave per (n, c).
-__global__ void __launch_bounds__(256) global_avgpool_kernel(const float* __restrict__ x, int pack, int N, int C, int HW,
+// mean over H*W per (n, c); input in any fp32 layout, output [N, C] unpacked. One wave per (n, channel pack): a lane
+// reads whole packs (4, 16 or 32 contiguous bytes per pixel), so a wave's reads are contiguous in every layout.
+template <int P>
+__global__ void __launch_bounds__(256) global_avgpool_kernel(const float* __restrict__ x, int N, int C, int HW,
                                                              float* __restrict__ out) {
+    typedef float vec_t __attribute__((ext_vector_type(P)));
     const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6, lane = threadIdx.x & 63;
-    if (wave >= N * C) return;
-    const int n = wave / C, c = wave % C;
-    float s = 0.f;
-    for (int i = lane; i < HW; i += 64) s += x[elem_offset(pack, n, c, i, C, HW)];
+    const int CP = C / P;
+    if (wave >= N * CP) return;
+    const int n = wave / CP, cp = wave % CP;
+    const float* src = x + ((size_t)n * CP + cp) * HW * P;
+    float s[P];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s += __shfl_down(s, o, 64);
-    if (lane == 0) out[wave] = s / (float)HW;
+    for (int e = 0; e < P; ++e) s[e] = 0.f;
+    for (int i = lane; i < HW; i += 64) {
+        if constexpr (P == 1) {
+            s[0] += src[i];
+        } else {
+            const vec_t v = *reinterpret_cast<const vec_t*>(src + (size_t)i * P);
+#pragma unroll
+            for (int e = 0; e < P; ++e) s[e] += v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) s[e] += __shfl_down(s[e], o, 64);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int e = 0; e < P; ++e) out[(size_t)n * C + cp * P + e] = s[e] / (float)HW;
+    }
 }
 
-// y[n][o] = sum_i x[n][i] * w[o][i] + b[o]   (Tensor/InnerProductLayer.cpp:176-, fp32). One wave per output.
+// y[n][o] = sum_i x[n][i] * w[o][i] + b[o]   (Tensor/InnerProductLayer.cpp:176-, fp32).
+// A workgroup owns IP_OB outputs x IP_NB images; its four waves split the reduction index, every lane keeps the
+// IP_OB x IP_NB partial sums of its own indices in registers (each loaded weight is used IP_NB times, each input IP_OB
+// times), and the 256 partial sums per result are added up through LDS at the end.
+constexpr int IP_OB = 4, IP_NB = 8;
 __global__ void __launch_bounds__(256) inner_product_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             const float* __restrict__ b, float* __restrict__ y, int N,
                                                             int IN, int OUT) {
-    const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6, lane = threadIdx.x & 63;
-    if (wave >= N * OUT) return;
-    const int n = wave / OUT, o = wave % OUT;
-    float s = 0.f;
-    for (int i = lane; i < IN; i += 64) s = __fmaf_rn(x[(size_t)n * IN + i], w[(size_t)o * IN + i], s);
+    __shared__ float part[IP_OB * IP_NB][257];
+    const int o0 = blockIdx.x * IP_OB, n0 = blockIdx.y * IP_NB;
+    const float* wr[IP_OB];
+    const float* xr[IP_NB];
 #pragma unroll
-    for (int k = 32; k > 0; k >>= 1) s += __shfl_down(s, k, 64);
-    if (lane == 0) y[wave] = s + (b ? b[o] : 0.f);
+    for (int j = 0; j < IP_OB; ++j) wr[j] = w + (size_t)min(o0 + j, OUT - 1) * IN;  // clamped rows are computed, not stored
+#pragma unroll
+    for (int k = 0; k < IP_NB; ++k) xr[k] = x + (size_t)min(n0 + k, N - 1) * IN;
+    float acc[IP_OB][IP_NB];
+#pragma unroll
+    for (int j = 0; j < IP_OB; ++j)
+#pragma unroll
+        for (int k = 0; k < IP_NB; ++k) acc[j][k] = 0.f;
+    for (int i = threadIdx.x; i < IN; i += 256) {
+        float wv[IP_OB], xv[IP_NB];
+#pragma unroll
+        for (int j = 0; j < IP_OB; ++j) wv[j] = wr[j][i];
+#pragma unroll
+        for (int k = 0; k < IP_NB; ++k) xv[k] = xr[k][i];
+#pragma unroll
+        for (int j = 0; j < IP_OB; ++j)
+#pragma unroll
+            for (int k = 0; k < IP_NB; ++k) acc[j][k] = __fmaf_rn(wv[j], xv[k], acc[j][k]);
+    }
+#pragma unroll
+    for (int j = 0; j < IP_OB; ++j)
+#pragma unroll
+        for (int k = 0; k < IP_NB; ++k) part[j * IP_NB + k][threadIdx.x] = acc[j][k];
+    __syncthreads();
+    // four threads per result, 64 partial sums each
+    const int r = threadIdx.x >> 2, q = threadIdx.x & 3;
+    if (r >= IP_OB * IP_NB) return;  // whole waves: results 0..31 live in the first two
+    float s = 0.f;
+    for (int t = 0; t < 64; ++t) s += part[r][t * 4 + q];
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    const int o = o0 + r / IP_NB, n = n0 + r % IP_NB;
+    if (q == 0 && o < OUT && n < N) y[(size_t)n * OUT + o] = s + (b ? b[o] : 0.f);
 }
 
 hipError_t run_eltwise_add(const float* a, const float* b, float* out, size_t n, hipStream_t stream) {
@@ -67,14 +122,19 @@ hipError_t run_activation(float* x, size_t n, int act, float p0, hipStream_t str
 
 hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, float* out, hipStream_t stream) {
     if (N * C == 0) return hipSuccess;
-    hipLaunchKernelGGL(global_avgpool_kernel, dim3((N * C + 3) / 4), dim3(256), 0, stream, x, pack, N, C, HW, out);
+    const unsigned blocks = (unsigned)((N * (C / pack) + 3) / 4);
+    if (pack == 8) hipLaunchKernelGGL(global_avgpool_kernel<8>, dim3(blocks), dim3(256), 0, stream, x, N, C, HW, out);
+    else if (pack == 4) hipLaunchKernelGGL(global_avgpool_kernel<4>, dim3(blocks), dim3(256), 0, stream, x, N, C, HW, out);
+    else if (pack == 1) hipLaunchKernelGGL(global_avgpool_kernel<1>, dim3(blocks), dim3(256), 0, stream, x, N, C, HW, out);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream) {
     if (N * OUT == 0) return hipSuccess;
-    hipLaunchKernelGGL(inner_product_kernel, dim3((N * OUT + 3) / 4), dim3(256), 0, stream, x, w, b, y, N, IN, OUT);
+    hipLaunchKernelGGL(inner_product_kernel, dim3((OUT + IP_OB - 1) / IP_OB, (N + IP_NB - 1) / IP_NB), dim3(256), 0, stream,
+                       x, w, b, y, N, IN, OUT);
     return hipGetLastError();
 }
 

@@ -251,6 +251,29 @@ def test_random_shapes_against_oracle(hip, oracle, C, K, k, s, p, d, g, N, H, W)
             assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("shift", [0, 1, 2])
+@pytest.mark.parametrize("s", [1, 2])
+@pytest.mark.parametrize("family", [-2, -3], ids=["mfma", "valu"])
+def test_depthwise3x3_every_strip_height(hip, oracle, family, s, shift):
+    """The depthwise 3x3 kernels (matrix-core and vector-ALU family) are instantiated for three strip heights per
+    stride, chosen from the problem size: force each on shapes with ragged last strips, narrow images sharing a
+    wave, more than 64 columns, a channel count that ends on a single octet, pad 0, and every fast epilogue."""
+    rng = np.random.default_rng(10 * s + shift)
+    for (C, N, H, W, p) in [(16, 3, 19, 70, 1), (8, 7, 13, 9, 1), (24, 5, 8, 8, 0), (40, 3, 9, 5, 1),
+                            (8, 1, 33, 64, 1)]:
+        x, wq, ws, bias = _rand_problem(rng, C, C, 3, C, N, H, W)
+        for act, int8_out in ((3, True), (0, True), (1, False)):
+            want = oracle.conv_layer_forward(x, wq, ws, 20.0, stride=(s, s), pad=(p, p), groups=C, bias=bias,
+                                             top_scale=9.0, int8_out=int8_out, act_type=act)
+            out, kind = run_conv(hip, oracle, x, wq, ws, 20.0, stride=s, pad=p, groups=C, bias=bias, top_scale=9.0,
+                                 act=act, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32, tile=(family, shift))
+            assert kind == 2
+            if int8_out:
+                np.testing.assert_array_equal(out, want)
+            else:
+                assert_f32_close(out, want)
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

@@ -1,5 +1,6 @@
 // extern "C" boundary of the library (include/otter_hip_int8.h): argument checking, handle management,
 // weight re-layout at create time and kernel dispatch. No kernels live here.
+#include <cmath>
 #include <cstring>
 #include <new>
 #include <string>
@@ -53,6 +54,7 @@ struct otter_hip_conv {
     int8_t* w_igemm = nullptr;   // MFMA lane order            (groups == 1, C % 8 == 0)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
     int8_t* w_dw_mfma = nullptr; // block-diagonal MFMA operands (depthwise 3x3, C % 8 == 0)
+    bool so_positive = true;     // every output scale is finite and > 0
     float* scale_in = nullptr;   // [Kpad]
     float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
     float* scale_out = nullptr;  // [Kpad] or null
@@ -180,7 +182,10 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
         if ((rc = upload<float>(&h->bias, bias, bias ? K : 0, kpad, -0.0f))) break;
         if (d.out_kind == OTTER_HIP_OUT_I8) {
             std::vector<float> so(K);
-            for (int i = 0; i < K; ++i) so[i] = n_out_scale == 1 ? out_scale[0] : out_scale[i];
+            for (int i = 0; i < K; ++i) {
+                so[i] = n_out_scale == 1 ? out_scale[0] : out_scale[i];
+                if (!(so[i] > 0.f) || std::isinf(so[i])) h->so_positive = false;
+            }
             if ((rc = upload<float>(&h->scale_out, so.data(), K, kpad, 1.f))) break;
         }
         if ((rc = upload<float>(&h->in_scale, &in_scale, 1, 1, 0.f))) break;
@@ -188,9 +193,10 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             std::vector<int32_t> wm(dw_packed_weight_bytes(C, d.kernel_h, d.kernel_w) / sizeof(int32_t));
             dw_pack_weights(weight, C, d.kernel_h, d.kernel_w, wm.data());
             if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
-            if (d.kernel_h == 3 && d.kernel_w == 3) {
-                std::vector<int8_t> wa(dw_mfma_weight_bytes(C));
-                dw_mfma_pack_weights(weight, C, wa.data());
+            if (d.kernel_h == 3 && d.kernel_w == 3 && d.stride_h == d.stride_w && (d.stride_w == 1 || d.stride_w == 2) &&
+                d.pad_w <= 1) {
+                std::vector<int8_t> wa(dw_mfma_weight_bytes(C, d.stride_w));
+                dw_mfma_pack_weights(weight, C, d.stride_w, d.pad_w, wa.data());
                 if ((rc = upload<int8_t>(&h->w_dw_mfma, wa.data(), wa.size(), wa.size(), 0))) break;
             }
         } else if (g == 1 && C % 8 == 0) {
@@ -353,7 +359,7 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         // set_tile(-2, s): force the strip height; set_tile(-3, s): same, on the vector-ALU kernels
         const int dw_shift = (h->force_tm == -2 || h->force_tm == -3) ? h->force_tn : -1;
         const int epi = pick_epilogue(ep, g.K);
-        const bool mfma = h->w_dw_mfma && h->force_tm != -3 && dw_mfma_applicable(g, ep, epi);
+        const bool mfma = h->w_dw_mfma && h->force_tm != -3 && dw_mfma_applicable(g, ep, epi, h->so_positive);
         // the (image group, channel group) index rides on grid.y: run a very large batch in slices
         const int per = 32768 / (g.C / 8);
         if (per < 1) return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: too many channels");

@@ -3,18 +3,21 @@
 //
 // Why matrix cores for a layer with no channel reduction: with dot4 on the vector ALU the layer costs ~20 vector
 // instructions per output value (9 dot4 + requantize) and is bound by the vector ALU at ~2x the time HBM needs.
-// v_mfma_i32_16x16x64_i8 computes D[16 ch][16 px] += A[16 ch][64] * B[64][16 px]. Give the 64-deep reduction the
-// meaning (column tap dx = 0..2 (+1 unused), channel j = 0..15) and let A be zero except A[i][(dx, i)] = w[i][dy][dx]:
-// one instruction then does one kernel ROW of 16 channels x 16 pixels, three instructions do the 3x3 window, and the
-// vector ALU is left with the requantize epilogue only. Three quarters of the multiplies are by zero; the matrix
-// pipe has the room (it runs beside the vector ALU).
+// v_mfma_i32_16x16x64_i8 computes D[16][16] += A[16][64] * B[64][16]. Here a B column n is a run of 4 output pixels
+// (stride 1; 2 for stride 2) of one channel octet, and its 64 reduction bytes are the 8 input pixels 4n-2 .. 4n+5 of
+// one input row x 8 channels: lane (n, g = lane / 16) supplies pixels 4n-2+2g and +1, i.e. ONE aligned 16-byte load.
+// A D row m is (output pixel phase p, channel c) and A is zero except A[(p, c)][(pixel e, channel c)] = w[c][dy][dx]
+// for the dx that connects input pixel e to output phase p. One instruction does one kernel ROW for 16 x 16 (phase,
+// channel, column) outputs, three do the 3x3 window, and the vector ALU is left with the requantize epilogue only.
+// Most multiplies are by zero; the matrix pipe has the room (it runs beside the vector ALU).
 //
-// The B operand needs no data movement beyond the load: lane (px = lane % 16, dx = lane / 16) supplies 16 reduction
-// bytes = channels 0..15 of input pixel (row, px*S + dx - pad) = two 8-byte Byte8 elements from two adjacent channel
-// octets. A lane's fragment of input row y serves kernel row 2 of output row y-2, row 1 of y-1 and row 0 of y (stride
-// 1), so a wave walks down a strip of output rows, loading each input row once and keeping three in registers.
+// Stride 1: two A sets (channels 0-3 and 4-7 of the octet) share the B fragment; a lane ends up with all 8 channels
+// of output pixel 4n + lane/16 and stores one Byte8 element. Stride 2: one A set, rows = 2 phases x 8 channels; a
+// lane ends up with 4 channels of output pixel 2n + lane/32.
+// A lane's fragment of input row y serves kernel row 2 of output row y-2, row 1 of y-1 and row 0 of y (stride 1),
+// so a wave walks down a strip of output rows with the input rows in a ring of registers, each loaded once.
 // Image borders cost no instructions: loads and stores go through buffer descriptors, a lane that falls outside
-// the image (or outside the channel count) carries an out-of-range offset, reads zero and writes nothing.
+// the image carries an out-of-range offset, reads zero and writes nothing.
 #include <algorithm>
 
 #include "common.hpp"
@@ -24,19 +27,34 @@ namespace ohip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v4u_store __attribute__((__vector_size__(4 * sizeof(unsigned))));
+typedef unsigned v2u_store __attribute__((__vector_size__(2 * sizeof(unsigned))));
 
-// weight [C, 1, 3, 3] int8 -> A operands [C/16 groups][kernel row 3][lane 64][16 bytes]:
-// lane (i = lane % 16, dx = lane / 16) holds w[16*group + i][row][dx] in byte i, zero elsewhere
-size_t dw_mfma_weight_bytes(int C) { return (size_t)((C + 15) / 16) * 3 * 64 * 16; }
+// weight [C, 1, 3, 3] int8 -> A operands [C/8 octets][kernel row 3][set T][lane 64][16 bytes], T = 2 for stride 1
+// (set t = channels 4t..4t+3) and 1 for stride 2. Lane (r = lane % 16, g = lane / 16) holds A[row r][16g .. 16g+15];
+// reduction byte 16g + 8e + j is (input pixel 4n-2+2g+e, channel j).
+static int dw_mfma_sets(int stride) { return stride == 1 ? 2 : 1; }
+size_t dw_mfma_weight_bytes(int C, int stride) { return (size_t)(C / 8) * 3 * dw_mfma_sets(stride) * 64 * 16; }
 
-void dw_mfma_pack_weights(const int8_t* w, int C, int8_t* dst) {
-    std::fill(dst, dst + dw_mfma_weight_bytes(C), (int8_t)0);
-    for (int c = 0; c < C; ++c)
+void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t* dst) {
+    const int T = dw_mfma_sets(stride);
+    std::fill(dst, dst + dw_mfma_weight_bytes(C, stride), (int8_t)0);
+    for (int o = 0; o < C / 8; ++o)
         for (int dy = 0; dy < 3; ++dy)
-            for (int dx = 0; dx < 3; ++dx) {
-                const int grp = c / 16, i = c % 16, lane = dx * 16 + i;
-                dst[(((size_t)grp * 3 + dy) * 64 + lane) * 16 + i] = w[(size_t)c * 9 + dy * 3 + dx];
-            }
+            for (int t = 0; t < T; ++t)
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int r = lane % 16, g = lane / 16;
+                    // D row r -> (output pixel phase p, channel c of the octet)
+                    const int p = stride == 1 ? r / 4 : r / 8;
+                    const int c = stride == 1 ? 4 * t + r % 4 : r % 8;
+                    for (int e = 0; e < 2; ++e) {
+                        // input pixel 4n - 2 + 2g + e feeds output pixel (4/stride) n + p through tap dx
+                        const int dx = 2 * g + e - 2 - stride * p + pad_w;
+                        if (dx < 0 || dx > 2) continue;
+                        dst[((((size_t)o * 3 + dy) * T + t) * 64 + lane) * 16 + 8 * e + c] =
+                            w[(size_t)(8 * o + c) * 9 + dy * 3 + dx];
+                    }
+                }
 }
 
 constexpr unsigned DW_OOB = 0x80000000u;  // beyond any descriptor this file builds (tensors are kept below 2 GiB)
@@ -45,38 +63,86 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t dw_rsrc(const void* p, unsigne
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
 
-// A wave owns 16 output columns x 16 channels and walks down `rps` output rows. The input rows live in a ring of 8
-// register fragments: a step computes 8/S output rows from the ring and refills every slot as soon as its last reader
-// has issued, so the loads run 5 input rows ahead of the matrix instructions for the whole walk.
-template <int S, int EPI>
+// Requantize four accumulators into four saturated bytes of one dword.
+// The activation clamp [0, hi] is applied AFTER scaling and rounding, on the packed int16 values, instead of on the
+// float before them: x -> trunc(fl(fl(x * so) + half)) is monotone for so > 0, so clamping its argument to [0, hi]
+// equals clamping its result to [trunc(0 + half), trunc(fl(fl(hi * so) + half))] = [0, qh], bit for bit; qh (capped at
+// the int8 saturation bound 127) is computed once per wave by dw_clamp_pair. Without an activation there is no clamp.
+__device__ __forceinline__ unsigned dw_clamp_pair(const Epilogue& ep, int so0, int so1) {
+    const int q0 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, __int_as_float(so0)), ep.round_half), 127);
+    const int q1 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, __int_as_float(so1)), ep.round_half), 127);
+    return (unsigned)(q0 & 0xffff) | ((unsigned)q1 << 16);
+}
+
+template <bool NONNEG>
+__device__ __forceinline__ unsigned dw_requant4(const Epilogue& ep, const v4i& acc, const v4i& si, const v4i& bi,
+                                                const v4i& so, unsigned qh01, unsigned qh23) {
+    int qv[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = __fmaf_rn((float)acc[e], __int_as_float(si[e]), __int_as_float(bi[e]));
+        v = __fmul_rn(v, __int_as_float(so[e]));
+        const float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
+        qv[e] = (int)adj;  // toward zero, saturating
+    }
+    ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[0], qv[1]));
+    ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[2], qv[3]));
+    if (NONNEG) {
+        const ohip_v2s zero = {0, 0};
+        lo = __builtin_elementwise_max(__builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2s, qh01)), zero);
+        hi = __builtin_elementwise_max(__builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2s, qh23)), zero);
+    } else {
+        const ohip_v2s top = {127, 127}, bot = {-127, -127};
+        lo = __builtin_elementwise_max(__builtin_elementwise_min(lo, top), bot);
+        hi = __builtin_elementwise_max(__builtin_elementwise_min(hi, top), bot);
+    }
+    return __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
+}
+
+__device__ __forceinline__ v4i dw_dequant4(const Epilogue& ep, const v4i& acc, const v4i& si, const v4i& bi) {
+    v4i res;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = __fmaf_rn((float)acc[e], __int_as_float(si[e]), __int_as_float(bi[e]));
+        v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        res[e] = __float_as_int(v);
+    }
+    return res;
+}
+
+// A wave owns one channel octet x 16 lane columns (64 output pixels of a row at stride 1, 32 at stride 2) and walks
+// down `rps` output rows. The input rows live in a ring of 8 register fragments: a step computes 8/S output rows
+// from the ring and refills every slot as soon as its last reader has issued, so the loads run 5 input rows ahead of
+// the matrix instructions for the whole walk. Narrow images sit side by side in the wave (`lpi` lane columns each).
+template <int S, int EPI, bool ODDW>
 __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wa,
                                                               void* __restrict__ out, ConvGeom g, Epilogue ep,
-                                                              int n_strips, int rps, int col_chunks, int ipw,
+                                                              int n_strips, int rps, int col_chunks, int lpi, int ipw,
                                                               unsigned in_bytes, unsigned out_bytes) {
-    constexpr int RING = 8, U = RING / S;  // output rows per step
-    const int C8 = g.C / 8, G16 = (C8 + 1) / 2;
-    const int grp = blockIdx.y % G16;
-    const int n0 = (blockIdx.y / G16) * ipw;
+    constexpr int RING = 8, U = RING / S;  // U output rows per step
+    constexpr int PH = 4 / S;              // output pixels per lane column
+    constexpr int T = S == 1 ? 2 : 1;      // A sets
+    const int C8 = g.C / 8;
+    const int o = blockIdx.y % C8;
+    const int n0 = (blockIdx.y / C8) * ipw;
     const int chunk = blockIdx.x % col_chunks;
     const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (strip >= n_strips) return;  // whole wave
-    const int lane = threadIdx.x & 63, px = lane & 15, q = lane >> 4;
-    // 16 output columns per wave; images of at most 8 columns sit side by side (same channels, consecutive images)
-    int di = 0, ox = chunk * 16 + px;
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    int di = 0, nl = chunk * 16 + n;  // image within the wave, lane column within the image
     if (ipw > 1) {
-        di = px / g.OW;
-        ox = px - di * g.OW;
+        di = n / lpi;
+        nl = n - di * lpi;
     }
-    const bool lane_ok = ox < g.OW && di < ipw && n0 + di < g.N;
-    const bool has_hi = 2 * grp + 1 < C8;  // the group's second octet exists (C % 16 == 8 ends on a single octet)
+    const bool lane_ok = di < ipw && n0 + di < g.N;
 
-    // ---- input: per-lane byte offset (fixed for the whole walk) + per-row scalar offset -------------------------
+    // ---- input: one 16-byte load per lane and row; per-lane byte offset fixed for the walk + per-row scalar offset --
     const unsigned HW8 = (unsigned)(g.H * g.W * 8);
-    const int ix = ox * S - g.pw + q;
-    const bool col_ok = lane_ok && q < 3 && ix >= 0 && ix < g.W;
-    const unsigned v_lo = col_ok ? (unsigned)di * (unsigned)C8 * HW8 + (unsigned)ix * 8u : DW_OOB;
-    const unsigned v_hi = (col_ok && has_hi) ? v_lo + HW8 : DW_OOB;
-    const unsigned s_in = (unsigned)(n0 * C8 + 2 * grp) * HW8;
+    const int ic = 4 * nl - 2 + 2 * q;  // first input pixel of this lane's pair
+    const bool in_ok = lane_ok && ic >= 0 && ic < g.W;
+    const unsigned v_in = in_ok ? (unsigned)di * (unsigned)C8 * HW8 + (unsigned)ic * 8u : DW_OOB;
+    const unsigned v_in2 = (in_ok && ic + 1 < g.W) ? v_in + 8u : DW_OOB;  // second pixel of the pair (odd widths only)
+    const unsigned s_in = (unsigned)(n0 * C8 + o) * HW8;
     const __amdgpu_buffer_rsrc_t rin = dw_rsrc(x, in_bytes);
 
     const int oy0 = strip * rps;
@@ -86,97 +152,125 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
         const int iy = iy0 + j;
         const bool ok = iy >= 0 && iy < g.H && j < rows_needed;  // wave-uniform
         const unsigned s_row = ok ? s_in + (unsigned)(iy * g.W * 8) : 0u;
-        const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(ok ? v_lo : DW_OOB), (int)s_row, 0));
-        const v2i hi = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(ok ? v_hi : DW_OOB), (int)s_row, 0));
-        return v4i{lo[0], lo[1], hi[0], hi[1]};
+        if constexpr (ODDW) {  // odd width: a row ends on half a pair, which is loaded as 8 bytes + zero
+            const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(ok ? v_in : DW_OOB), (int)s_row, 0));
+            const v2i hi = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(ok ? v_in2 : DW_OOB), (int)s_row, 0));
+            return v4i{lo[0], lo[1], hi[0], hi[1]};
+        }
+        const v4i f = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)(ok ? v_in : DW_OOB), (int)s_row, 0));
+        return f;
     };
 
     v4i frag[RING];
 #pragma unroll
     for (int j = 0; j < RING; ++j) frag[j] = load_row(j);
 
-    const v4i* ap = reinterpret_cast<const v4i*>(wa) + (size_t)grp * 3 * 64 + lane;
-    const v4i a0 = ap[0], a1 = ap[64], a2 = ap[128];
+    v4i a[3][T];
+    {
+        const v4i* ap = reinterpret_cast<const v4i*>(wa) + (size_t)o * 3 * T * 64 + lane;
+#pragma unroll
+        for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+            for (int t = 0; t < T; ++t) a[dy][t] = ap[(dy * T + t) * 64];
+    }
 
-    // ---- epilogue constants of this lane's four channels 16*grp + 4*q .. +3 (arrays are padded past K) ---------
-    const int ch = 16 * grp + 4 * q;
-    const v4i si4 = *reinterpret_cast<const v4i*>(ep.scale_in + ch);
-    const v4i bi4 = *reinterpret_cast<const v4i*>(ep.bias + ch);
-    v4i so4 = {0, 0, 0, 0};
-    if constexpr (EPI != EPI_F32_P4) so4 = *reinterpret_cast<const v4i*>(ep.scale_out + ch);
+    // ---- epilogue constants: stride 1 -> the octet's 8 channels (same for every lane); stride 2 -> this lane's 4 ----
+    const int ch = 8 * o + (S == 1 ? 0 : 4 * (q & 1));
+    v4i si[T], bi[T], so[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        si[t] = *reinterpret_cast<const v4i*>(ep.scale_in + ch + 4 * t);
+        bi[t] = *reinterpret_cast<const v4i*>(ep.bias + ch + 4 * t);
+        so[t] = v4i{0, 0, 0, 0};
+        if constexpr (EPI != EPI_F32_P4) so[t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
+    }
+    unsigned qh[T][2] = {};
+    if constexpr (EPI == EPI_I8_P8_NONNEG) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            qh[t][0] = dw_clamp_pair(ep, so[t][0], so[t][1]);
+            qh[t][1] = dw_clamp_pair(ep, so[t][2], so[t][3]);
+        }
+    }
 
-    // ---- output: same scheme --------------------------------------------------------------------------------
+    // ---- output: this lane's pixel of the row, same addressing scheme ----------------------------------------------
     const unsigned OHW = (unsigned)(g.OH * g.OW);
-    const bool st_ok = lane_ok && (q < 2 || has_hi);
+    const int ox = PH * nl + (S == 1 ? q : (q >> 1));
+    const bool st_ok = lane_ok && ox < g.OW;
     unsigned v_out, s_out, row_bytes;
-    if constexpr (EPI == EPI_F32_P4) {  // Float4: [N][C/4][OH*OW][4 floats]; this lane's channels are pack 4*grp + q
-        v_out = st_ok ? ((unsigned)di * (unsigned)(g.C / 4) + (unsigned)q) * OHW * 16u + (unsigned)ox * 16u : DW_OOB;
-        s_out = (unsigned)(n0 * (g.C / 4) + 4 * grp) * OHW * 16u;
-        row_bytes = (unsigned)g.OW * 16u;
-    } else {  // Byte8: [N][C/8][OH*OW][8 bytes]; octet 2*grp + q/2, bytes 4*(q%2)..+3
-        v_out = st_ok ? ((unsigned)di * (unsigned)C8 + (unsigned)(q >> 1)) * OHW * 8u + (unsigned)ox * 8u + (unsigned)(q & 1) * 4u
+    if constexpr (EPI == EPI_F32_P4) {  // Float4: [N][C/4][OH*OW][4 floats]; packs 2o and 2o+1
+        v_out = st_ok ? ((unsigned)di * (unsigned)(g.C / 4) + (S == 1 ? 0u : (unsigned)(q & 1))) * OHW * 16u + (unsigned)ox * 16u
                       : DW_OOB;
-        s_out = (unsigned)(n0 * C8 + 2 * grp) * OHW * 8u;
+        s_out = (unsigned)(n0 * (g.C / 4) + 2 * o) * OHW * 16u;
+        row_bytes = (unsigned)g.OW * 16u;
+    } else {  // Byte8: [N][C/8][OH*OW][8 bytes]
+        v_out = st_ok ? (unsigned)di * (unsigned)C8 * OHW * 8u + (unsigned)ox * 8u + (S == 1 ? 0u : (unsigned)(q & 1) * 4u)
+                      : DW_OOB;
+        s_out = (unsigned)(n0 * C8 + o) * OHW * 8u;
         row_bytes = (unsigned)g.OW * 8u;
     }
     const __amdgpu_buffer_rsrc_t rout = dw_rsrc(out, out_bytes);
 
+    // Software pipeline, one output row deep: a step issues the matrix instructions of row r+1, refills the ring slots
+    // they free, and then runs the epilogue of row r while those instructions execute. The scheduling barriers keep
+    // the compiler from batching all matrix instructions at the top of the loop (which exposes the load latency).
+    auto row_mfma = [&](int u, v4i (&acc)[T]) {  // u: output row within the step (ring phase)
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc[t] = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int dy = 0; dy < 3; ++dy)
+                acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[dy][t], frag[(u * S + dy) % RING], acc[t], 0, 0, 0);
+        }
+    };
+    v4i cur[T], nxt[T];
+    row_mfma(0, cur);
+#pragma unroll
+    for (int k = 0; k < S; ++k) frag[k % RING] = load_row(k + RING);
+    __builtin_amdgcn_sched_barrier(0);
+
     for (int rb = 0; rb < rps; rb += U) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int oy = oy0 + rb + u;
-            v4i acc = {0, 0, 0, 0};
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, frag[(u * S + 0) % RING], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, frag[(u * S + 1) % RING], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, frag[(u * S + 2) % RING], acc, 0, 0, 0);
-            // the S oldest rows are dead now: refill their slots with the rows one ring ahead
+            const int r = rb + u;  // output row of the strip whose epilogue runs in this step
+            // row r+1: its input rows start (r+1)*S rows into the strip; the ring phase repeats every U rows
+            row_mfma((u + 1) % U, nxt);
 #pragma unroll
-            for (int k = 0; k < S; ++k) frag[(u * S + k) % RING] = load_row((rb + u) * S + k + RING);
-            const bool row_ok = oy < g.OH && rb + u < rps;  // rows past the strip / image are dropped
+            for (int k = 0; k < S; ++k) frag[((u + 1) * S + k) % RING] = load_row((r + 1) * S + k + RING);
+            const int oy = oy0 + r;
+            const bool row_ok = oy < g.OH && r < rps;  // rows past the strip / image are dropped
             const unsigned s_row = row_ok ? s_out + (unsigned)oy * row_bytes : 0u;
             const unsigned v_o = row_ok ? v_out : DW_OOB;
             if constexpr (EPI == EPI_F32_P4) {
-                v4i res;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v = __fmaf_rn((float)acc[e], __int_as_float(si4[e]), __int_as_float(bi4[e]));
-                    v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
-                    res[e] = __float_as_int(v);
+                for (int t = 0; t < T; ++t) {
+                    const v4i res = dw_dequant4(ep, cur[t], si[t], bi[t]);
+                    // the second set's channels 4..7 are the next Float4 pack: one plane further
+                    const unsigned vo_t = (t == 0 || !row_ok) ? v_o : v_o + OHW * 16u;
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, res), rout, (int)vo_t, (int)s_row, 0);
                 }
-                __builtin_amdgcn_raw_buffer_store_b128(
-                    __builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, res), rout, (int)v_o,
-                    (int)s_row, 0);
             } else {
                 constexpr bool NONNEG = EPI == EPI_I8_P8_NONNEG;
-                int qv[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v = __fmaf_rn((float)acc[e], __int_as_float(si4[e]), __int_as_float(bi4[e]));
-                    v = __builtin_amdgcn_fmed3f(v, ep.act_lo, ep.act_hi);
-                    v = __fmul_rn(v, __int_as_float(so4[e]));
-                    const float adj =
-                        NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
-                    qv[e] = (int)adj;  // toward zero, saturating
+                if constexpr (S == 1) {
+                    v2i w2;
+                    w2[0] = (int)dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                    w2[1] = (int)dw_requant4<NONNEG>(ep, cur[T - 1], si[T - 1], bi[T - 1], so[T - 1], qh[T - 1][0], qh[T - 1][1]);
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, w2), rout, (int)v_o, (int)s_row, 0);
+                } else {
+                    const unsigned w1 = dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                    __builtin_amdgcn_raw_buffer_store_b32(w1, rout, (int)v_o, (int)s_row, 0);
                 }
-                ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[0], qv[1]));
-                ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[2], qv[3]));
-                const ohip_v2s top = {127, 127}, bot = {-127, -127};
-                lo = __builtin_elementwise_min(lo, top);
-                hi = __builtin_elementwise_min(hi, top);
-                if (!NONNEG) {
-                    lo = __builtin_elementwise_max(lo, bot);
-                    hi = __builtin_elementwise_max(hi, bot);
-                }
-                const unsigned word =
-                    __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
-                __builtin_amdgcn_raw_buffer_store_b32(word, rout, (int)v_o, (int)s_row, 0);
             }
+#pragma unroll
+            for (int t = 0; t < T; ++t) cur[t] = nxt[t];
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
 
 // true when this layer / batch can take the matrix-core kernel (the caller falls back to the vector kernels otherwise)
-bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi) {
+bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive) {
+    if (epi == EPI_I8_P8_NONNEG && !scale_out_positive) return false;  // the clamp is moved past the output scale
     if (!(g.kh == 3 && g.kw == 3 && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2))) return false;
     if (g.ph > 1 || g.pw > 1 || g.C % 8 != 0 || g.C != g.K) return false;
     if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4) return false;
@@ -188,28 +282,41 @@ bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi) {
 hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
                             int strip_blocks, hipStream_t stream) {
     if (g.N == 0 || g.OH * g.OW == 0) return hipSuccess;
-    const int G16 = (g.C / 8 + 1) / 2;
-    const int col_chunks = (g.OW + 15) / 16;
-    const int ipw = g.OW <= 8 ? std::min(16 / g.OW, g.N) : 1;
-    const long groups = (long)((g.N + ipw - 1) / ipw) * G16;
+    const int C8 = g.C / 8;
+    const int PH = 4 / g.sh;  // output pixels per lane column
+    // lane columns an image row needs
+    const int cols = (g.OW + PH - 1) / PH;
+    int lpi = 16, ipw = 1, col_chunks = (cols + 15) / 16;
+    if (cols <= 8) {  // narrow images side by side in one wave
+        lpi = cols;
+        ipw = std::min(16 / lpi, g.N);
+        col_chunks = 1;
+    }
+    const long groups = (long)((g.N + ipw - 1) / ipw) * C8;
     if (groups > 65535) return hipErrorInvalidValue;  // grid.y limit; the caller splits the batch
     // strip height in steps of U = 8/stride output rows: the tallest strip (setup and halo rows amortised over the
-    // longest walk) that still leaves about four waves per SIMD
+    // longest walk) that still leaves about two waves per SIMD (measured: fewer, longer waves win)
     const int U = 8 / g.sh;
     const int blocks_total = (g.OH + U - 1) / U;
     int k = blocks_total;
     if (strip_blocks > 0) k = std::min(strip_blocks, blocks_total);
     else
-        while (k > 1 && (long)col_chunks * ((blocks_total + k - 1) / k) * groups < 4096) --k;
+        while (k > 1 && (long)col_chunks * ((blocks_total + k - 1) / k) * groups < 2048) --k;
     const int rps = k * U;
     const int n_strips = (g.OH + rps - 1) / rps;
     const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
     const dim3 grid((unsigned)(col_chunks * (n_strips / wpb)), (unsigned)groups), block(64 * wpb);
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1));
-#define OHIP_DWM(S_, E_)                                                                                               \
-    hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_>), grid, block, 0, stream, x, wa, out, g, ep, n_strips, rps, col_chunks, \
-                       ipw, in_bytes, out_bytes)
+#define OHIP_DWM(S_, E_) \
+    do {                                                                                                               \
+        if (g.W & 1)                                                                                                   \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, true>), grid, block, 0, stream, x, wa, out, g, ep, n_strips, \
+                               rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
+        else                                                                                                           \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, false>), grid, block, 0, stream, x, wa, out, g, ep, n_strips, \
+                               rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
+    } while (0)
 #define OHIP_DWM_E(S_)                                                \
     do {                                                              \
         if (epi == EPI_I8_P8_NONNEG) OHIP_DWM(S_, EPI_I8_P8_NONNEG);  \

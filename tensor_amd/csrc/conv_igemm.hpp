@@ -24,9 +24,9 @@ hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void*
                            const Epilogue& ep, hipStream_t stream);
 
 // conv_dw.hip
-size_t dw_mfma_weight_bytes(int C);
-void dw_mfma_pack_weights(const int8_t* w, int C, int8_t* dst);
-bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi);
+size_t dw_mfma_weight_bytes(int C, int stride);
+void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t* dst);
+bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
                             int strip_shift, hipStream_t stream);
 size_t dw_packed_weight_bytes(int C, int kh, int kw);

@@ -273,26 +273,38 @@ static ConvGeom make_geom(const otter_hip_conv_desc& d, int n, int in_h, int in_
     return g;
 }
 
+static Epilogue make_epilogue(const otter_hip_conv* h, int out_layout) {
+    const otter_hip_conv_desc& d = h->d;
+    Epilogue ep;
+    ep.scale_in = h->scale_in, ep.bias = h->bias, ep.scale_out = h->scale_out;
+    ep.act = d.activation_type, ep.act_p0 = d.activation_param0, ep.round_mode = d.out_round_mode;
+    ep.out_kind = d.out_kind, ep.out_layout = out_layout;
+    ep.act_lo = (d.activation_type == 1 || d.activation_type == 3) ? 0.f : -__builtin_inff();
+    ep.act_hi = d.activation_type == 3 ? 6.f : __builtin_inff();
+    ep.round_half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    return ep;
+}
+
 // 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS
-static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g) {
+static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g, const Epilogue& ep) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
         if (h->w_igemm) {
             if (h->force_tm > 0) return 1;
-            if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g)) return 3;
+            if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g, ep)) return 3;
             return 1;
         }
     }
     return 0;
 }
 
-int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int) {
+int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int out_layout) {
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
     if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
     ConvGeom g = make_geom(h->d, n, in_h, in_w);
     if (h->c_pad) l = OTTER_HIP_I8_P8, g.C = h->c_pad;
-    return pick_kernel(h, l, g);
+    return pick_kernel(h, l, g, make_epilogue(h, out_layout));
 }
 
 int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
@@ -342,16 +354,10 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         xq = (const int8_t*)workspace;
     }
 
-    Epilogue ep;
-    ep.scale_in = h->scale_in, ep.bias = h->bias, ep.scale_out = h->scale_out;
-    ep.act = d.activation_type, ep.act_p0 = d.activation_param0, ep.round_mode = d.out_round_mode;
-    ep.out_kind = d.out_kind, ep.out_layout = out_layout;
-    ep.act_lo = (d.activation_type == 1 || d.activation_type == 3) ? 0.f : -__builtin_inff();
-    ep.act_hi = d.activation_type == 3 ? 6.f : __builtin_inff();
-    ep.round_half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    const Epilogue ep = make_epilogue(h, out_layout);
 
     // (2)+(3)+(4) convolution with the fused epilogue
-    switch (pick_kernel(h, q_layout, g)) {
+    switch (pick_kernel(h, q_layout, g, ep)) {
     case 3:
         OHIP_CHECK(run_conv3x3_halo(xq, h->w_igemm, out, g, ep, h->force_tm < 0 ? h->force_tn : 0, stream));
         break;
@@ -374,7 +380,8 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         break;
     }
     case 1:
-        OHIP_CHECK(run_conv_igemm(xq, h->w_igemm, out, g, ep, h->force_tm, h->force_tn, stream));
+        OHIP_CHECK(run_conv_igemm(xq, h->w_igemm, out, g, ep, h->force_tm > 0 ? h->force_tm : 0,
+                                  h->force_tm > 0 ? h->force_tn : 0, stream));
         break;
     default:
         OHIP_CHECK(run_conv_direct(xq, layout_pack(q_layout), h->w_raw, out, g, ep, stream));

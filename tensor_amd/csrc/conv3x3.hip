@@ -1,19 +1,23 @@
 // Dense int8 3x3 stride-1 convolution on the gfx950 matrix cores with the input halo resident in LDS.
 //
 // A workgroup owns a run of PT consecutive output pixels of one image (row-major, so a few whole output rows)
-// and a block of output channels. The input rows that run touches (+1 halo row above and below, +1 zero column
-// left and right) are staged into LDS ONCE, as [channel pair-of-octets][row][column][16 bytes]; after that the
-// nine filter taps are nine shifted views of the same LDS tile, so every input byte is fetched from memory once
-// per workgroup instead of nine times, and the main loop has no barrier at all:
-//   * the MFMA "B" operand (16 input channels of one pixel) is one ds_read_b128 per lane, conflict-free because
-//     the 16 lanes of a row group read 16 consecutive pixels = 256 consecutive bytes;
+// and a block of output channels. The input rows that run touches (+1 halo row above and below, +2 zero columns
+// left and right) are staged into LDS ONCE, as [octet pair][row][octet of the pair][PITCH bytes of 8-byte pixels] -
+// image rows as they lie in the Byte8 tensor, on a power-of-two pitch - so every input byte is fetched from memory
+// once per workgroup instead of nine times, the nine filter taps are nine shifted views of the same LDS tile at
+// compile-time offsets from one address register per fragment, and the main loop has no barrier at all:
+//   * staging is done by the LDS-DMA path (buffer_load_dwordx4 ... lds): one instruction moves one image row of one
+//     octet, 16 bytes = two pixels per lane, global memory -> LDS without passing through registers. Padding costs
+//     nothing: lanes on the zero columns and rows outside the image carry an out-of-range buffer offset, for which
+//     the hardware writes zeros. The transfer for the NEXT tile is issued as soon as the last matrix instruction of
+//     this tile has read LDS, so it runs under the epilogue;
+//   * the MFMA "B" operand (16 input channels of one pixel) is two ds_read_b64 per lane (the two octets),
+//     conflict-free because the 16 lanes of a row group read 16 consecutive pixels = 128 consecutive bytes;
 //   * the MFMA "A" operand (weights) is read straight from global memory, already in MFMA lane order
-//     (igemm_pack_weights), one coalesced 1 KB read per 16x64 fragment, prefetched one k-chunk ahead. Every
+//     (igemm_pack_weights), one coalesced 1 KB read per 16x64 fragment, prefetched two k-chunks ahead. Every
 //     workgroup reads the same <= 147 KB of weights, so they stay in L2.
-// Zero padding costs nothing: the halo columns / out-of-image rows are written as zeros while staging.
+// The image width must be even (a lane moves an aligned pixel pair) and the input below 2 GiB (32-bit offsets).
 #include "common.hpp"
-#include <cstdlib>
-
 #include "conv_igemm.hpp"
 
 namespace ohip {
@@ -21,23 +25,28 @@ namespace ohip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
-template <int FM, int FN, int WM, int WN, int EPI>
+constexpr unsigned HALO_OOB = 0x80000000u;  // beyond the buffer descriptor: reads as zero
+
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
 __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                            void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
-                                                           int c_groups, int r_max, int cb, int tiles_per_img, int prm_ofs, int total_tiles,
-                                                           int stagger) {
+                                                           int c_groups, int r_max, int cb, int tiles_per_img, int prm_ofs,
+                                                           int total_tiles, unsigned in_bytes) {
     static_assert(WM * WN == 4 && FM % 2 == 0, "four waves, row fragments in pairs");
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     constexpr int PT = WN * FN * 16;
+    constexpr int PITCH = 1 << LOGP;  // bytes per (octet, row) line in LDS; holds pixels -2 .. W+1
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
 
     const int mt_base = blockIdx.y * (WM * FM) + wm * FM;  // first 16-row tile of this wave
     const int OHW = g.OH * g.OW;
     const int C8 = g.C / 8;
+    const int EW = g.W + 4;                  // pixels -2 .. W+1 of a row, 8 bytes each (EW * 8 <= PITCH)
+    const int pair_bytes = r_max * 2 * PITCH;  // LDS bytes between octet pairs
     // The per-channel epilogue constants of this workgroup's row block go to LDS now (behind the halo tile), so
     // that the epilogue does not end on a chain of global-memory round trips.
     constexpr int ROWS = WM * FM * 16;
@@ -48,35 +57,83 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
         lds_prm[i] = src ? src[c] : 1.f;
     }
 
-    // Persistent workgroups: the grid holds at most two workgroups per CU and each walks over tiles. The
-    // workgroups in the second residency slot of a CU start `stagger` sleeps late, so that for the rest of the
-    // kernel one workgroup's staging / epilogue (memory latency, VALU) runs under the other's MFMA phase instead
-    // of both doing the same thing at the same time.
-    if (stagger > 0 && ((blockIdx.x >> 8) & 1))
-        for (int i = 0; i < stagger; ++i) __builtin_amdgcn_s_sleep(32);
-    for (int wg0 = blockIdx.x; wg0 < total_tiles; wg0 += gridDim.x) {
-        // consecutive tiles (which share halo rows) go to the same XCD / L2
+    const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x), 0, (int)in_bytes, 0x00020000);
+
+    // tile index -> (image, first pixel); consecutive tiles (which share halo rows) go to the same XCD / L2
+    auto tile_of = [&](int wg0, int& n, int& p0) {
         int wg = wg0;
-        {
-            const int per = total_tiles / 8;
-            if (per > 0 && wg < per * 8) wg = (wg % 8) * per + wg / 8;
-        }
-        const int n = wg / tiles_per_img;
-        const int t = wg % tiles_per_img;
-        const int8_t* xn = x + (size_t)n * C8 * g.H * g.W * 8;
-        const int p0 = t * PT;
+        const int per = total_tiles / 8;
+        if (per > 0 && wg < per * 8) wg = (wg % 8) * per + wg / 8;
+        n = wg / tiles_per_img;
+        p0 = (wg % tiles_per_img) * PT;
+    };
+    // Issue the LDS-DMA transfers of one (tile, channel block): this wave moves octets wave, wave+4, ...
+    auto stage = [&](int n, int p0, int cb0) {
         const int p_last = min(p0 + PT, OHW) - 1;
         const int r_lo = p0 / g.OW;
         const int R = p_last / g.OW - r_lo + 3;
-        const int cols = g.W + 2;
-        const int plane = r_max * cols * 16;  // bytes between channel pairs
+        if constexpr (LOGP == 9) {
+            // 512-byte lines: one instruction moves a row of BOTH octets of a pair (adjacent lines in LDS): lanes 0-31
+            // the first octet, lanes 32-63 the second, 16 bytes = pixels 2*pp-2 and 2*pp-1 each
+            const int hl = lane >> 5, pp = lane & 31;
+            const bool col_ok = pp >= 1 && 2 * pp - 1 < g.W;
+            const unsigned v_px = (unsigned)(2 * pp - 2) * 8u;
+            const unsigned v_both = col_ok ? v_px + (unsigned)hl * (unsigned)(g.H * g.W * 8) : HALO_OOB;
+            const unsigned v_first = (col_ok && hl == 0) ? v_px : HALO_OOB;  // an odd octet count ends on half a pair
+            if (2 * pp < EW) {
+                for (int pj = wave; pj < cb / 16; pj += 4) {
+                    const int o = cb0 / 8 + 2 * pj;
+                    const bool both = o + 1 < C8;
+                    for (int r = 0; r < R; ++r) {
+                        const int iy = r_lo - g.ph + r;
+                        const bool ok = o < C8 && iy >= 0 && iy < g.H;  // wave-uniform
+                        const unsigned s_off = ok ? (unsigned)((n * C8 + o) * g.H + iy) * (unsigned)(g.W * 8) : 0u;
+                        int8_t* dst = lds + (size_t)pj * pair_bytes + (size_t)((2 * r) << LOGP);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, (__attribute__((address_space(3))) void*)dst, 16,
+                                                                 (int)(ok ? (both ? v_both : v_first) : HALO_OOB), (int)s_off,
+                                                                 0, 0);
+                    }
+                }
+            }
+        } else {
+            const bool col_ok = lane >= 1 && 2 * lane - 1 < g.W;  // lane: pixels 2*lane-2 and 2*lane-1
+            const unsigned v_col = col_ok ? (unsigned)(2 * lane - 2) * 8u : HALO_OOB;
+            if (2 * lane < EW) {
+                for (int oc = wave; oc < cb / 8; oc += 4) {
+                    const int o = cb0 / 8 + oc;
+                    for (int r = 0; r < R; ++r) {
+                        const int iy = r_lo - g.ph + r;
+                        const bool ok = o < C8 && iy >= 0 && iy < g.H;  // wave-uniform
+                        const unsigned s_off = ok ? (unsigned)((n * C8 + o) * g.H + iy) * (unsigned)(g.W * 8) : 0u;
+                        int8_t* dst = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((2 * r + (oc & 1)) << LOGP);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, (__attribute__((address_space(3))) void*)dst, 16,
+                                                                 (int)(ok ? v_col : HALO_OOB), (int)s_off, 0, 0);
+                    }
+                }
+            }
+        }
+    };
 
-        int bofs[FN];
+    int n, p0;
+    if ((int)blockIdx.x < total_tiles) {
+        tile_of(blockIdx.x, n, p0);
+        stage(n, p0, 0);
+    }
+
+    // Persistent workgroups: the grid holds at most two workgroups per CU and each walks over tiles.
+    for (int wg0 = blockIdx.x; wg0 < total_tiles; wg0 += gridDim.x) {
+        tile_of(wg0, n, p0);
+        const int r_lo = p0 / g.OW;
+
+        // LDS address of this lane's pixel (tap 0,0) per fragment, octet pair lane/16 of the current k-chunk; walks
+        // forward by one chunk after the ninth tap and is wound back at the end of a stage
+        // (kept as LDS byte offsets: a generic pointer here would turn the ds_read into a flat load)
+        int bcc[FN];
 #pragma unroll
         for (int f = 0; f < FN; ++f) {
             const int pix = min(p0 + (wn * FN + f) * 16 + (lane & 15), OHW - 1);
             const int oy = pix / g.OW, ox = pix % g.OW;
-            bofs[f] = (oy - r_lo) * cols + ox + 1 - g.pw + (lane >> 4) * (plane / 16);  // in 16-byte units
+            bcc[f] = (oy - r_lo) * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
         }
 
         v4i acc[FM][FN];
@@ -90,76 +147,77 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
         const size_t kc_stride = (size_t)m_tiles16 * 1024;
 
         for (int cb0 = 0; cb0 < c_groups * 64; cb0 += cb) {
-            __syncthreads();  // everyone is done reading the previous channel block
-            // Stage the halo: one wave per (channel pair, row) line, lanes along the columns, so that the only
-            // divisions are wave-uniform (scalar) and a wave reads 2 x 512 contiguous bytes per line. Lines are taken
-            // in batches of SB with all loads of a batch issued before the first LDS write, so a batch costs one
-            // memory round trip.
-            {
-                constexpr int SB = 12;
-                const int lines = (cb / 16) * R;
-                for (int xc0 = 0; xc0 < cols; xc0 += 64) {
-                    const int xc = xc0 + lane;
-                    const int ix = xc - 1;
-                    const bool col_ok = ix >= 0 && ix < g.W;
-                    for (int l0 = wave; l0 < lines; l0 += 4 * SB) {
-                        v2i lo[SB], hi[SB];
-#pragma unroll
-                        for (int k = 0; k < SB; ++k) {
-                            const int line = min(l0 + 4 * k, lines - 1);
-                            const int j = line / R, r = line - j * R;
-                            const int iy = r_lo - g.ph + r;
-                            const int o0 = cb0 / 8 + 2 * j;
-                            const bool ok = col_ok && iy >= 0 && iy < g.H;
-                            const int8_t* px = xn + ((size_t)iy * g.W + ix) * 8;
-                            lo[k] = (ok && o0 < C8) ? *reinterpret_cast<const v2i*>(px + (size_t)o0 * g.H * g.W * 8) : v2i{0, 0};
-                            hi[k] = (ok && o0 + 1 < C8) ? *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * g.H * g.W * 8)
-                                                        : v2i{0, 0};
-                        }
-#pragma unroll
-                        for (int k = 0; k < SB; ++k) {
-                            const int line = l0 + 4 * k;
-                            const int j = line / R, r = line - j * R;
-                            if (line < lines && xc < cols)
-                                *reinterpret_cast<v4i*>(lds + (size_t)j * plane + ((size_t)r * cols + xc) * 16) =
-                                    v4i{lo[k][0], lo[k][1], hi[k][0], hi[k][1]};
-                        }
-                    }
-                }
-            }
-            __syncthreads();
-
             // Main loop: no barrier, no branch. The nine taps are unrolled; weight fragments travel through a ring of
             // three register stages and are requested two k-chunks (~0.4 us of MFMA work) before use. Every load is
             // unconditional (the weight rows are padded to whole row blocks and the chunk index is clamped), so that
             // the compiler can count outstanding loads and wait only for the oldest stage.
-            v4i ring[3][FM];
+            constexpr int RD = FN >= 7 ? 2 : 3;  // weight ring depth: the widest tile has registers for two stages only
+            v4i ring[RD][FM];
             const int cg0 = cb0 / 64;
+            auto a_ptr = [&](int cc, int tap) { return wlane + (size_t)(tap * c_groups + cg0 + cc) * kc_stride; };
             auto load_a = [&](int cc, int tap, v4i (&a)[FM]) {
-                const int8_t* p = wlane + (size_t)(tap * c_groups + cg0 + cc) * kc_stride;
+                const int8_t* p = a_ptr(cc, tap);
 #pragma unroll
                 for (int i = 0; i < FM; ++i) a[i] = *reinterpret_cast<const v4i*>(p + i * 1024);
             };
+            typedef __attribute__((address_space(3))) const int8_t* lds_cptr;
+            typedef __attribute__((address_space(3))) const v2i* lds_v2i;
+            const lds_cptr lds3 = (lds_cptr)lds;
+            auto read_b = [&](int off) {
+                const v2i lo = *(lds_v2i)(lds3 + off);
+                const v2i hi = *(lds_v2i)(lds3 + off + PITCH);
+                return v4i{lo[0], lo[1], hi[0], hi[1]};
+            };
+            // the halo transfers of this stage were issued one stage ago: wait for this wave's, then for everyone's
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
             load_a(0, 0, ring[0]);
-            load_a(0, 1, ring[1]);
+            if constexpr (RD == 3) load_a(0, 1, ring[1]);
+            v4i b[FN];
+#pragma unroll
+            for (int f = 0; f < FN; ++f) b[f] = read_b(bcc[f]);
+            // The schedule is written out by hand, one group per pixel fragment: the FM matrix instructions that use
+            // b[f], then the LDS read that refills b[f] for the NEXT tap (in place: its last reader has just issued),
+            // then one weight-fragment load for the tap after next. Every operand is requested several hundred
+            // cycles before its use and no extra registers are needed; the barriers pin the order.
             for (int cc = 0; cc < nck; ++cc) {
                 const int cc_next = min(cc + 1, nck - 1);
-                const int ccofs = cc * 4 * (plane / 16);
+                const int to_next = (cc_next - cc) * 4 * pair_bytes;  // the last chunk re-reads itself: unused data
 #pragma unroll
                 for (int tap = 0; tap < 9; ++tap) {
-                    if (tap + 2 < 9) load_a(cc, tap + 2, ring[(tap + 2) % 3]);
-                    else load_a(cc_next, tap + 2 - 9, ring[(tap + 2) % 3]);
-                    const int tapofs = (tap / 3) * cols + tap % 3 + ccofs;  // 16-byte units: keeps ds_read_b128
-                    v4i b[FN];
+                    constexpr int AH = RD - 1;  // taps ahead
+                    const int8_t* pa = tap + AH < 9 ? a_ptr(cc, tap + AH) : a_ptr(cc_next, tap + AH - 9);
+                    constexpr int kRowB = 2 * PITCH;
+                    const int nofs = tap < 8 ? ((tap + 1) / 3) * kRowB + ((tap + 1) % 3) * 8 : 0;  // compile-time
 #pragma unroll
-                    for (int f = 0; f < FN; ++f) b[f] = reinterpret_cast<const v4i*>(lds)[bofs[f] + tapofs];
+                    for (int f = 0; f < FN; ++f) {
 #pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int f = 0; f < FN; ++f)
-                            acc[i][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[tap % 3][i], b[f], acc[i][f], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);  // keep the prefetch distance: no hoisting of later taps' loads
+                        for (int i = 0; i < FM; ++i)
+                            acc[i][f] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ring[tap % RD][i], b[f], acc[i][f], 0, 0, 0);
+                        if (tap == 8) bcc[f] += to_next;
+                        b[f] = read_b(bcc[f] + nofs);
+                        if (f < FM) ring[(tap + AH) % RD][f] = *reinterpret_cast<const v4i*>(pa + f * 1024);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
+                if constexpr (RD == 2) {
+                    // nine taps flip the parity of a two-stage ring: move the fragments just requested (next chunk,
+                    // tap 0) to the stage tap 0 reads
+#pragma unroll
+                    for (int i = 0; i < FM; ++i) ring[0][i] = ring[1][i];
+                }
+            }
+#pragma unroll
+            for (int f = 0; f < FN; ++f) bcc[f] -= (nck - 1) * 4 * pair_bytes;
+            __syncthreads();  // everyone is done reading this stage: its LDS may be overwritten
+            // next stage = next channel block of this tile, or the first block of this workgroup's next tile: its
+            // transfers run under the rest of this tile's work (the epilogue, for the last block)
+            if (cb0 + cb < c_groups * 64) {
+                stage(n, p0, cb0 + cb);
+            } else if (wg0 + (int)gridDim.x < total_tiles) {
+                int n2, p2;
+                tile_of(wg0 + gridDim.x, n2, p2);
+                stage(n2, p2, 0);
             }
         }
 
@@ -218,7 +276,7 @@ constexpr int kMaxLdsBytes = 64 * 1024;  // halo tile per workgroup: leaves room
 constexpr int kPrmLdsBytes = 3 * 128 * 4 + 16;  // epilogue constants behind it
 
 struct HaloPlan {
-    int fn, r_max, cb, tiles_per_img;
+    int fn, r_max, cb, tiles_per_img, logp;
     size_t lds_bytes;
     double cost;
 };
@@ -234,10 +292,10 @@ int halo_rows(int pt, int OW, int OHW) {
     return worst;
 }
 
-template <int FM, int FN, int WM, int WN, int EPI>
-hipError_t launch_halo_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
+hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                          const HaloPlan& pl, hipStream_t stream) {
-    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI>;
+    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI, LOGP>;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -252,13 +310,18 @@ hipError_t launch_halo_e(const int8_t* x, const int8_t* wpk, void* out, const Co
     int grid_x = 512 / m_blocks;  // two resident workgroups per CU
     if (grid_x < 8) grid_x = 8;
     if (grid_x > total_tiles) grid_x = total_tiles;
-    // stagger only pays when every slot has at least two tiles to walk through
-    static const char* env = getenv("OHIP_HALO_STAGGER");
-    const int stagger = env ? atoi(env) : 0;
+    const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     hipLaunchKernelGGL(kern, dim3(grid_x, m_blocks), dim3(256), prm_ofs + 3 * WM * FM * 16 * sizeof(float), stream, x, wpk,
                        out, g, ep, mpad / 16, igemm_channel_groups(g.C), pl.r_max, pl.cb, pl.tiles_per_img, prm_ofs,
-                       total_tiles, (grid_x == 512 / m_blocks && grid_x >= 512) ? stagger : 0);
+                       total_tiles, in_bytes);
     return hipGetLastError();
+}
+
+template <int FM, int FN, int WM, int WN, int EPI>
+hipError_t launch_halo_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                         const HaloPlan& pl, hipStream_t stream) {
+    if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9>(x, wpk, out, g, ep, pl, stream);
+    return launch_halo_p<FM, FN, WM, WN, EPI, 10>(x, wpk, out, g, ep, pl, stream);
 }
 
 template <int FM, int FN, int WM, int WN>
@@ -272,7 +335,7 @@ hipError_t launch_halo(const int8_t* x, const int8_t* wpk, void* out, const Conv
     case EPI_F32_P4:
         return launch_halo_e<FM, FN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, pl, stream);
     default:
-        return launch_halo_e<FM, FN, WM, WN, EPI_GENERIC>(x, wpk, out, g, ep, pl, stream);
+        return hipErrorInvalidValue;  // other epilogues take the generic implicit-GEMM kernel
     }
 }
 
@@ -284,20 +347,24 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
     const int cpad = igemm_channel_groups(g.C) * 64;
     const bool wide = igemm_padded_rows(g.K) > 64;
     const int m_blocks = wide ? (igemm_padded_rows(g.K) / 16 + 7) / 8 : 1;
+    // LDS line pitch: 512 bytes hold rows of up to 60 pixels (+4 padding pixels), 1024 bytes up to 124
+    const int logp = (g.W + 4) * 8 <= 512 ? 9 : 10;
+    if ((g.W + 4) * 8 > (1 << logp)) return false;
     bool found = false;
     for (int fn = 4; fn <= 7; ++fn) {  // 8 fragments would spill at two waves per SIMD
         if (force_fn && fn != force_fn) continue;
         const int pt = (wide ? 32 : 64) * fn;
         HaloPlan p;
         p.fn = fn;
+        p.logp = logp;
         p.r_max = halo_rows(pt, g.OW, OHW);
-        const size_t per64 = (size_t)64 * p.r_max * (g.W + 2);
+        const size_t per64 = (size_t)8 * p.r_max << logp;  // 64 channels = 8 octets
         if (per64 > (size_t)kMaxLdsBytes) continue;
         int cb = (int)(kMaxLdsBytes / per64) * 64;
         if (cb > cpad) cb = cpad;
         while (cpad % cb) cb -= 64;  // equal channel blocks
         p.cb = cb;
-        p.lds_bytes = (size_t)cb * p.r_max * (g.W + 2);
+        p.lds_bytes = (size_t)(cb / 8) * p.r_max << logp;
         p.tiles_per_img = (OHW + pt - 1) / pt;
         const long wgs = (long)g.N * p.tiles_per_img * m_blocks;
         const long slots = 512;
@@ -314,9 +381,11 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
 
 }  // namespace
 
-bool conv3x3_halo_supported(const ConvGeom& g) {
+bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep) {
     if (!(g.kh == 3 && g.kw == 3 && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.groups == 1)) return false;
     if (g.ph > 1 || g.pw > 1 || g.C % 8) return false;
+    if ((g.W & 1) || (size_t)g.N * g.C * g.H * g.W >= ((size_t)1 << 31)) return false;  // pixel pairs, 32-bit offsets
+    if (pick_epilogue(ep, g.K) == EPI_GENERIC) return false;
     HaloPlan p;
     return plan_halo(g, 0, &p);
 }
@@ -324,7 +393,8 @@ bool conv3x3_halo_supported(const ConvGeom& g) {
 hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                             int force_fn, hipStream_t stream) {
     HaloPlan p;
-    if (!plan_halo(g, force_fn, &p)) return hipErrorInvalidValue;
+    // a forced fragment count that does not fit LDS falls back to the automatic choice
+    if (!plan_halo(g, force_fn, &p) && !plan_halo(g, 0, &p)) return hipErrorInvalidValue;
     const bool wide = igemm_padded_rows(g.K) > 64;
 #define OHIP_HALO(FN_)                                                                  \
     case FN_:                                                                           \

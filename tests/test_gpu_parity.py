@@ -188,11 +188,13 @@ def test_igemm_every_tile_shape(hip, oracle, tile):
 
 @pytest.mark.parametrize("fn", [4, 5, 6, 7])
 def test_halo3x3_every_fragment_count(hip, oracle, fn):
-    """The 3x3 stride-1 LDS-halo MFMA kernel: wide (K > 64) and narrow wave layouts, padded channel counts,
-    pad 0 and 1, ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at once)."""
+    """The 3x3 stride-1 LDS-halo MFMA kernel (even image widths): wide (K > 64) and narrow wave layouts, padded
+    channel counts, pad 0 and 1, ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at
+    once), both LDS line pitches (up to 60 columns and up to 124), several tiles per workgroup."""
     rng = np.random.default_rng(fn)
-    for (C, K, p, N, H, W) in [(128, 128, 1, 2, 19, 23), (64, 64, 1, 1, 56, 56), (72, 24, 0, 2, 11, 9),
-                               (16, 160, 1, 1, 7, 7), (320, 96, 1, 1, 14, 30)]:
+    for (C, K, p, N, H, W) in [(128, 128, 1, 2, 19, 22), (64, 64, 1, 1, 56, 56), (72, 24, 0, 2, 11, 10),
+                               (16, 160, 1, 1, 7, 8), (320, 96, 1, 1, 14, 30), (8, 16, 1, 1, 9, 66),
+                               (16, 136, 1, 3, 5, 124)]:
         x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
         in_scale = 25.0
         for int8_out in (True, False):
@@ -205,7 +207,9 @@ def test_halo3x3_every_fragment_count(hip, oracle, fn):
                 np.testing.assert_array_equal(out, want)
             else:
                 assert_f32_close(out, want)
-        acc, _ = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, out_kind=capi.OUT_I32, tile=(-1, fn))
+        # odd widths and raw accumulators take the generic implicit-GEMM kernel
+        acc, kind = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, out_kind=capi.OUT_I32, tile=(-1, fn))
+        assert kind == 1
         np.testing.assert_array_equal(acc, acc_want)
 
 

@@ -282,6 +282,7 @@ static Epilogue make_epilogue(const otter_hip_conv* h, int out_layout) {
     ep.act_lo = (d.activation_type == 1 || d.activation_type == 3) ? 0.f : -__builtin_inff();
     ep.act_hi = d.activation_type == 3 ? 6.f : __builtin_inff();
     ep.round_half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    ep.so_positive = h->so_positive;
     return ep;
 }
 

@@ -112,6 +112,7 @@ struct Epilogue {
     // fast epilogues (activation none / ReLU / clip[0,6] as one clamp, rounding mode as one constant)
     float act_lo, act_hi;  // v = min(max(v, act_lo), act_hi)
     float round_half;      // 0.5f (ROUND_SSE) or 0.49999997f (ROUND_EXACT)
+    bool so_positive;      // every output scale is finite and > 0 (lets the int8 epilogue clamp after rounding)
 };
 
 // which epilogue code a kernel instance carries
@@ -121,8 +122,11 @@ enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3 };
 // or (F32_P4) fp32 output in Float4 with K % 4 == 0.
 __host__ inline int pick_epilogue(const Epilogue& ep, int K) {
     const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3;
-    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0)
-        return ep.act != 0 ? EPI_I8_P8_NONNEG : EPI_I8_P8;  // after ReLU / clip the value to round is never negative
+    if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0) {
+        if (ep.act == 0) return EPI_I8_P8;
+        // after ReLU / clip the value to round is never negative; the fast path needs positive output scales
+        return ep.so_positive ? EPI_I8_P8_NONNEG : EPI_GENERIC;
+    }
     if (clamp_act && ep.out_kind == OTTER_HIP_OUT_F32 && ep.out_layout == OTTER_HIP_F32_P4 && K % 4 == 0) return EPI_F32_P4;
     return EPI_GENERIC;
 }
@@ -216,7 +220,10 @@ __device__ __noinline__ void epilogue_store8_generic(void* __restrict__ out, con
 // (filled with -0.0f when the layer has no bias: fma(a, s, -0.0f) == a * s bit for bit, sign of zero included).
 struct Epi8 {
     float si[8], bi[8], so[8];
+    unsigned qh[4];  // upper clamp of the rounded result per channel, as packed int16 pairs (epi8_clamp_init)
 };
+
+__device__ __forceinline__ void epi8_clamp_init(const Epilogue& ep, Epi8& p);
 
 template <int EPI>
 __device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) {
@@ -238,13 +245,26 @@ __device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) 
             p.so[e] = __int_as_float(o0[e]);
             p.so[4 + e] = __int_as_float(o1[e]);
         }
+        if constexpr (EPI == EPI_I8_P8_NONNEG) epi8_clamp_init(ep, p);
     }
 }
 
-// requantize 8 channels and store one Byte8 element. NONNEG: the activation clamp has a lower bound of 0, so the
-// value handed to the rounding step is >= 0: copysign(half, v) is just half and only the upper saturation can bind.
-// The median-of-three clamp differs from max/min only in the sign of a zero result, which the rounding discards.
+// requantize 8 channels and store one Byte8 element.
+// NONNEG (ReLU / clip [0, hi], output scales > 0): the clamp is applied AFTER scaling and rounding, on the packed
+// int16 values, instead of on the float before them. x -> trunc(fl(fl(x * so) + half)) is monotone for so > 0, so
+// clamping its argument to [0, hi] equals clamping its result to [trunc(0 + half), trunc(fl(fl(hi * so) + half))]
+// = [0, qh], bit for bit; qh (capped at the int8 saturation bound 127) is computed once per channel octet by
+// epi8_clamp_init. Without an activation (!NONNEG) there is nothing to clamp but the int8 range.
 typedef short ohip_v2s __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void epi8_clamp_init(const Epilogue& ep, Epi8& p) {
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int q0 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, p.so[2 * h]), ep.round_half), 127);
+        const int q1 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, p.so[2 * h + 1]), ep.round_half), 127);
+        p.qh[h] = (unsigned)(q0 & 0xffff) | ((unsigned)q1 << 16);
+    }
+}
 
 template <bool NONNEG>
 __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const Epilogue& ep, const Epi8& p, size_t elem,
@@ -253,7 +273,6 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float v = __fmaf_rn((float)a8[e], p.si[e], p.bi[e]);
-        v = __builtin_amdgcn_fmed3f(v, ep.act_lo, ep.act_hi);
         v = __fmul_rn(v, p.so[e]);
         float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
         q[e] = (int)adj;  // toward zero, saturating
@@ -264,12 +283,14 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
         // two int32 -> two saturated int16 in one dword, clamp both halves at once, then gather the low bytes
         ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h], q[4 * h + 1]));
         ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h + 2], q[4 * h + 3]));
-        const ohip_v2s top = {127, 127}, bot = {-127, -127};
-        lo = __builtin_elementwise_min(lo, top);
-        hi = __builtin_elementwise_min(hi, top);
-        if (!NONNEG) {
-            lo = __builtin_elementwise_max(lo, bot);
-            hi = __builtin_elementwise_max(hi, bot);
+        if (NONNEG) {
+            const ohip_v2s zero = {0, 0};
+            lo = __builtin_elementwise_max(__builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2s, p.qh[2 * h])), zero);
+            hi = __builtin_elementwise_max(__builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2s, p.qh[2 * h + 1])), zero);
+        } else {
+            const ohip_v2s top = {127, 127}, bot = {-127, -127};
+            lo = __builtin_elementwise_max(__builtin_elementwise_min(lo, top), bot);
+            hi = __builtin_elementwise_max(__builtin_elementwise_min(hi, top), bot);
         }
         pk[h] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
     }

@@ -31,7 +31,7 @@ template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
 __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                            void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
                                                            int c_groups, int r_max, int cb, int tiles_per_img, int prm_ofs,
-                                                           int total_tiles, unsigned in_bytes) {
+                                                           int total_tiles, unsigned in_bytes, int tile_inv) {
     static_assert(WM * WN == 4 && FM % 2 == 0, "four waves, row fragments in pairs");
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     constexpr int PT = WN * FN * 16;
@@ -50,7 +50,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
     // The per-channel epilogue constants of this workgroup's row block go to LDS now (behind the halo tile), so
     // that the epilogue does not end on a chain of global-memory round trips.
     constexpr int ROWS = WM * FM * 16;
-    float* lds_prm = reinterpret_cast<float*>(lds + prm_ofs);
+    // (a separate LDS object from the halo tile: the compiler then knows that reading it does not touch what the
+    // LDS-DMA transfers write, and does not make the epilogue wait for the transfers of the next tile)
+    __shared__ __attribute__((aligned(16))) float lds_prm[3 * ROWS];
     for (int i = tid; i < 3 * ROWS; i += 256) {
         const int which = i / ROWS, c = blockIdx.y * ROWS + (i - which * ROWS);
         const float* src = which == 0 ? ep.scale_in : (which == 1 ? ep.bias : ep.scale_out);
@@ -121,19 +123,22 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
     }
 
     // Persistent workgroups: the grid holds at most two workgroups per CU and each walks over tiles.
+    int bcc[FN];
     for (int wg0 = blockIdx.x; wg0 < total_tiles; wg0 += gridDim.x) {
         tile_of(wg0, n, p0);
         const int r_lo = p0 / g.OW;
 
         // LDS address of this lane's pixel (tap 0,0) per fragment, octet pair lane/16 of the current k-chunk; walks
         // forward by one chunk after the ninth tap and is wound back at the end of a stage
-        // (kept as LDS byte offsets: a generic pointer here would turn the ds_read into a flat load)
-        int bcc[FN];
+        // (kept as LDS byte offsets: a generic pointer here would turn the ds_read into a flat load).
+        // When a tile is a whole number of image rows the offsets are the same for every tile: computed once.
+        if (wg0 == (int)blockIdx.x || !tile_inv) {
 #pragma unroll
-        for (int f = 0; f < FN; ++f) {
-            const int pix = min(p0 + (wn * FN + f) * 16 + (lane & 15), OHW - 1);
-            const int oy = pix / g.OW, ox = pix % g.OW;
-            bcc[f] = (oy - r_lo) * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
+            for (int f = 0; f < FN; ++f) {
+                const int pix = min(p0 + (wn * FN + f) * 16 + (lane & 15), OHW - 1);
+                const int oy = pix / g.OW, ox = pix % g.OW;
+                bcc[f] = (oy - r_lo) * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
+            }
         }
 
         v4i acc[FM][FN];
@@ -209,6 +214,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
             }
 #pragma unroll
             for (int f = 0; f < FN; ++f) bcc[f] -= (nck - 1) * 4 * pair_bytes;
+            // drain the (unused) weight fragments requested past the last tap, so that no register has a load pending
+            // when the transfers below are issued: the compiler then needs no memory wait inside the epilogue
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
             __syncthreads();  // everyone is done reading this stage: its LDS may be overwritten
             // next stage = next channel block of this tile, or the first block of this workgroup's next tile: its
             // transfers run under the rest of this tile's work (the epilogue, for the last block)
@@ -229,13 +237,30 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
             const bool ch_ok = ch0 < g.K;
             Epi8 prm;
             if constexpr (EPI != EPI_GENERIC) {
+                // The constants come from LDS through hand-written reads: the compiler would order a ds_read it can
+                // see after the LDS-DMA transfers issued above (they write LDS) by waiting for all of them, which
+                // would put the next tile's halo transfer back on the critical path. The constants live in their own
+                // LDS array, which the transfers never touch.
                 const int cl = ch0 - blockIdx.y * ROWS;  // channel within the row block
+                const unsigned pa = (unsigned)(size_t)(__attribute__((address_space(3))) float*)lds_prm + (unsigned)cl * 4u;
+                v4i r0, r1, r2, r3, r4, r5;
+                asm volatile("ds_read_b128 %0, %1" : "=v"(r0) : "v"(pa));
+                asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(r1) : "v"(pa));
+                asm volatile("ds_read_b128 %0, %1" : "=v"(r2) : "v"(pa + ROWS * 4));
+                asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(r3) : "v"(pa + ROWS * 4));
+                asm volatile("ds_read_b128 %0, %1" : "=v"(r4) : "v"(pa + 2 * ROWS * 4));
+                asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(r5) : "v"(pa + 2 * ROWS * 4));
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3), "+v"(r4), "+v"(r5));
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    prm.si[e] = lds_prm[cl + e];
-                    prm.bi[e] = lds_prm[ROWS + cl + e];
-                    prm.so[e] = lds_prm[2 * ROWS + cl + e];
+                for (int e = 0; e < 4; ++e) {
+                    prm.si[e] = __int_as_float(r0[e]);
+                    prm.si[4 + e] = __int_as_float(r1[e]);
+                    prm.bi[e] = __int_as_float(r2[e]);
+                    prm.bi[4 + e] = __int_as_float(r3[e]);
+                    prm.so[e] = __int_as_float(r4[e]);
+                    prm.so[4 + e] = __int_as_float(r5[e]);
                 }
+                if constexpr (EPI == EPI_I8_P8_NONNEG) epi8_clamp_init(ep, prm);
             }
 #pragma unroll
             for (int f = 0; f < FN; ++f) {
@@ -313,7 +338,7 @@ hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const Co
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     hipLaunchKernelGGL(kern, dim3(grid_x, m_blocks), dim3(256), prm_ofs + 3 * WM * FM * 16 * sizeof(float), stream, x, wpk,
                        out, g, ep, mpad / 16, igemm_channel_groups(g.C), pl.r_max, pl.cb, pl.tiles_per_img, prm_ofs,
-                       total_tiles, in_bytes);
+                       total_tiles, in_bytes, (WN * FN * 16) % g.OW == 0 ? 1 : 0);
     return hipGetLastError();
 }
 

@@ -68,6 +68,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_kernel(const int8_t* __restric
         prm.bi[e] = ep.bias[o * 8 + e];
         prm.so[e] = ep.scale_out ? ep.scale_out[o * 8 + e] : 1.f;
     }
+    if constexpr (EPI == EPI_I8_P8_NONNEG) epi8_clamp_init(ep, prm);
 
     const int8_t* xp = x + (size_t)plane * g.H * g.W * 8;
     const int ix0 = ox * S - g.pw;

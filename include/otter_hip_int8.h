@@ -144,7 +144,8 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
  * {64,128,256}). tm < 0: keep the 3x3 halo kernel where it applies and force its pixel-fragment count to tn
  * (4..7, 0 = automatic). tm == -2 on a depthwise 3x3 layer: force the matrix-core kernel's strip height to tn
  * steps of 8 / stride output rows (0 = automatic). tm == -3: use the vector-ALU depthwise kernels instead, with a
- * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. */
+ * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. tm == -4: the generic
+ * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo kernel would be picked. */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
 /* ------------------------------------------------------------------------------------------------ */

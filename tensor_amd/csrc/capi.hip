@@ -291,7 +291,7 @@ static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom&
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
         if (h->w_igemm) {
-            if (h->force_tm > 0) return 1;
+            if (h->force_tm > 0 || h->force_tm == -4) return 1;  // forced generic kernel (-4: with automatic tiles)
             if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g, ep)) return 3;
             return 1;
         }

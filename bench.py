@@ -271,6 +271,14 @@ def cpu_baseline(wl, budget_s=15.0):
                     sample="%d images, scalar C restatement" % n_img)
     if name == "copy":
         return None
+    if name == "c4":
+        # the reference layer by layer in a child process (a crash or hang in it must not take the GPU figures along)
+        import subprocess
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--c4-cpu-child"], capture_output=True, text=True,
+                           timeout=300)
+        if r.returncode != 0:
+            raise RuntimeError("c4 CPU child failed (%d): %s" % (r.returncode, r.stderr[-200:]))
+        return json.loads(r.stdout.strip().splitlines()[-1])
     if name in ("c2", "c0"):
         n_img = min(4, N)
         K = p[0]["wq"].shape[0]
@@ -287,6 +295,48 @@ def cpu_baseline(wl, budget_s=15.0):
             return dict(value=ops / t / 1e12, unit="TOPS", cores=R.num_threads(), kind="reference",
                         sample="%d images, reference layer forward, min of 5" % n_img)
     return None
+
+
+def c4_cpu_child():
+    """Times the reference's ConvolutionLayer::forward for each of the 52 convolutions of the c4 network on ONE image
+    (synthetic inputs of each layer's shape and dtype, weights pre-packed, min of 3) and prints images/s of their sum.
+    The glue layers (adds, pooling, inner product) are left out: the reference has no int8 path for them."""
+    from oracle import binding
+    from tensor_amd import mobilenet
+    R = binding.Ref()
+    rng = np.random.default_rng(0)
+    layers = mobilenet.describe()
+    params = mobilenet.init_weights(layers, rng)
+    size, int8_blob = {"data": 224}, {"data": False}
+    total = 0.0
+    for l in layers:
+        if l["kind"] == "add":
+            size[l["name"]], int8_blob[l["name"]] = size[l["a"]], False
+            continue
+        if l["kind"] != "conv":
+            continue
+        hin = size[l["input"]]
+        hout = (hin + 2 * (l["k"] // 2) - l["k"]) // l["stride"] + 1
+        size[l["name"]], int8_blob[l["name"]] = hout, l["int8_out"]
+        pr = params[l["name"]]
+        dw = l["groups"] == l["cin"] == l["cout"]
+        opts = {"type": "Convolution", "in_channels": l["cin"], "out_channels": l["cout"], "kernel": l["k"],
+                "stride": l["stride"], "padding": l["k"] // 2, "groups": l["groups"],
+                "int8_scale_term": (1 if dw else 2) + (100 if l["int8_out"] else 0)}
+        if l["act"]:
+            opts["activation"] = l["act"]
+        if int8_blob[l["input"]]:
+            x = rng.integers(-127, 128, (1, l["cin"], hin, hin)).astype(np.int8)
+        else:
+            x = rng.uniform(0, 1, (1, l["cin"], hin, hin)).astype(np.float32)
+        L = R.conv_layer(opts, (1, l["cin"], hin, hin), pr["wq"], pr["bias"], pr["ws"], 100.0, 20.0, True)
+        _, t = L.forward(x, repeat=3, want_out=False)
+        L.close()
+        total += t
+    print(json.dumps(dict(value=1.0 / total, unit="images/s", cores=R.num_threads(), kind="reference",
+                          sample="1 image: the 52 convolution layers through the reference ConvolutionLayer::forward, one "
+                                 "by one (weights pre-packed, synthetic layer inputs), min of 3 each; glue layers not "
+                                 "included")))
 
 
 def measured_traffic(name):
@@ -328,6 +378,9 @@ def measure(wl, timer, steps, warmup, unit_main):
 
 
 def main():
+    if "--c4-cpu-child" in sys.argv:
+        c4_cpu_child()
+        return
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)

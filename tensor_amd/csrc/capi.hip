@@ -283,6 +283,7 @@ static Epilogue make_epilogue(const otter_hip_conv* h, int out_layout) {
     ep.act_hi = d.activation_type == 3 ? 6.f : __builtin_inff();
     ep.round_half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
     ep.so_positive = h->so_positive;
+    ep.lrelu = d.activation_type == 2 && d.activation_param0 >= 0.f && d.activation_param0 <= 1.f;
     return ep;
 }
 

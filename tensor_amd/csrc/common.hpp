@@ -113,17 +113,19 @@ struct Epilogue {
     float act_lo, act_hi;  // v = min(max(v, act_lo), act_hi)
     float round_half;      // 0.5f (ROUND_SSE) or 0.49999997f (ROUND_EXACT)
     bool so_positive;      // every output scale is finite and > 0 (lets the int8 epilogue clamp after rounding)
+    bool lrelu;            // LeakyReLU with a slope in [0, 1]: v = max(v, v * act_p0), applied by the fast epilogues
 };
 
 // which epilogue code a kernel instance carries
 enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3 };
 
-// The fast epilogues need: activation in {none, ReLU, clip}, and (I8_P8) int8 output in Byte8 with K % 8 == 0
-// or (F32_P4) fp32 output in Float4 with K % 4 == 0.
+// The fast epilogues need: activation in {none, ReLU, clip, LeakyReLU with a slope in [0, 1]}, and (I8_P8) int8
+// output in Byte8 with K % 8 == 0 or (F32_P4) fp32 output in Float4 with K % 4 == 0.
+// LeakyReLU there is v = max(v, v * slope): equal to (v > 0 ? v : v * slope) for every v when 0 <= slope <= 1.
 __host__ inline int pick_epilogue(const Epilogue& ep, int K) {
-    const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3;
+    const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3 || (ep.act == 2 && ep.lrelu);
     if (clamp_act && ep.out_kind == OTTER_HIP_OUT_I8 && ep.out_layout == OTTER_HIP_I8_P8 && K % 8 == 0) {
-        if (ep.act == 0) return EPI_I8_P8;
+        if (ep.act == 0 || ep.act == 2) return EPI_I8_P8;  // signed result: no clamp but the int8 range
         // after ReLU / clip the value to round is never negative; the fast path needs positive output scales
         return ep.so_positive ? EPI_I8_P8_NONNEG : EPI_GENERIC;
     }
@@ -273,6 +275,7 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float v = __fmaf_rn((float)a8[e], p.si[e], p.bi[e]);
+        if (!NONNEG && ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch
         v = __fmul_rn(v, p.so[e]);
         float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
         q[e] = (int)adj;  // toward zero, saturating
@@ -306,6 +309,7 @@ __device__ __forceinline__ void epi4_store_f32p4(float* __restrict__ out, const 
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)a[e], si[e], bi[e]);
         v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
         r[e] = __float_as_int(v);
     }
     *reinterpret_cast<ohip_v4i*>(out + elem) = r;

@@ -193,6 +193,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_i8_kernel(const int8_t* __rest
                 for (int k = 1; k < 9; ++k) acc = __builtin_amdgcn_sdot4(rows[r * S + k / 3][k % 3][h], wm[k][e], acc, false);
                 float v = __fmaf_rn((float)acc, si[e], bi[e]);
                 v = __builtin_amdgcn_fmed3f(v, ep.act_lo, ep.act_hi);
+                if (!NONNEG && ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch
                 v = __fmul_rn(v, so[e]);
                 const float adj =
                     NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));

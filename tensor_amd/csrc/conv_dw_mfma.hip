@@ -81,6 +81,7 @@ __device__ __forceinline__ unsigned dw_requant4(const Epilogue& ep, const v4i& a
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)acc[e], __int_as_float(si[e]), __int_as_float(bi[e]));
+        if (!NONNEG && ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch
         v = __fmul_rn(v, __int_as_float(so[e]));
         const float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
         qv[e] = (int)adj;  // toward zero, saturating
@@ -105,6 +106,7 @@ __device__ __forceinline__ v4i dw_dequant4(const Epilogue& ep, const v4i& acc, c
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)acc[e], __int_as_float(si[e]), __int_as_float(bi[e]));
         v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
         res[e] = __float_as_int(v);
     }
     return res;

@@ -278,6 +278,30 @@ def test_depthwise3x3_every_strip_height(hip, oracle, family, s, shift):
                 assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,kind", [
+    (64, 96, 3, 1, 1, 1, 2, 14, 16, 3),     # 3x3 LDS-halo kernel
+    (48, 72, 1, 1, 0, 1, 2, 13, 11, 1),     # 1x1 implicit GEMM
+    (32, 64, 3, 2, 1, 1, 2, 15, 15, 1),     # 3x3 stride 2 implicit GEMM
+    (40, 40, 3, 1, 1, 40, 3, 12, 20, 2),    # depthwise stride 1
+    (24, 24, 3, 2, 1, 24, 3, 13, 18, 2),    # depthwise stride 2
+])
+def test_leaky_relu_fast_epilogues(hip, oracle, C, K, k, s, p, g, N, H, W, kind):
+    """LeakyReLU 0.1 is the activation of the reference's own int8 models (benchmark/nanodet-plus-m-1.5x_416_int8_*.otter):
+    the fused epilogues evaluate it as max(v, v * slope); int8 and fp32 outputs against the oracle."""
+    rng = np.random.default_rng(C + K + k + s)
+    x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W)
+    for int8_out in (True, False):
+        want = oracle.conv_layer_forward(x, wq, ws, 18.0, stride=(s, s), pad=(p, p), groups=g, bias=bias, top_scale=13.0,
+                                         int8_out=int8_out, act_type=2, act_params=[0.1])
+        out, got_kind = run_conv(hip, oracle, x, wq, ws, 18.0, stride=s, pad=p, groups=g, bias=bias, top_scale=13.0,
+                                 act=2, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        assert got_kind == kind
+        if int8_out:
+            np.testing.assert_array_equal(out, want)
+        else:
+            assert_f32_close(out, want)
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

@@ -185,6 +185,10 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
         bi[t] = *reinterpret_cast<const v4i*>(ep.bias + ch + 4 * t);
         so[t] = v4i{0, 0, 0, 0};
         if constexpr (EPI != EPI_F32_P4) so[t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
+        // the bias is the fma's vector operand in every row: keep it resident (the compiler would otherwise re-copy
+        // it from scalar registers row after row)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(bi[t][e]));
     }
     unsigned qh[T][2] = {};
     if constexpr (EPI == EPI_I8_P8_NONNEG) {
@@ -231,41 +235,77 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
     for (int k = 0; k < S; ++k) frag[k % RING] = load_row(k + RING);
     __builtin_amdgcn_sched_barrier(0);
 
-    for (int rb = 0; rb < rps; rb += U) {
+    auto epilogue_store = [&](unsigned v_o, unsigned s_row, bool row_ok) {
+        if constexpr (EPI == EPI_F32_P4) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int r = rb + u;  // output row of the strip whose epilogue runs in this step
-            // row r+1: its input rows start (r+1)*S rows into the strip; the ring phase repeats every U rows
-            row_mfma((u + 1) % U, nxt);
-#pragma unroll
-            for (int k = 0; k < S; ++k) frag[((u + 1) * S + k) % RING] = load_row((r + 1) * S + k + RING);
-            const int oy = oy0 + r;
-            const bool row_ok = oy < g.OH && r < rps;  // rows past the strip / image are dropped
-            const unsigned s_row = row_ok ? s_out + (unsigned)oy * row_bytes : 0u;
-            const unsigned v_o = row_ok ? v_out : DW_OOB;
-            if constexpr (EPI == EPI_F32_P4) {
-#pragma unroll
-                for (int t = 0; t < T; ++t) {
-                    const v4i res = dw_dequant4(ep, cur[t], si[t], bi[t]);
-                    // the second set's channels 4..7 are the next Float4 pack: one plane further
-                    const unsigned vo_t = (t == 0 || !row_ok) ? v_o : v_o + OHW * 16u;
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, res), rout, (int)vo_t, (int)s_row, 0);
-                }
-            } else {
-                constexpr bool NONNEG = EPI == EPI_I8_P8_NONNEG;
-                if constexpr (S == 1) {
-                    v2i w2;
-                    w2[0] = (int)dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
-                    w2[1] = (int)dw_requant4<NONNEG>(ep, cur[T - 1], si[T - 1], bi[T - 1], so[T - 1], qh[T - 1][0], qh[T - 1][1]);
-                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, w2), rout, (int)v_o, (int)s_row, 0);
-                } else {
-                    const unsigned w1 = dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
-                    __builtin_amdgcn_raw_buffer_store_b32(w1, rout, (int)v_o, (int)s_row, 0);
-                }
+            for (int t = 0; t < T; ++t) {
+                const v4i res = dw_dequant4(ep, cur[t], si[t], bi[t]);
+                // the second set's channels 4..7 are the next Float4 pack: one plane further
+                const unsigned vo_t = (t == 0 || !row_ok) ? v_o : v_o + OHW * 16u;
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, res), rout, (int)vo_t, (int)s_row, 0);
             }
+        } else {
+            constexpr bool NONNEG = EPI == EPI_I8_P8_NONNEG;
+            if constexpr (S == 1) {
+                v2i w2;
+                w2[0] = (int)dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                w2[1] = (int)dw_requant4<NONNEG>(ep, cur[T - 1], si[T - 1], bi[T - 1], so[T - 1], qh[T - 1][0], qh[T - 1][1]);
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, w2), rout, (int)v_o, (int)s_row, 0);
+            } else {
+                const unsigned w1 = dw_requant4<NONNEG>(ep, cur[0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                __builtin_amdgcn_raw_buffer_store_b32(w1, rout, (int)v_o, (int)s_row, 0);
+            }
+        }
+    };
+
+    // A step of U rows is "interior" when every row it stores lies inside the strip and every row it loads inside
+    // the image: then the per-row scalar offsets just advance and nothing is predicated. The steps at the
+    // end of a strip take the checked path, which also leaves as soon as the strip's last row is stored (a strip need
+    // not be a whole number of steps).
+    const int nrows = min(rps, g.OH - oy0);
+    // loads of rows [RING, in_rows_ok) stay inside the image (iy0 + RING > 0); the few an interior step fetches past
+    // the strip's own last row are rows the next strip reads anyway
+    const int in_rows_ok = g.H - iy0;
+    const unsigned in_row_bytes = (unsigned)(g.W * 8);
+    for (int rb = 0; rb < nrows; rb += U) {
+        if (rb + U <= nrows && (rb + U) * S + S - 1 + RING < in_rows_ok) {
+            unsigned s_ld = s_in + (unsigned)(iy0 + (rb + 1) * S + RING) * in_row_bytes;
+            unsigned s_st = s_out + (unsigned)(oy0 + rb) * row_bytes;
 #pragma unroll
-            for (int t = 0; t < T; ++t) cur[t] = nxt[t];
-            __builtin_amdgcn_sched_barrier(0);
+            for (int u = 0; u < U; ++u) {
+                row_mfma((u + 1) % U, nxt);
+#pragma unroll
+                for (int k = 0; k < S; ++k) {
+                    v4i& f = frag[((u + 1) * S + k) % RING];
+                    if constexpr (ODDW) {
+                        const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)v_in, (int)s_ld, 0));
+                        const v2i hi = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)v_in2, (int)s_ld, 0));
+                        f = v4i{lo[0], lo[1], hi[0], hi[1]};
+                    } else {
+                        f = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)v_in, (int)s_ld, 0));
+                    }
+                    s_ld += in_row_bytes;
+                }
+                epilogue_store(v_out, s_st, true);
+                s_st += row_bytes;
+#pragma unroll
+                for (int t = 0; t < T; ++t) cur[t] = nxt[t];
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int r = rb + u;  // output row of the strip whose epilogue runs now
+                if (r >= nrows) return;  // wave-uniform
+                // row r+1: its input rows start (r+1)*S rows into the strip; the ring phase repeats every U rows
+                row_mfma((u + 1) % U, nxt);
+#pragma unroll
+                for (int k = 0; k < S; ++k) frag[((u + 1) * S + k) % RING] = load_row((r + 1) * S + k + RING);
+                epilogue_store(v_out, s_out + (unsigned)(oy0 + r) * row_bytes, true);
+#pragma unroll
+                for (int t = 0; t < T; ++t) cur[t] = nxt[t];
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
 }
@@ -296,27 +336,39 @@ hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const 
     }
     const long groups = (long)((g.N + ipw - 1) / ipw) * C8;
     if (groups > 65535) return hipErrorInvalidValue;  // grid.y limit; the caller splits the batch
-    // strip height in steps of U = 8/stride output rows: the tallest strip (setup and halo rows amortised over the
-    // longest walk) that still leaves about two waves per SIMD (measured: fewer, longer waves win)
+    // strip height: the tallest strips (setup and halo rows amortised over the longest walk) that still give about two
+    // waves per SIMD (measured: fewer, longer waves win), all of the same height so that the waves finish together
     const int U = 8 / g.sh;
     const int blocks_total = (g.OH + U - 1) / U;
-    int k = blocks_total;
-    if (strip_blocks > 0) k = std::min(strip_blocks, blocks_total);
-    else
-        while (k > 1 && (long)col_chunks * ((blocks_total + k - 1) / k) * groups < 2048) --k;
-    const int rps = k * U;
+    int rps;
+    if (strip_blocks > 0) {
+        rps = std::min(strip_blocks, blocks_total) * U;
+    } else {
+        int ns = 1;
+        while (ns < blocks_total && (long)col_chunks * ns * groups < 2048) ++ns;
+        rps = (g.OH + ns - 1) / ns;
+    }
     const int n_strips = (g.OH + rps - 1) / rps;
     const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
     const dim3 grid((unsigned)(col_chunks * (n_strips / wpb)), (unsigned)groups), block(64 * wpb);
+    // A grid of at most a few workgroups per CU is resident all at once, and the dispatcher is free to give one CU
+    // three of them and another one: the kernel then lasts as long as the fullest CU. Reserving a share of the CU's
+    // 160 KB of LDS per workgroup (the kernel uses none) caps the workgroups per CU at the even share.
+    constexpr long kCUs = 256;
+    const long wgs = (long)grid.x * grid.y;
+    const long per_cu = (wgs + kCUs - 1) / kCUs;
+    unsigned lds_reserve = 0;
+    if (wpb == 4 && per_cu >= 2 && per_cu <= 4) lds_reserve = (unsigned)(160 * 1024 / per_cu) / 1024 * 1024;
+    if (lds_reserve > 64 * 1024) lds_reserve = 64 * 1024;  // the default limit of dynamic LDS; still two per CU
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1));
 #define OHIP_DWM(S_, E_) \
     do {                                                                                                               \
         if (g.W & 1)                                                                                                   \
-            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, true>), grid, block, 0, stream, x, wa, out, g, ep, n_strips, \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, true>), grid, block, lds_reserve, stream, x, wa, out, g, ep, n_strips, \
                                rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
         else                                                                                                           \
-            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, false>), grid, block, 0, stream, x, wa, out, g, ep, n_strips, \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, false>), grid, block, lds_reserve, stream, x, wa, out, g, ep, n_strips, \
                                rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
     } while (0)
 #define OHIP_DWM_E(S_)                                                \

@@ -195,6 +195,36 @@ int otter_hip_global_avgpool(const float* src, int src_layout, int n, int c, int
 int otter_hip_inner_product(const float* x, int n, int in_features, const float* weight, const float* bias,
                             int out_features, float* y, void* stream);
 
+/* ------------------------------------------------------------------------------------------------ */
+/* fp32 layout glue of the reference's int8 model files (benchmark/nanodet-plus-m-1.5x_416_int8_*.otter):  */
+/* every blob between their convolutions is fp32; src and dst may be in any fp32 layout each          */
+/* ------------------------------------------------------------------------------------------------ */
+
+/* dst[:, dst_c0 : dst_c0+count] = src[:, src_c0 : src_c0+count] over channels. One call per input is
+ * ConcatLayer::forward with axis 1 (Tensor/ConcatLayer.cpp:54-67); with dst_c = count, dst_c0 = 0 it is
+ * CropLayer::forward with axis 1 (Tensor/CropLayer.cpp:69-75, native::slice on the logical channel index). */
+int otter_hip_copy_channels(const float* src, int src_layout, int src_c, int src_c0, float* dst, int dst_layout,
+                            int dst_c, int dst_c0, int count, int n, int h, int w, void* stream);
+
+/* ChannelShuffleLayer::forward (Tensor/ChannelShuffleLayer.cpp:37-41, Tensor/ChannelShuffleKernel.cpp:19-55):
+ * out[:, j*groups + i] = in[:, i*(C/groups) + j]. */
+int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,
+                              int groups, void* stream);
+
+/* MaxPoolLayer::forward (Tensor/MaxPoolLayer.cpp:123-134): max over a kernel window of the padded input; out_h /
+ * out_w as MaxPoolLayer::compute_output_shape gives them (Tensor/Pool.hpp:33-50). pad_value is what a tap outside
+ * the image counts as: -INFINITY in the reference's generic kernel, 0 in its packed 3x3 and 2x2 stride-2 kernels,
+ * which pad the blob with zeros first (Tensor/Pool.cpp:752-1160; selection rule at :1185-1199). */
+int otter_hip_maxpool2d(const float* src, int src_layout, int n, int c, int h, int w, int kernel_h, int kernel_w,
+                        int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w, int out_h,
+                        int out_w, float pad_value, float* dst, int dst_layout, void* stream);
+
+/* UpsampleLayer::forward (Tensor/UpsampleLayer.cpp:108-124) through otter::Interpolate's packed path
+ * (Tensor/TensorInterpolation.cpp:16-45 coefficients, :161-272 bilinear, :670-690 nearest), which is what the
+ * reference's Net runs for channel counts that are multiples of 4. mode 1 nearest, 2 bilinear. */
+int otter_hip_upsample2d(const float* src, int src_layout, int n, int c, int h, int w, int out_h, int out_w, int mode,
+                         int align_corner, float* dst, int dst_layout, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -255,6 +255,23 @@ class Ref:
                                                   C.c_int(int(packing)), _p(out, _i8p)))
         return out
 
+    # ---- model files and whole networks (Tensor/Otter.cpp, Tensor/Initializer.cpp, Tensor/Net.cpp) ----
+    def otter_dump(self, path):
+        """The reference's parse of a `.otter` file: 'N name', 'G key=value', 'T block', 'P key=value' lines."""
+        self.lib.otter_ref_otter_dump.restype = C.c_long
+        buf = C.create_string_buffer(1 << 24)
+        n = self.lib.otter_ref_otter_dump(os.fsencode(path), buf, C.c_size_t(len(buf)))
+        self._check(0 if n >= 0 else -1)
+        return buf.raw[:n].decode(errors="surrogateescape")
+
+    @property
+    def ncnn_read_entry(self):
+        """(function, error function) of the reference's `.bin` reader, same signature as the host library's."""
+        return self.lib.otter_ref_ncnn_read, self.lib.otter_ref_last_error
+
+    def net(self, otter_path, bin_path=None, use_packing=True):
+        return RefNet(self, otter_path, bin_path, use_packing)
+
     def conv_layer(self, options, in_shape, wq, bias, weight_scales, in_scale, top_scale=1.0, use_packing=True):
         return RefConvLayer(self, options, in_shape, wq, bias, weight_scales, in_scale, top_scale, use_packing)
 
@@ -305,6 +322,50 @@ class RefConvLayer:
     def close(self):
         if self.h:
             self.ref.lib.otter_ref_conv_layer_destroy(C.c_void_p(self.h))
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class RefNet:
+    """The reference's Net over a `.otter` description and an ncnn `.bin` (batch 1, every blob kept)."""
+
+    def __init__(self, ref, otter_path, bin_path, use_packing):
+        self.ref = ref
+        L = ref.lib
+        L.otter_ref_net_open.restype = C.c_void_p
+        L.otter_ref_net_run.restype = C.c_double
+        self.h = C.c_void_p(L.otter_ref_net_open(os.fsencode(otter_path), os.fsencode(bin_path) if bin_path else None,
+                                                 C.c_int(int(use_packing))))
+        if not self.h:
+            raise RuntimeError("reference: " + L.otter_ref_last_error().decode(errors="replace"))
+
+    def run(self, input_blob, x, names):
+        """x: [1, C, H, W] fp32. Returns ({name: unpacked array}, seconds spent extracting names[0])."""
+        x = _f32(x)
+        assert x.ndim == 4 and x.shape[0] == 1
+        L = self.ref.lib
+        c_names = (C.c_char_p * len(names))(*[n.encode() for n in names])
+        secs = L.otter_ref_net_run(self.h, input_blob.encode(), _p(x, _f32p), x.shape[1], x.shape[2], x.shape[3], c_names,
+                                   len(names))
+        if secs < 0:
+            raise RuntimeError("reference: " + L.otter_ref_last_error().decode(errors="replace"))
+        out = {}
+        for i, n in enumerate(names):
+            dims, is8 = (C.c_longlong * 4)(), C.c_int()
+            self.ref._check(L.otter_ref_net_blob_info(self.h, i, dims, C.byref(is8)))
+            a = np.empty(tuple(dims), np.int8 if is8.value else np.float32)
+            self.ref._check(L.otter_ref_net_blob_copy(self.h, i, a.ctypes.data_as(C.c_void_p), C.c_size_t(a.nbytes)))
+            out[n] = a
+        return out, secs
+
+    def close(self):
+        if self.h:
+            self.ref.lib.otter_ref_net_close(self.h)
             self.h = None
 
     def __del__(self):

@@ -26,6 +26,9 @@
 #include "NetOption.hpp"
 #include "Net.hpp"
 #include "ParamDict.hpp"
+#include "Otter.hpp"
+#include "Initializer.hpp"
+#include "DataReader.hpp"
 
 #include <chrono>
 #include <cstring>
@@ -324,6 +327,152 @@ __attribute__((visibility("default"))) double otter_ref_conv_layer_forward(const
         fail(e.what());
         return -1.0;
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Net level: the reference's own Net reading a `.otter` description (Tensor/Net.cpp:518-536) and an ncnn `.bin`
+// (Tensor/Net.cpp:538-586), run on one image with every intermediate blob kept.
+// ---------------------------------------------------------------------------------------------
+struct RefNet {
+    otter::Net net;
+    std::vector<Tensor> blobs;       // unpacked copies of every blob of the last run
+    std::vector<std::string> names;  // blob names in index order
+};
+
+__attribute__((visibility("default"))) void* otter_ref_net_open(const char* otter_path, const char* bin_path,
+                                                                int use_packing_layout) {
+    try {
+        RefNet* h = new RefNet();
+        h->net.option.use_packing_layout = use_packing_layout != 0;
+        h->net.option.lightmode = false;
+        if (h->net.load_otter(otter_path, otter::CompileMode::Inference) != 0) {
+            delete h;
+            fail("load_otter failed");
+            return nullptr;
+        }
+        if (bin_path && h->net.load_weight(bin_path, otter::Net::WeightType::Ncnn) != 0) {
+            delete h;
+            fail("load_weight failed");
+            return nullptr;
+        }
+        return h;
+    } catch (const std::exception& e) {
+        fail(e.what());
+        return nullptr;
+    }
+}
+
+__attribute__((visibility("default"))) void otter_ref_net_close(void* h) { delete static_cast<RefNet*>(h); }
+
+// Runs the net on one fp32 image [1, c, hh, w] fed to `input_blob` and extracts `n_names` blobs (each unpacked to
+// elempack 1 by Extractor::extract(..., 0), Tensor/Net.cpp:729-731). Returns seconds spent in the extraction of
+// the LAST name (the whole forward pass when the earlier names are upstream of it is then already done, so pass
+// the final outputs first to time the network), or a negative value on error.
+__attribute__((visibility("default"))) double otter_ref_net_run(void* hv, const char* input_blob, const float* x, int c,
+                                                                int hh, int w, const char* const* names, int n_names) {
+    RefNet* h = static_cast<RefNet*>(hv);
+    try {
+        auto ex = h->net.create_extractor();
+        ex.set_lightmode(false);
+        if (ex.input(std::string(input_blob), make_f32(x, {1, c, hh, w})) != 0) return fail("unknown input blob");
+        h->blobs.clear();
+        h->names.clear();
+        double first = -1.0;
+        for (int i = 0; i < n_names; ++i) {
+            Tensor t;
+            auto t0 = std::chrono::steady_clock::now();
+            int rc = ex.extract(std::string(names[i]), t, 0);
+            auto t1 = std::chrono::steady_clock::now();
+            if (rc != 0) return fail(std::string("extract failed for ") + names[i]);
+            if (i == 0) first = std::chrono::duration<double>(t1 - t0).count();
+            h->blobs.push_back(t.contiguous());
+            h->names.push_back(names[i]);
+        }
+        return first;
+    } catch (const std::exception& e) {
+        fail(e.what());
+        return -1.0;
+    }
+}
+
+// Shape and element type of an extracted blob: dims[0..3] (missing leading dims = 1), *is_int8.
+__attribute__((visibility("default"))) int otter_ref_net_blob_info(void* hv, int index, long long* dims, int* is_int8) {
+    RefNet* h = static_cast<RefNet*>(hv);
+    if (index < 0 || index >= (int)h->blobs.size()) return fail("blob index");
+    const Tensor& t = h->blobs[index];
+    for (int i = 0; i < 4; ++i) dims[i] = 1;
+    const int nd = (int)t.dim();
+    for (int i = 0; i < nd && i < 4; ++i) dims[4 - nd + i] = t.size(i);
+    *is_int8 = t.scalar_type() == ScalarType::Byte;
+    return t.scalar_type() == ScalarType::Byte || t.scalar_type() == ScalarType::Float ? 0 : fail("blob dtype");
+}
+
+__attribute__((visibility("default"))) int otter_ref_net_blob_copy(void* hv, int index, void* dst, size_t capacity) {
+    RefNet* h = static_cast<RefNet*>(hv);
+    if (index < 0 || index >= (int)h->blobs.size()) return fail("blob index");
+    const Tensor& t = h->blobs[index];
+    const size_t bytes = (size_t)t.numel() * (t.scalar_type() == ScalarType::Byte ? 1 : 4);
+    if (bytes > capacity) return fail("blob larger than the buffer");
+    std::memcpy(dst, t.data_ptr(), bytes);
+    return 0;
+}
+
+// The reference's reading of a `.otter` file as text: "T <block name>" per layer block followed by "P <key>=<value>"
+// per option that Net::load_otter would see (OtterLeader::getTeamParams), "N <project name>" first.
+__attribute__((visibility("default"))) long otter_ref_otter_dump(const char* path, char* buf, size_t capacity) {
+    try {
+        otter::core::OtterLeader leader;
+        if (!leader.readProject(path)) return fail("readProject failed");
+        std::string out = "N " + leader.getProjectName() + "\n";
+        for (size_t i = 0; i < leader.params_size(); ++i) out += "G " + leader.getParam((int)i).type + "=" + leader.getParam((int)i).info + "\n";
+        for (size_t i = 0; i < leader.teams_size(); ++i) {
+            out += "T " + leader.getTeamName((int)i) + "\n";
+            for (const auto& p : leader.getTeamParams((int)i)) out += "P " + p.type + "=" + p.info + "\n";
+        }
+        if (out.size() + 1 > capacity) return fail("dump larger than the buffer");
+        std::memcpy(buf, out.c_str(), out.size() + 1);
+        return (long)out.size();
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// InitializerNcnnFromDataReader over a file (Tensor/Initializer.cpp:56-190): reads `n` tensors of the given shapes
+// (4 entries each, unused trailing entries 0) and kinds (0 weight with tag, 1 plain fp32), appends their bytes to
+// `out`, records 0 (fp32) / 1 (int8) / -1 (undefined) per tensor in `dtypes`, and reports the bytes left in the file.
+__attribute__((visibility("default"))) long otter_ref_ncnn_read(const char* path, int n, const long long* shapes,
+                                                                const int* kinds, int* dtypes, unsigned char* out,
+                                                                size_t capacity, long long* remain) {
+    FILE* f = std::fopen(path, "rb");
+    if (!f) return fail("cannot open file");
+    size_t used = 0;
+    try {
+        otter::DataReaderFromStdio dr(f);
+        otter::InitializerNcnnFromDataReader init(dr);
+        for (int i = 0; i < n; ++i) {
+            std::vector<int64_t> shape;
+            for (int d = 0; d < 4 && shapes[i * 4 + d] > 0; ++d) shape.push_back(shapes[i * 4 + d]);
+            Tensor t = init.load(shape, kinds[i]);
+            if (!t.defined()) {
+                dtypes[i] = -1;
+                continue;
+            }
+            dtypes[i] = t.scalar_type() == ScalarType::Byte ? 1 : 0;
+            const size_t bytes = (size_t)t.numel() * (dtypes[i] ? 1 : 4);
+            if (used + bytes > capacity) {
+                std::fclose(f);
+                return fail("tensors larger than the buffer");
+            }
+            std::memcpy(out + used, t.data_ptr(), bytes);
+            used += bytes;
+        }
+        *remain = (long long)dr.remain();
+    } catch (const std::exception& e) {
+        std::fclose(f);
+        return fail(e.what());
+    }
+    std::fclose(f);
+    return (long)used;
 }
 
 }  // extern "C"

@@ -493,4 +493,73 @@ int otter_hip_inner_product(const float* x, int n, int in_features, const float*
     return OTTER_HIP_OK;
 }
 
+// -----------------------------------------------------------------------------------------------------
+// fp32 layout glue of the reference's int8 model files
+// -----------------------------------------------------------------------------------------------------
+
+static int check_f32_pair(const char* who, const void* src, const void* dst, int sl, int dl, int sc, int dc) {
+    if (!src || !dst) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": null");
+    if (!valid_layout(sl) || !valid_layout(dl) || layout_elem(sl) != 0 || layout_elem(dl) != 0)
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": fp32 layouts expected");
+    if (sc < 1 || dc < 1 || sc % layout_pack(sl) || dc % layout_pack(dl))
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": pack does not divide C");
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_copy_channels(const float* src, int src_layout, int src_c, int src_c0, float* dst, int dst_layout,
+                            int dst_c, int dst_c0, int count, int n, int h, int w, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_copy_channels", src, dst, src_layout, dst_layout, src_c, dst_c)) return rc;
+    if (n < 0 || h < 1 || w < 1 || count < 0 || src_c0 < 0 || dst_c0 < 0 || src_c0 + count > src_c || dst_c0 + count > dst_c)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_copy_channels: channel range outside the blob");
+    if ((size_t)n * src_c * h * w >= (1ull << 31) || (size_t)n * dst_c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_copy_channels: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_copy_channels(src, src_c, layout_pack(src_layout), src_c0, dst, dst_c, layout_pack(dst_layout), dst_c0,
+                                 count, n, h, w, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,
+                              int groups, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_channel_shuffle", src, dst, src_layout, dst_layout, c, c)) return rc;
+    if (n < 0 || h < 1 || w < 1 || groups < 1 || c % groups)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_channel_shuffle: groups must divide C");
+    if ((size_t)n * c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_channel_shuffle: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_channel_shuffle(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h, w, groups,
+                                   (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_maxpool2d(const float* src, int src_layout, int n, int c, int h, int w, int kernel_h, int kernel_w,
+                        int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w, int out_h,
+                        int out_w, float pad_value, float* dst, int dst_layout, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_maxpool2d", src, dst, src_layout, dst_layout, c, c)) return rc;
+    if (n < 0 || h < 1 || w < 1 || kernel_h < 1 || kernel_w < 1 || stride_h < 1 || stride_w < 1 || pad_h < 0 || pad_w < 0 ||
+        dilation_h < 1 || dilation_w < 1 || out_h < 1 || out_w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_maxpool2d: bad geometry");
+    // every window must start inside the padded input (what the reference's shape rule guarantees)
+    if ((out_h - 1) * stride_h >= h + pad_h || (out_w - 1) * stride_w >= w + pad_w)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_maxpool2d: output larger than the pooling geometry allows");
+    if ((size_t)n * c * h * w >= (1ull << 31) || (size_t)n * c * out_h * out_w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_maxpool2d: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_maxpool(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h, w, out_h, out_w, kernel_h,
+                           kernel_w, stride_h, stride_w, pad_h, pad_w, dilation_h, dilation_w, pad_value, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_upsample2d(const float* src, int src_layout, int n, int c, int h, int w, int out_h, int out_w, int mode,
+                         int align_corner, float* dst, int dst_layout, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_upsample2d", src, dst, src_layout, dst_layout, c, c)) return rc;
+    if (n < 0 || h < 1 || w < 1 || out_h < 1 || out_w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_upsample2d: bad shape");
+    if (mode != 1 && mode != 2) return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_upsample2d: mode must be 1 or 2");
+    if (mode == 2 && (h < 2 || w < 2))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_upsample2d: bilinear needs at least 2x2 input");
+    if ((size_t)n * c * h * w >= (1ull << 31) || (size_t)n * c * out_h * out_w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_upsample2d: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_upsample(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h, w, out_h, out_w, mode,
+                            align_corner ? 1 : 0, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
 }  // extern "C"

@@ -55,4 +55,14 @@ hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, fl
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream);
 
+// reshape.hip: fp32 layout glue (pack = elempack of the layout on that side)
+hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
+                             int H, int W, hipStream_t stream);
+hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
+                               hipStream_t stream);
+hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int kh,
+                       int kw, int sh, int sw, int ph, int pw, int dh, int dw, float pad_value, hipStream_t stream);
+hipError_t run_upsample(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int mode,
+                        int align_corner, hipStream_t stream);
+
 }  // namespace ohip

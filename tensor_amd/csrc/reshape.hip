@@ -1,0 +1,200 @@
+// fp32 layout glue between the convolutions of a detection backbone (the layers the reference's int8 model files
+// put around their convolutions): channel-range copy (Concat / Crop), channel shuffle, max pooling, 2-D upsampling.
+// Every kernel takes any of the fp32 activation layouts on either side (elempack 1, 4 or 8: memory order
+// n, c/p, h, w, c%p) and is a pure gather: one thread per destination element (or per group of four where source
+// and destination packs line up), enumerated in destination memory order so that the writes are contiguous.
+#include "common.hpp"
+#include "conv_igemm.hpp"
+
+namespace ohip {
+
+__device__ __forceinline__ size_t packed_off(int n, int c, int y, int x, int C, int H, int W, int p) {
+    return ((((size_t)n * (C / p) + c / p) * H + y) * W + x) * p + c % p;
+}
+
+// destination memory order restricted to a channel range that starts and ends on a pack boundary:
+// linear index -> (n, c, y, x)
+struct DstIndex {
+    int n, c, y, x;
+};
+__device__ __forceinline__ DstIndex dst_index(size_t i, int c0, int cnt, int H, int W, int p) {
+    DstIndex d;
+    const int e = (int)(i % p);
+    i /= p;
+    d.x = (int)(i % W);
+    i /= W;
+    d.y = (int)(i % H);
+    i /= H;
+    const int packs = cnt / p;
+    d.c = c0 + (int)(i % packs) * p + e;
+    d.n = (int)(i / packs);
+    return d;
+}
+
+// dst[:, cd0 : cd0+cnt] = src[:, cs0 : cs0+cnt]   (Tensor/ConcatLayer.cpp:54-67 one input at a time;
+// Tensor/CropLayer.cpp:69-75 with axis 1). ALIGNED: cd0 and cnt are multiples of the destination pack.
+template <bool ALIGNED>
+__global__ void __launch_bounds__(256) copy_channels_kernel(const float* __restrict__ src, int Cs, int ps, int cs0,
+                                                            float* __restrict__ dst, int Cd, int pd, int cd0, int cnt,
+                                                            int N, int H, int W, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    DstIndex d;
+    if (ALIGNED) {
+        d = dst_index(i, cd0, cnt, H, W, pd);
+    } else {  // channel-major enumeration; the writes of a packed destination are strided then
+        size_t r = i;
+        d.x = (int)(r % W), r /= W;
+        d.y = (int)(r % H), r /= H;
+        d.c = cd0 + (int)(r % cnt);
+        d.n = (int)(r / cnt);
+    }
+    dst[packed_off(d.n, d.c, d.y, d.x, Cd, H, W, pd)] = src[packed_off(d.n, d.c - cd0 + cs0, d.y, d.x, Cs, H, W, ps)];
+}
+
+// same, four floats per thread: both packs are multiples of 4, the source offset is a multiple of 4 and the
+// destination range starts and ends on a destination pack boundary
+__global__ void __launch_bounds__(256) copy_channels4_kernel(const float* __restrict__ src, int Cs, int ps, int cs0,
+                                                             float* __restrict__ dst, int Cd, int pd, int cd0, int cnt,
+                                                             int N, int H, int W, size_t total4) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total4) return;
+    // quads of the destination range in memory order: (n, pack, y, x, quad within the pack)
+    size_t r = i;
+    const int qd = pd / 4;
+    const int q = (int)(r % qd);
+    r /= qd;
+    const int x = (int)(r % W);
+    r /= W;
+    const int y = (int)(r % H);
+    r /= H;
+    const int packs = cnt / pd;
+    const int c = cd0 + (int)(r % packs) * pd + 4 * q;
+    const int n = (int)(r / packs);
+    const float4 v = *reinterpret_cast<const float4*>(src + packed_off(n, c - cd0 + cs0, y, x, Cs, H, W, ps));
+    *reinterpret_cast<float4*>(dst + packed_off(n, c, y, x, Cd, H, W, pd)) = v;
+}
+
+hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
+                             int H, int W, hipStream_t stream) {
+    const size_t total = (size_t)N * cnt * H * W;
+    if (total == 0) return hipSuccess;
+    const bool whole = cd0 % pd == 0 && cnt % pd == 0;
+    if (whole && ps % 4 == 0 && pd % 4 == 0 && cs0 % 4 == 0) {
+        const size_t total4 = total / 4;
+        hipLaunchKernelGGL(copy_channels4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, src, Cs, ps,
+                           cs0, dst, Cd, pd, cd0, cnt, N, H, W, total4);
+    } else if (whole) {
+        hipLaunchKernelGGL(copy_channels_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, Cs,
+                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, total);
+    } else {
+        hipLaunchKernelGGL(copy_channels_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, Cs,
+                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, total);
+    }
+    return hipGetLastError();
+}
+
+// Tensor/ChannelShuffleKernel.cpp:19-55: input seen as [n, g, C/g, ...], output as [n, C/g, g, ...]
+__global__ void __launch_bounds__(256) channel_shuffle_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst,
+                                                              int pd, int N, int C, int H, int W, int groups, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const DstIndex d = dst_index(i, 0, C, H, W, pd);
+    const int cpg = C / groups;
+    const int cs = (d.c % groups) * cpg + d.c / groups;
+    dst[i] = src[packed_off(d.n, cs, d.y, d.x, C, H, W, ps)];
+}
+
+hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
+                               hipStream_t stream) {
+    const size_t total = (size_t)N * C * H * W;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(channel_shuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd,
+                       N, C, H, W, groups, total);
+    return hipGetLastError();
+}
+
+// Tensor/MaxPoolLayer.cpp:123-134 -> otter::max_pool2d: window over the padded input; a NaN in the window wins
+// (Tensor/MaxPoolKernel.cpp, the comparison `(val > maxval) || isnan(val)`). pad_value is what a tap outside the
+// image counts as: -inf in the reference's generic kernel, 0 in its packed 3x3 / 2x2 stride-2 kernels
+// (Tensor/Pool.cpp:974, which pad the blob with zeros first).
+__global__ void __launch_bounds__(256) maxpool_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
+                                                      int N, int C, int H, int W, int OH, int OW, int kh, int kw, int sh,
+                                                      int sw, int ph, int pw, int dh, int dw, float pad_value, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const DstIndex d = dst_index(i, 0, C, OH, OW, pd);
+    float m = -__builtin_inff();
+    for (int u = 0; u < kh; ++u) {
+        const int iy = d.y * sh - ph + u * dh;
+        for (int v = 0; v < kw; ++v) {
+            const int ix = d.x * sw - pw + v * dw;
+            const bool inside = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            const float val = inside ? src[packed_off(d.n, d.c, iy, ix, C, H, W, ps)] : pad_value;
+            if (val > m || val != val) m = val;
+        }
+    }
+    dst[i] = m;
+}
+
+hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int kh,
+                       int kw, int sh, int sw, int ph, int pw, int dh, int dw, float pad_value, hipStream_t stream) {
+    const size_t total = (size_t)N * C * OH * OW;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
+                       W, OH, OW, kh, kw, sh, sw, ph, pw, dh, dw, pad_value, total);
+    return hipGetLastError();
+}
+
+// Source index and weight of one output coordinate: Tensor/TensorInterpolation.cpp:16-45 (linear_coeffs), the
+// coefficient computation in double precision, the clamp at both borders included.
+__device__ __forceinline__ void linear_coeff(int in_size, int out_size, int d, int align_corner, int& s, float& f) {
+    double scale = (double)in_size / out_size;
+    if (align_corner) scale = (double)(in_size - 1) / (out_size - 1);
+    f = (float)((d + 0.5) * scale - 0.5);
+    if (align_corner) f = (float)(d * scale);
+    s = (int)floorf(f);
+    f -= (float)s;
+    if (s < 0) s = 0, f = 0.f;
+    if (s >= in_size - 1) s = in_size - 2, f = 1.f;
+}
+
+// mode 1 nearest (Tensor/TensorInterpolation.cpp:670-690: source = min(int(d * in/out), in-1), the ratio in fp32),
+// mode 2 bilinear (Tensor/TensorInterpolation.cpp:161-272: rows = S0*a0 then fma(S1, a1, .); out = rows0*b0 then
+// fma(rows1, b1, .)) -- the arithmetic of the reference's packed path, which is what its Net runs when the channel
+// count is a multiple of 4.
+__global__ void __launch_bounds__(256) upsample_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
+                                                       int N, int C, int H, int W, int OH, int OW, int mode,
+                                                       int align_corner, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const DstIndex d = dst_index(i, 0, C, OH, OW, pd);
+    if (mode == 1) {
+        const float hs = (float)H / (float)OH, ws = (float)W / (float)OW;
+        const int iy = min((int)(d.y * hs), H - 1), ix = min((int)(d.x * ws), W - 1);
+        dst[i] = src[packed_off(d.n, d.c, iy, ix, C, H, W, ps)];
+        return;
+    }
+    int sx, sy;
+    float fx, fy;
+    linear_coeff(W, OW, d.x, align_corner, sx, fx);
+    linear_coeff(H, OH, d.y, align_corner, sy, fy);
+    const float a0 = 1.f - fx, a1 = fx, b0 = 1.f - fy, b1 = fy;
+    const float s00 = src[packed_off(d.n, d.c, sy, sx, C, H, W, ps)], s01 = src[packed_off(d.n, d.c, sy, sx + 1, C, H, W, ps)];
+    const float s10 = src[packed_off(d.n, d.c, sy + 1, sx, C, H, W, ps)],
+                s11 = src[packed_off(d.n, d.c, sy + 1, sx + 1, C, H, W, ps)];
+    const float r0 = __fmaf_rn(s01, a1, __fmul_rn(s00, a0));
+    const float r1 = __fmaf_rn(s11, a1, __fmul_rn(s10, a0));
+    dst[i] = __fmaf_rn(r1, b1, __fmul_rn(r0, b0));
+}
+
+hipError_t run_upsample(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int mode,
+                        int align_corner, hipStream_t stream) {
+    const size_t total = (size_t)N * C * OH * OW;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(upsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
+                       W, OH, OW, mode, align_corner, total);
+    return hipGetLastError();
+}
+
+}  // namespace ohip

@@ -5,6 +5,7 @@
 #include <string>
 
 #include "../../include/otter_hip_int8.h"
+#include "otter_file.hpp"
 #include "otter_hip.hpp"
 
 using namespace otter;
@@ -235,6 +236,132 @@ int otter_host_functional_chain(const float* x, int n, int c, int h, int w, floa
     } catch (const std::exception& e) {
         return fail(e.what());
     }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// model files
+// ---------------------------------------------------------------------------------------------------
+
+// Net::load_otter (Tensor/Net.cpp:518-536)
+int otter_host_net_load_otter(void* net, const char* path, int initial) {
+    try {
+        if (static_cast<Net*>(net)->load_otter(path, initial ? CompileMode::Initial : CompileMode::Inference))
+            return fail(std::string("cannot read ") + path);
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// Net::load_weight (Tensor/Net.cpp:538-586); ncnn != 0: ncnn `.bin`, else Otter's fp32 stream
+int otter_host_net_load_weight(void* net, const char* path, int ncnn) {
+    try {
+        const int rc = static_cast<Net*>(net)->load_weight(path, ncnn ? Net::WeightType::Ncnn : Net::WeightType::Otter);
+        return rc ? fail("load_weight returned " + std::to_string(rc) + ": " + otter_hip_last_error()) : 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// One line per layer, "type name bottoms tops" and for a convolution its shape as load_model will ask for it:
+// "Convolution conv_1 data_1 conv_1 K C groups kh kw bias_term int8_scale_term".
+long otter_host_net_describe(void* net, char* buf, size_t capacity) {
+    try {
+        const std::string out = static_cast<Net*>(net)->describe();
+        if (out.size() + 1 > capacity) return fail("description larger than the buffer");
+        std::memcpy(buf, out.c_str(), out.size() + 1);
+        return (long)out.size();
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// One pass with any number of blobs set beforehand (Extractor::input on each), e.g. a layer's bottoms when a test
+// drives a single layer: inputs are NCHW fp32 / int8 on the host, shapes4 holds 4 entries per input.
+int otter_host_net_eval(void* net, int n_inputs, const char* const* in_names, const void* const* in_ptrs,
+                        const int* in_is_int8, const int64_t* shapes4, const char* out_name, void* out,
+                        size_t out_capacity_bytes, int* out_dtype, int64_t* out_shape4) {
+    try {
+        Net* N = static_cast<Net*>(net);
+        Extractor ex = N->create_extractor();
+        ex.set_lightmode(false);
+        for (int i = 0; i < n_inputs; ++i) {
+            const int64_t* s = shapes4 + 4 * i;
+            Tensor in = Tensor::from_blob(in_ptrs[i], {s[0], s[1], s[2], s[3]}, in_is_int8[i] ? ScalarType::Byte : ScalarType::Float);
+            if (ex.input(in_names[i], in)) return fail(std::string("unknown blob ") + in_names[i]);
+        }
+        Tensor feat;
+        const int rc = ex.extract(out_name, feat, 0);
+        if (rc) return fail("forward failed with code " + std::to_string(rc) + ": " + otter_hip_last_error());
+        if (feat.dim() == 4 && feat.elempack() != 1) feat = feat.packing(1);
+        const ScalarType b = base_of(feat.scalar_type());
+        if (out_dtype) *out_dtype = b == ScalarType::Float ? 0 : (b == ScalarType::Byte ? 1 : 2);
+        if (out_shape4)
+            for (int i = 0; i < 4; ++i) out_shape4[i] = i < feat.dim() ? feat.size(i) : 1;
+        if (out) {
+            if (feat.nbytes() > out_capacity_bytes) return fail("output buffer too small");
+            std::memcpy(out, feat.data_ptr(), feat.nbytes());
+        }
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// What OtterLeader::readProject makes of a file, as text: "N <project name>", "G key=value" per file-level
+// parameter, then per block "T <name>" and "P key=value" for every option Net::load_otter passes to the layer.
+long otter_host_otter_dump(const char* path, char* buf, size_t capacity) {
+    try {
+        core::OtterLeader leader;
+        if (!leader.readProject(path)) return fail("readProject failed");
+        std::string out = "N " + leader.getProjectName() + "\n";
+        for (const core::Param& p : leader.getParams()) out += "G " + p.type + "=" + p.info + "\n";
+        for (size_t i = 0; i < leader.teams_size(); ++i) {
+            out += "T " + leader.getTeamName((int)i) + "\n";
+            for (const core::Param& p : leader.getTeamParams((int)i)) out += "P " + p.type + "=" + p.info + "\n";
+        }
+        if (out.size() + 1 > capacity) return fail("dump larger than the buffer");
+        std::memcpy(buf, out.c_str(), out.size() + 1);
+        return (long)out.size();
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
+// InitializerNcnnFromDataReader over a file: reads `n` tensors of the given shapes (4 entries each, unused trailing
+// entries 0) and kinds (0 weight with tag, 1 plain fp32), appends their bytes to `out`, records 0 (fp32) / 1 (int8) /
+// -1 (undefined) per tensor in `dtypes`, and reports the bytes left in the file.
+long otter_host_ncnn_read(const char* path, int n, const long long* shapes, const int* kinds, int* dtypes,
+                          unsigned char* out, size_t capacity, long long* remain) {
+    FILE* f = std::fopen(path, "rb");
+    if (!f) return fail("cannot open file");
+    size_t used = 0;
+    try {
+        DataReaderFromStdio dr(f);
+        InitializerNcnnFromDataReader init(dr);
+        for (int i = 0; i < n; ++i) {
+            std::vector<int64_t> shape;
+            for (int d = 0; d < 4 && shapes[i * 4 + d] > 0; ++d) shape.push_back(shapes[i * 4 + d]);
+            Tensor t = init.load(shape, kinds[i]);
+            if (!t.defined()) {
+                dtypes[i] = -1;
+                continue;
+            }
+            dtypes[i] = t.scalar_type() == ScalarType::Byte ? 1 : 0;
+            if (used + t.nbytes() > capacity) {
+                std::fclose(f);
+                return fail("tensors larger than the buffer");
+            }
+            std::memcpy(out + used, t.data_ptr(), t.nbytes());
+            used += t.nbytes();
+        }
+        *remain = (long long)dr.remain();
+    } catch (const std::exception& e) {
+        std::fclose(f);
+        return fail(e.what());
+    }
+    std::fclose(f);
+    return (long)used;
 }
 
 }  // extern "C"

@@ -10,6 +10,7 @@
 #include <sstream>
 
 #include "../../include/otter_hip_int8.h"
+#include "otter_file.hpp"
 
 namespace otter {
 
@@ -492,8 +493,16 @@ int ConvolutionLayer::init_model() {
 }
 
 // order of the ncnn weight stream: Tensor/ConvolutionLayer.cpp:245-296
+// Tensor/ConvolutionLayer.cpp:245-293: Otter's own stream holds the bias before the weight and no scales; ncnn's
+// holds weight, bias, then the int8 scales
 int ConvolutionLayer::load_model(const Initializer& in) {
+    if (in.type != InitializerType::Ncnn) {
+        if (bias_term) bias_data = in.load({out_channels}, 1);
+        weight_data = in.load({out_channels, in_channels / groups, kernel_height, kernel_width}, 0);
+        return weight_data.defined() && (!bias_term || bias_data.defined()) ? 0 : -1;
+    }
     weight_data = in.load({out_channels, in_channels / groups, kernel_height, kernel_width}, 0);
+    if (!weight_data.defined()) return -1;
     if (bias_term) bias_data = in.load({out_channels}, 1);
     const bool dw = in_channels == groups && groups == out_channels;
     auto replicate = [&](const Tensor& one, int n) {
@@ -814,6 +823,306 @@ public:
     std::string type() const override { return "GlobalAvgPool"; }
 };
 
+// the fp32 layers that the reference's int8 model files put between their convolutions; every one takes a 4-D fp32
+// blob in any elempack on the device and leaves its result there
+static bool f32_4d(const Tensor& t) { return t.defined() && t.dim() == 4 && base_of(t.scalar_type()) == ScalarType::Float; }
+static int best_pack(int64_t channels) { return channels % 8 == 0 ? 8 : (channels % 4 == 0 ? 4 : 1); }
+static Tensor empty_f32_device(int64_t n, int64_t c, int64_t h, int64_t w) {
+    const int p = best_pack(c);  // what Net::convert_layout would hand to the next packing-aware layer
+    return Tensor::empty_device({n, c / p, h, w}, scalar_type_of(ScalarType::Float, p));
+}
+
+class MaxPoolLayer : public Layer {  // Tensor/MaxPoolLayer.cpp
+public:
+    MaxPoolLayer() {
+        one_blob_only = true;
+        support_packing = true;
+    }
+    int parse_param(LayerOption& o, ParamDict& pd) override {  // Tensor/MaxPoolLayer.cpp:26-72
+        auto pair = [&](const char* kh, const char* kw, const char* k, int def, int min_ok, int& h, int& w) {
+            h = opt_find_int(o, kh, -1), w = opt_find_int(o, kw, -1);
+            const int both = opt_find_int(o, k, def);
+            if (h < min_ok || w < min_ok) {
+                if (h < 0) h = both;
+                if (w < 0) w = both;
+            }
+        };
+        int sh, sw, kh, kw, ph, pw, dh, dw;
+        pair("stride_h", "stride_w", "stride", 1, 1, sh, sw);
+        kh = opt_find_int(o, "kernel_h", -1), kw = opt_find_int(o, "kernel_w", -1);
+        const int k = opt_find_int(o, "kernel", opt_find_int(o, "stride", 1));
+        if (kh < 1 || kw < 1) {
+            if (kh < 0) kh = k;
+            if (kw < 0) kw = k;
+        }
+        pair("padding_h", "padding_w", "padding", 0, 0, ph, pw);
+        pair("dilation_h", "dilation_w", "dilation", 1, 1, dh, dw);
+        pd.set(0, kh), pd.set(1, kw), pd.set(2, sh), pd.set(3, sw), pd.set(4, ph), pd.set(5, pw), pd.set(6, dh), pd.set(7, dw);
+        pd.set(8, opt_find(o, "ceil_mode") ? 1 : 0);
+        if (opt_find(o, "darknet_mode")) return -1;  // darknet's asymmetric padding: not on this path
+        return 0;
+    }
+    // Tensor/Pool.hpp:33-50
+    static int out_size(int in, int k, int p, int s, int d, bool ceil_mode) {
+        const int num = in + 2 * p - d * (k - 1) - 1 + (ceil_mode ? s - 1 : 0);
+        int out = (num >= 0 ? num / s : -((-num + s - 1) / s)) + 1;
+        if (ceil_mode && (out - 1) * s >= in + p) --out;
+        return out;
+    }
+    int compute_output_shape(ParamDict& pd) override {
+        const auto& in = bottom_shapes[0];
+        const bool cm = pd.get(8, 0) != 0;
+        top_shapes = {{in[0], in[1], out_size((int)in[2], pd.get(0, 3), pd.get(4, 0), pd.get(2, 1), pd.get(6, 1), cm),
+                       out_size((int)in[3], pd.get(1, 3), pd.get(5, 0), pd.get(3, 1), pd.get(7, 1), cm)}};
+        return 0;
+    }
+    int load_param(const ParamDict& pd) override {
+        kh_ = pd.get(0, 1), kw_ = pd.get(1, 1), sh_ = pd.get(2, 1), sw_ = pd.get(3, 1), ph_ = pd.get(4, 0), pw_ = pd.get(5, 0);
+        dh_ = pd.get(6, 1), dw_ = pd.get(7, 1), ceil_ = pd.get(8, 0) != 0;
+        return 0;
+    }
+    // Tensor/Pool.cpp:1185-1199: on x86 a packed blob (what Net::convert_layout makes of a channel count that is a
+    // multiple of 4) takes dedicated stride-2 kernels -- 3x3 for elempack 8 and 4, 2x2 for elempack 4 only (the
+    // elempack-8 branch repeats the 3x3 test) -- and those pad with zeros; everything else pads with -inf.
+    float pad_value(int64_t channels, const NetOption& opt) const {
+        const bool plain = !ceil_ && dh_ == 1 && dw_ == 1 && sh_ == 2 && sw_ == 2;
+        const int pack = !opt.use_packing_layout ? 1 : (channels % 8 == 0 ? 8 : (channels % 4 == 0 ? 4 : 1));
+        const bool k3 = kh_ == 3 && kw_ == 3, k2 = kh_ == 2 && kw_ == 2;
+        if (plain && ((k3 && pack != 1) || (k2 && pack == 4))) return 0.f;
+        return -__builtin_inff();
+    }
+    int forward(const Tensor& b, Tensor& top, const NetOption& opt) const override {
+        if (!f32_4d(b)) return -1;
+        const int H = (int)b.size(2), W = (int)b.size(3);
+        const int OH = out_size(H, kh_, ph_, sh_, dh_, ceil_), OW = out_size(W, kw_, pw_, sw_, dw_, ceil_);
+        if (OH < 1 || OW < 1) return -1;
+        top = empty_f32_device(b.size(0), b.channels(), OH, OW);
+        if (otter_hip_maxpool2d((const float*)b.device_ptr(), hip_layout_of(b.scalar_type()), (int)b.size(0), (int)b.channels(),
+                                H, W, kh_, kw_, sh_, sw_, ph_, pw_, dh_, dw_, OH, OW, pad_value(b.channels(), opt),
+                                (float*)top.device_ptr(), hip_layout_of(top.scalar_type()), nullptr))
+            return -1;
+        top.mark_device_written();
+        return 0;
+    }
+    std::string type() const override { return "MaxPool"; }
+
+private:
+    int kh_ = 1, kw_ = 1, sh_ = 1, sw_ = 1, ph_ = 0, pw_ = 0, dh_ = 1, dw_ = 1;
+    bool ceil_ = false;
+};
+
+class ConcatLayer : public Layer {  // Tensor/ConcatLayer.cpp, channel axis
+public:
+    ConcatLayer() { support_packing = true; }
+    int parse_param(LayerOption& o, ParamDict& pd) override {
+        pd.set(0, opt_find_int(o, "axis", 1));
+        return pd.get(0, 1) == 1 ? 0 : -1;  // the reference's model files concatenate channels only
+    }
+    int compute_output_shape(ParamDict&) override {
+        auto s = bottom_shapes[0];
+        for (size_t i = 1; i < bottom_shapes.size(); ++i) s[1] += bottom_shapes[i][1];
+        top_shapes = {s};
+        return 0;
+    }
+    int forward(const std::vector<Tensor>& b, std::vector<Tensor>& tops, const NetOption&) const override {
+        if (b.empty()) return -1;
+        int64_t C = 0;
+        for (const Tensor& t : b) {
+            if (!f32_4d(t) || t.size(0) != b[0].size(0) || t.size(2) != b[0].size(2) || t.size(3) != b[0].size(3)) return -1;
+            C += t.channels();
+        }
+        Tensor out = empty_f32_device(b[0].size(0), C, b[0].size(2), b[0].size(3));
+        int at = 0;
+        for (const Tensor& t : b) {
+            const int c = (int)t.channels();
+            if (otter_hip_copy_channels((const float*)t.device_ptr(), hip_layout_of(t.scalar_type()), c, 0,
+                                        (float*)out.device_ptr(), hip_layout_of(out.scalar_type()), (int)C, at, c,
+                                        (int)t.size(0), (int)t.size(2), (int)t.size(3), nullptr))
+                return -1;
+            at += c;
+        }
+        out.mark_device_written();
+        tops.assign(1, out);
+        return 0;
+    }
+    std::string type() const override { return "Concat"; }
+};
+
+class CropLayer : public Layer {  // Tensor/CropLayer.cpp, channel axis
+public:
+    CropLayer() {
+        one_blob_only = true;
+        support_packing = true;
+    }
+    int parse_param(LayerOption& o, ParamDict& pd) override {
+        pd.set(0, opt_find_int(o, "axis", 1)), pd.set(1, opt_find_int(o, "start", -1)), pd.set(2, opt_find_int(o, "end", -1));
+        return pd.get(0, 1) == 1 ? 0 : -1;
+    }
+    int compute_output_shape(ParamDict& pd) override {
+        auto s = bottom_shapes[0];
+        s[1] = pd.get(2, -1) - pd.get(1, -1);
+        top_shapes = {s};
+        return 0;
+    }
+    int load_param(const ParamDict& pd) override {
+        start_ = pd.get(1, -1), end_ = pd.get(2, -1);
+        return 0;
+    }
+    // native::slice on the logical channel index (Tensor/TensorShape.cpp:264-294): negative bounds count from the
+    // end, both are clamped to [0, C]
+    int forward(const Tensor& b, Tensor& top, const NetOption&) const override {
+        if (!f32_4d(b)) return -1;
+        const int C = (int)b.channels();
+        int lo = start_, hi = end_ == -1 ? C : end_;
+        if (lo < 0) lo += C;
+        if (hi < 0) hi += C;
+        lo = std::min(std::max(lo, 0), C);
+        hi = std::min(std::max(hi, lo), C);
+        if (hi == lo) return -1;
+        top = empty_f32_device(b.size(0), hi - lo, b.size(2), b.size(3));
+        if (otter_hip_copy_channels((const float*)b.device_ptr(), hip_layout_of(b.scalar_type()), C, lo, (float*)top.device_ptr(),
+                                    hip_layout_of(top.scalar_type()), hi - lo, 0, hi - lo, (int)b.size(0), (int)b.size(2),
+                                    (int)b.size(3), nullptr))
+            return -1;
+        top.mark_device_written();
+        return 0;
+    }
+    std::string type() const override { return "Crop"; }
+
+private:
+    int start_ = -1, end_ = -1;
+};
+
+class ChannelShuffleLayer : public Layer {  // Tensor/ChannelShuffleLayer.cpp
+public:
+    ChannelShuffleLayer() {
+        one_blob_only = true;
+        support_packing = true;  // the kernel reads and writes any elempack, so no unpacking round trip is needed
+    }
+    int parse_param(LayerOption& o, ParamDict& pd) override {
+        pd.set(0, opt_find_int(o, "groups", 1));
+        return 0;
+    }
+    int load_param(const ParamDict& pd) override {
+        groups_ = pd.get(0, 1);
+        return 0;
+    }
+    int forward(const Tensor& b, Tensor& top, const NetOption&) const override {
+        if (!f32_4d(b) || groups_ < 1 || b.channels() % groups_) return -1;
+        top = Tensor::empty_device(b.sizes(), b.scalar_type());
+        const int l = hip_layout_of(b.scalar_type());
+        if (otter_hip_channel_shuffle((const float*)b.device_ptr(), l, (float*)top.device_ptr(), l, (int)b.size(0),
+                                      (int)b.channels(), (int)b.size(2), (int)b.size(3), groups_, nullptr))
+            return -1;
+        top.mark_device_written();
+        return 0;
+    }
+    std::string type() const override { return "ChannelShuffle"; }
+
+private:
+    int groups_ = 1;
+};
+
+class ShortCutLayer : public Layer {  // Tensor/ShortCutLayer.cpp: element-wise sum of blobs of equal channel count
+public:
+    ShortCutLayer() { support_packing = true; }
+    int compute_output_shape(ParamDict&) override {
+        top_shapes = {bottom_shapes[0]};
+        return 0;
+    }
+    int forward(const std::vector<Tensor>& b, std::vector<Tensor>& tops, const NetOption&) const override {
+        if (b.size() < 2 || !f32_4d(b[0])) return -1;
+        Tensor acc = b[0];
+        for (size_t i = 1; i < b.size(); ++i) {
+            // different channel counts select darknet's partial shortcut, which the reference leaves unimplemented
+            if (!f32_4d(b[i]) || b[i].channels() != acc.channels() || b[i].size(2) != acc.size(2) || b[i].size(3) != acc.size(3))
+                return -1;
+            Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
+            Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
+            if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
+                                      (size_t)acc.numel() * acc.elempack(), nullptr))
+                return -1;
+            out.mark_device_written();
+            acc = out;
+        }
+        tops.assign(1, acc);
+        return 0;
+    }
+    std::string type() const override { return "ShortCut"; }
+};
+
+// Post-processing heads of the reference's model files (box decoding, NMS): host code outside the convolution path.
+// The layer type is known so that such a file compiles; asking for its output fails with -1 ("not supported",
+// Tensor/Layer.cpp:50-59) while every blob that feeds it can be extracted.
+class OffPathLayer : public Layer {
+public:
+    explicit OffPathLayer(const char* name) : name_(name) {}
+    int compute_output_shape(ParamDict&) override {
+        top_shapes.assign(tops.size(), bottom_shapes.empty() ? std::vector<int64_t>{1, 1, 1, 1} : bottom_shapes[0]);
+        return 0;
+    }
+    int forward(const std::vector<Tensor>&, std::vector<Tensor>&, const NetOption&) const override { return -1; }
+    std::string type() const override { return name_; }
+
+private:
+    const char* name_;
+};
+
+class UpsampleLayer : public Layer {  // Tensor/UpsampleLayer.cpp
+public:
+    UpsampleLayer() {
+        one_blob_only = true;
+        support_packing = true;
+    }
+    int parse_param(LayerOption& o, ParamDict& pd) override {  // Tensor/UpsampleLayer.cpp:25-60
+        const std::string m = opt_find_string(o, "upsample_mode", "nearest");
+        const int mode = m == "nearest" ? 1 : (m == "bilinear" ? 2 : (m == "bicubic" ? 3 : -1));
+        OTTER_CHECK(mode <= 2, "Unsupport upsample type");
+        pd.set(0, mode);
+        pd.set(1, opt_find_int(o, "output_height", 0)), pd.set(2, opt_find_int(o, "output_width", 0));
+        pd.set(3, opt_find_float(o, "scale_height", 1.f)), pd.set(4, opt_find_float(o, "scale_width", 1.f));
+        pd.set(5, opt_find_float(o, "stride", 1.f));
+        pd.set(6, opt_find(o, "align_corner") && o["align_corner"] != "false" ? 1 : 0);
+        return mode < 1 ? -1 : 0;
+    }
+    int compute_output_shape(ParamDict& pd) override {  // Tensor/UpsampleLayer.cpp:62-96
+        const auto& in = bottom_shapes[0];
+        int oh = pd.get(1, 0), ow = pd.get(2, 0);
+        float shf = pd.get(3, 0.f), swf = pd.get(4, 0.f);
+        const float stride = pd.get(5, 1.f);
+        if (oh && ow) shf = (float)(oh / in[2]), swf = (float)(ow / in[3]);
+        if (stride != 0) shf = swf = stride;
+        if (shf && swf) oh = (int)(in[2] * shf), ow = (int)(in[3] * swf);
+        pd.set(3, shf), pd.set(4, swf), pd.set(1, oh), pd.set(2, ow);
+        top_shapes = {{in[0], in[1], oh, ow}};
+        return 0;
+    }
+    int load_param(const ParamDict& pd) override {
+        mode_ = pd.get(0, 0), scale_h_ = pd.get(3, 0.f), scale_w_ = pd.get(4, 0.f), align_corner_ = pd.get(6, 0);
+        return 0;
+    }
+    // Tensor/UpsampleLayer.cpp:108-124: the output size from the scales; packed blobs go through otter::Interpolate,
+    // whose align_corners argument the layer leaves at its default (false). Blobs whose channel count is not a multiple
+    // of 4 take the reference's unpacked kernels, which interpolate differently: they are not on this path.
+    int forward(const Tensor& b, Tensor& top, const NetOption&) const override {
+        if (!f32_4d(b) || b.channels() % 4) return -1;
+        const int H = (int)b.size(2), W = (int)b.size(3);
+        const int OH = (int)(H * scale_h_), OW = (int)(W * scale_w_);
+        if (OH < 1 || OW < 1) return -1;
+        top = empty_f32_device(b.size(0), b.channels(), OH, OW);
+        if (otter_hip_upsample2d((const float*)b.device_ptr(), hip_layout_of(b.scalar_type()), (int)b.size(0), (int)b.channels(),
+                                 H, W, OH, OW, mode_, 0, (float*)top.device_ptr(), hip_layout_of(top.scalar_type()), nullptr))
+            return -1;
+        top.mark_device_written();
+        return 0;
+    }
+    std::string type() const override { return "Upsample"; }
+
+private:
+    int mode_ = 1, align_corner_ = 0;
+    float scale_h_ = 1.f, scale_w_ = 1.f;
+};
+
 }  // namespace
 
 // Tensor/InnerProductLayer.cpp (fp32 only in the reference as well)
@@ -877,6 +1186,14 @@ void register_hip_layers() {
     LayerRegistry::AddCreator("Split", []() -> Layer* { return new SplitLayer(); });
     LayerRegistry::AddCreator("InnerProduct", []() -> Layer* { return new InnerProductLayer(); });
     LayerRegistry::AddCreator("GlobalAvgPool", []() -> Layer* { return new GlobalAvgPoolLayer(); });
+    LayerRegistry::AddCreator("MaxPool", []() -> Layer* { return new MaxPoolLayer(); });
+    LayerRegistry::AddCreator("Concat", []() -> Layer* { return new ConcatLayer(); });
+    LayerRegistry::AddCreator("Crop", []() -> Layer* { return new CropLayer(); });
+    LayerRegistry::AddCreator("ChannelShuffle", []() -> Layer* { return new ChannelShuffleLayer(); });
+    LayerRegistry::AddCreator("ShortCut", []() -> Layer* { return new ShortCutLayer(); });
+    LayerRegistry::AddCreator("Upsample", []() -> Layer* { return new UpsampleLayer(); });
+    LayerRegistry::AddCreator("NanodetPlusDetectionOutput",
+                              []() -> Layer* { return new OffPathLayer("NanodetPlusDetectionOutput"); });
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -986,7 +1303,76 @@ void Net::compile(CompileMode mode) {
     }
 }
 
-// Tensor/Net.cpp:538-611: every layer reads its tensors from the stream in order, then builds its pipeline
+// Tensor/Net.cpp:518-536: one layer per block of the file, the block's name as its type, its parameters (those of
+// the nested `Param` block included) as its options
+int Net::load_otter(const char* model_structure, CompileMode compile_mode) {
+    core::OtterLeader leader;
+    if (!leader.readProject(model_structure)) return -1;
+    for (size_t i = 0; i < leader.teams_size(); ++i) {
+        LayerOption opt;
+        opt["type"] = leader.getTeamName((int)i);
+        for (const core::Param& p : leader.getTeamParams((int)i)) opt[p.type] = p.info;
+        addLayer(opt);
+    }
+    compile(compile_mode);
+    return 0;
+}
+
+// Tensor/Net.cpp:538-586
+int Net::load_weight(const char* weight_path, WeightType type) {
+    FILE* fp = std::fopen(weight_path, "rb");
+    if (!fp) {
+        std::fprintf(stderr, "Open weight file fail!\n");
+        return -1;
+    }
+    const int status = load_weight(fp, type);
+    std::fclose(fp);
+    return status;
+}
+
+int Net::load_weight(FILE* f, WeightType type) {
+    if (layers_.empty()) {
+        std::fprintf(stderr, "[Net] Empty graph!\n");
+        return -1;
+    }
+    DataReaderFromStdio dr(f);
+    if (type == WeightType::Ncnn) {
+        InitializerNcnnFromDataReader initializer(dr);
+        const int ret = load_weight(initializer);
+        const size_t remain = dr.remain();
+        if (remain) std::printf("Network may initialize fail, remain weight %zd\n", remain);
+        return remain || ret;
+    }
+    int version[2];  // Tensor/Net.cpp:507-516: Otter's stream starts with major / minor
+    if (dr.read(version, sizeof(version)) != sizeof(version)) return -1;
+    InitializerFromDataReader initializer(dr);
+    return load_weight(initializer);
+}
+
+const std::vector<std::string> Net::blob_names() const {
+    std::vector<std::string> v;
+    for (const Blob& b : blobs_) v.push_back(b.name);
+    return v;
+}
+
+std::string Net::describe() const {
+    std::ostringstream o;
+    for (const Layer* l : layers_) {
+        auto join = [&](const std::vector<int>& v) {
+            std::string s;
+            for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + blobs_[v[i]].name;
+            return s.empty() ? std::string("-") : s;
+        };
+        o << l->type() << ' ' << l->name << ' ' << join(l->bottoms) << ' ' << join(l->tops);
+        if (const auto* c = dynamic_cast<const ConvolutionLayer*>(l))
+            o << ' ' << c->out_channels << ' ' << c->in_channels << ' ' << c->groups << ' ' << c->kernel_height << ' '
+              << c->kernel_width << ' ' << c->bias_term << ' ' << c->int8_scale_term;
+        o << '\n';
+    }
+    return o.str();
+}
+
+// Tensor/Net.cpp:588-611: every layer reads its tensors from the stream in order, then builds its pipeline
 int Net::load_weight(const Initializer& initializer) {
     for (Layer* l : layers_) {
         int rc = l->load_model(initializer);

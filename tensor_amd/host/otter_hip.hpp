@@ -121,10 +121,12 @@ std::string opt_find_string(const LayerOption& o, const std::string& k, const st
 
 // Weight source of load_model (Tensor/Initializer.hpp): hands out consecutive tensors of a weight stream.
 // type 0 = weight (may be int8), 1 = fp32 vector.
+enum class InitializerType { Otter, Ncnn };
 class Initializer {
 public:
     virtual ~Initializer() = default;
     virtual Tensor load(const std::vector<int64_t>& shape, int type) const = 0;
+    InitializerType type = InitializerType::Ncnn;  // decides the order in which a layer asks for its tensors
 };
 
 // Tensor/Layer.hpp:23-62
@@ -243,8 +245,15 @@ public:
     ~Net();
     void addLayer(LayerOption option);
     void compile(CompileMode mode = CompileMode::Initial);
+    // Tensor/Net.hpp:38-48: a `.otter` description, then a weight stream (Otter's fp32 stream or ncnn's `.bin`)
+    enum class WeightType { Otter, Ncnn };
+    int load_otter(const char* model_structure, CompileMode compile_mode);
+    int load_weight(const char* weight_path, WeightType type = WeightType::Otter);
+    int load_weight(FILE* f, WeightType type = WeightType::Otter);
     int load_weight(const Initializer& initializer);
     Extractor create_extractor() const;
+    const std::vector<std::string> blob_names() const;
+    std::string describe() const;  // one line per layer: type, name, bottoms, tops, convolution shape
     int find_blob_index_by_name(const std::string& name) const;
     Layer* layer_by_name(const std::string& name) const;
     size_t layer_count() const { return layers_.size(); }

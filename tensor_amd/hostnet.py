@@ -12,7 +12,8 @@ EXPORTS = ["otter_host_last_error", "otter_host_net_create", "otter_host_net_des
            "otter_host_net_compile", "otter_host_net_set_conv", "otter_host_net_get_scale_in",
            "otter_host_net_set_inner_product", "otter_host_net_run", "otter_host_session_create",
            "otter_host_session_pass", "otter_host_session_fetch", "otter_host_session_destroy",
-           "otter_host_functional_chain"]
+           "otter_host_functional_chain", "otter_host_net_load_otter", "otter_host_net_load_weight",
+           "otter_host_net_describe", "otter_host_net_eval", "otter_host_otter_dump", "otter_host_ncnn_read"]
 
 
 def load_cdll():
@@ -23,6 +24,9 @@ def load_cdll():
     lib.otter_host_net_create.restype = C.c_void_p
     lib.otter_host_session_create.restype = C.c_void_p
     lib.otter_host_session_fetch.restype = C.c_long
+    lib.otter_host_net_describe.restype = C.c_long
+    lib.otter_host_otter_dump.restype = C.c_long
+    lib.otter_host_ncnn_read.restype = C.c_long
     return lib
 
 
@@ -95,6 +99,48 @@ class Net:
     def session(self, in_name, x, out_name):
         return Session(self, in_name, x, out_name)
 
+    # ---- model files (Net::load_otter / Net::load_weight of the reference) ----
+    def load_otter(self, path, initial=False):
+        self._check(self.lib.otter_host_net_load_otter(self.h, os.fsencode(path), int(initial)))
+
+    def load_weight(self, path, ncnn=True):
+        self._check(self.lib.otter_host_net_load_weight(self.h, os.fsencode(path), int(ncnn)))
+
+    def describe(self):
+        """[(type, name, [bottom blobs], [top blobs], conv_shape or None)], conv_shape = dict(K, C, groups, kh, kw,
+        bias_term, int8_scale_term)."""
+        buf = C.create_string_buffer(1 << 22)
+        n = self.lib.otter_host_net_describe(self.h, buf, C.c_size_t(len(buf)))
+        if n < 0:
+            raise HostError(self.lib.otter_host_last_error().decode())
+        out = []
+        for line in buf.value.decode().splitlines():
+            f = line.split(" ")
+            conv = None
+            if len(f) > 4:
+                conv = dict(zip(("K", "C", "groups", "kh", "kw", "bias_term", "int8_scale_term"), map(int, f[4:11])))
+            out.append((f[0], f[1], [] if f[2] == "-" else f[2].split(","), [] if f[3] == "-" else f[3].split(","), conv))
+        return out
+
+    def eval(self, inputs, out_name):
+        """One pass with the blobs of `inputs` (name -> NCHW fp32 / int8 array) set beforehand; returns `out_name`
+        unpacked (Extractor::input + Extractor::extract(name, type 0))."""
+        names = [k.encode() for k in inputs]
+        arrs = [np.ascontiguousarray(v) for v in inputs.values()]
+        n = len(arrs)
+        c_names = (C.c_char_p * n)(*names)
+        c_ptrs = (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
+        c_i8 = (C.c_int * n)(*[int(a.dtype == np.int8) for a in arrs])
+        c_shapes = (C.c_int64 * (4 * n))(*[d for a in arrs for d in a.shape])
+        dtype, shape = C.c_int(), (C.c_int64 * 4)()
+        cap = 1 << 28
+        buf = np.empty(cap, np.uint8)
+        self._check(self.lib.otter_host_net_eval(self.h, n, c_names, c_ptrs, c_i8, c_shapes, out_name.encode(),
+                                                 buf.ctypes.data_as(C.c_void_p), C.c_size_t(cap), C.byref(dtype), shape))
+        np_dt = [np.float32, np.int8, np.int32][dtype.value]
+        count = int(np.prod(tuple(shape)))
+        return buf[:count * np.dtype(np_dt).itemsize].view(np_dt).reshape(tuple(shape)).copy()
+
     def close(self):
         if self.h:
             self.lib.otter_host_net_destroy(self.h)
@@ -152,3 +198,44 @@ def functional_chain(x, in_scale, wq, scale_in, bias, *, stride=1, pad=0, groups
     if rc != 0:
         raise HostError(lib.otter_host_last_error().decode(errors="replace"))
     return acc, out
+
+
+def otter_dump(path, lib=None):
+    """What the `.otter` parser makes of a file: 'N name', 'G key=value', 'T block', 'P key=value' lines."""
+    lib = lib or load_cdll()
+    buf = C.create_string_buffer(1 << 24)
+    n = lib.otter_host_otter_dump(os.fsencode(path), buf, C.c_size_t(len(buf)))
+    if n < 0:
+        raise HostError(lib.otter_host_last_error().decode())
+    return buf.raw[:n].decode(errors="surrogateescape")
+
+
+def ncnn_read(path, shapes, kinds, reader=None, err=None):
+    """Reads consecutive tensors from an ncnn `.bin` with InitializerNcnnFromDataReader. shapes: list of tuples
+    (<= 4 dims), kinds: 0 weight (tagged) / 1 plain fp32. Returns ([array or None], bytes left in the file).
+    `reader` / `err`: the same entry point of another library (the compiled reference's, in the tests)."""
+    if reader is None:
+        lib = load_cdll()
+        reader, err = lib.otter_host_ncnn_read, lib.otter_host_last_error
+    n = len(shapes)
+    flat = (C.c_longlong * (4 * n))(*[(list(s) + [0] * 4)[:4][d] for s in shapes for d in range(4)])
+    c_kinds = (C.c_int * n)(*kinds)
+    dtypes = (C.c_int * n)()
+    cap = 4 * sum(int(np.prod(s)) for s in shapes) + 64
+    out = np.empty(cap, np.uint8)
+    remain = C.c_longlong(-1)
+    reader.restype = C.c_long
+    used = reader(os.fsencode(path), n, flat, c_kinds, dtypes, out.ctypes.data_as(C.c_void_p), C.c_size_t(cap),
+                  C.byref(remain))
+    if used < 0:
+        raise HostError(err().decode() if err else "ncnn_read failed")
+    res, at = [], 0
+    for s, dt in zip(shapes, dtypes):
+        if dt < 0:
+            res.append(None)
+            continue
+        np_dt = np.int8 if dt == 1 else np.float32
+        nb = int(np.prod(s)) * np.dtype(np_dt).itemsize
+        res.append(out[at:at + nb].view(np_dt).reshape(s).copy())
+        at += nb
+    return res, remain.value

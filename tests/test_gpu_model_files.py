@@ -1,0 +1,184 @@
+"""Model files on the GPU: the reference's own int8 detection model description (benchmark/
+nanodet-plus-m-1.5x_416_int8_fused.otter, kept as a data file under tests/golden) is read by Net::load_otter, filled
+with synthetic int8 weights through an ncnn `.bin` read by Net::load_weight, and run on the GPU -- against the compiled
+reference's Net reading the same two files on the CPU (oracle/_ref travels with the tree; the reference sources do
+not). Small generated descriptions drive each fp32 glue layer alone through the same two Nets."""
+import os
+
+import numpy as np
+import pytest
+
+from tensor_amd import hostnet, modelfile
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+NANODET = os.path.join(GOLDEN, "nanodet-plus-m-1.5x_416_int8_fused.otter")
+HEADS = ["conv_95", "conv_100", "conv_105", "conv_110"]  # what feeds the detection post-processing
+
+
+@pytest.fixture(scope="module")
+def detector(ref, tmp_path_factory):
+    rng = np.random.default_rng(11)
+    net = hostnet.Net(lightmode=False)
+    net.load_otter(NANODET)
+    layers = net.describe()
+    blob, _ = modelfile.synthetic_int8_weights(layers, rng)
+    path = str(tmp_path_factory.mktemp("nanodet") / "nanodet_int8.bin")
+    with open(path, "wb") as f:
+        f.write(blob)
+    net.load_weight(path, ncnn=True)
+    rnet = ref.net(NANODET, path)
+    alias = {}  # blobs of the automatic Split layers -> the blob they share
+    for typ, _name, bottoms, tops, _conv in layers:
+        if typ == "Split":
+            for t in tops:
+                alias[t] = bottoms[0]
+    real = [l for l in layers if l[0] not in ("Input", "Split", "NanodetPlusDetectionOutput")]
+    return dict(net=net, rnet=rnet, layers=layers, real=real, alias=alias, rng=rng)
+
+
+def test_description_compiles_to_the_reference_graph(detector):
+    types = [l[0] for l in detector["layers"]]
+    assert types.count("Convolution") == 110 and types.count("Concat") == 28 and types.count("Crop") == 26
+    assert types.count("ChannelShuffle") == 16 and types.count("ShortCut") == 5 and types.count("Upsample") == 2
+    conv = {l[1]: l[4] for l in detector["layers"] if l[0] == "Convolution"}
+    assert conv["conv_1"] == dict(K=24, C=3, groups=1, kh=3, kw=3, bias_term=1, int8_scale_term=2)
+    assert conv["conv_2"]["groups"] == 24 and conv["conv_2"]["int8_scale_term"] == 101
+
+
+def test_every_layer_against_the_reference_on_the_reference_inputs(detector):
+    """Each layer of the GPU Net gets the reference's blobs as its inputs (Extractor::input) and must reproduce the
+    reference's output blob: int8 bit for bit, fp32 within 1e-5 relative (the glue layers move or add floats and the
+    bilinear arithmetic is restated operation by operation, so they are expected to be exact as well)."""
+    net, rnet, real, alias = detector["net"], detector["rnet"], detector["real"], detector["alias"]
+    x = detector["rng"].uniform(0, 1, (1, 3, 416, 416)).astype(np.float32)
+    names = [l[3][0] for l in real]
+    blobs, _ = rnet.run("data_1", x, names[::-1])
+    blobs["data_1"] = x
+    inexact = []
+    n_int8 = 0
+    for typ, name, bottoms, tops, _conv in real:
+        got = net.eval({b: blobs[alias.get(b, b)] for b in bottoms}, tops[0])
+        want = blobs[tops[0]]
+        assert got.shape == want.shape and got.dtype == want.dtype, (typ, name)
+        if got.dtype == np.int8:
+            n_int8 += 1
+            np.testing.assert_array_equal(got, want, err_msg="%s %s" % (typ, name))
+            assert np.abs(want).max() > 20 and (np.abs(want) == 127).mean() < 0.3, "degenerate activations at " + name
+        else:
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6, err_msg="%s %s" % (typ, name))
+            if not np.array_equal(got, want):
+                inexact.append(name)
+    assert n_int8 == 59  # the convolutions with int8_scale_term 101 / 102
+    assert not [n for n in inexact if not n.startswith("conv_")], inexact  # glue layers: exact
+
+
+def test_whole_network_free_running_and_batched(detector):
+    """The GPU Net on its own from the image to the four head blobs, and a batch of two images at once (the reference
+    runs one image at a time): every image must come out as the reference computes it alone."""
+    net, rnet = detector["net"], detector["rnet"]
+    xs = detector["rng"].uniform(0, 1, (2, 3, 416, 416)).astype(np.float32)
+    want = [rnet.run("data_1", xs[i:i + 1], HEADS)[0] for i in range(2)]
+    for h in HEADS:
+        both = net.eval({"data_1": xs}, h)
+        for i in range(2):
+            one = net.eval({"data_1": xs[i:i + 1]}, h)
+            np.testing.assert_array_equal(one, both[i:i + 1], err_msg="image %d alone vs in the batch, %s" % (i, h))
+            np.testing.assert_allclose(one, want[i][h], rtol=1e-5, atol=1e-5, err_msg="%s image %d" % (h, i))
+
+
+def test_detection_output_is_off_the_path(detector):
+    with pytest.raises(hostnet.HostError):
+        detector["net"].eval({"data_1": np.zeros((1, 3, 416, 416), np.float32)}, "nanodet")
+
+
+# -------------------------------------------------------------------------------------------------
+# the glue layers one at a time, through generated descriptions
+# -------------------------------------------------------------------------------------------------
+def _otter(c, h, w, body):
+    return ('name: "glue"\nInput {\n name: data\n output: data\n Param {\n  height: %d\n  width: %d\n  channel: %d\n }\n}\n'
+            % (h, w, c)) + body
+
+
+def _layer(typ, name, inputs, **params):
+    s = '%s {\n name: %s\n input: "%s"\n output: %s\n Param {\n' % (typ, name, ", ".join(inputs), name)
+    for k, v in params.items():
+        s += "  %s: %s\n" % (k, v)
+    return s + " }\n}\n"
+
+
+# The reference's Concat goes wrong when its inputs arrive in different elempacks (a Float4 blob followed by a
+# Float8 one: the channels of the second land in the wrong place) -- its own unpacked mode and plain numpy agree with
+# each other and with the GPU layer there. Cases marked "unpacked" are therefore checked against the reference's Net
+# with use_packing_layout off; every other case against the packed Net, which is what the GPU layers mirror (the
+# zero padding of the packed stride-2 pooling kernels included).
+UNPACKED_REFERENCE = {"shuffle_crop_concat", "crop_unaligned"}
+
+GLUE_CASES = [
+    # name, input (C, H, W), description body, blobs to compare
+    ("maxpool_3x3s2_pack8", (8, 13, 11), _layer("MaxPool", "p", ["data"], kernel=3, stride=2, padding=1), ["p"]),
+    ("maxpool_3x3s2_pack4", (12, 10, 10), _layer("MaxPool", "p", ["data"], kernel=3, stride=2, padding=1), ["p"]),
+    ("maxpool_3x3s2_unpacked", (6, 10, 9), _layer("MaxPool", "p", ["data"], kernel=3, stride=2, padding=1), ["p"]),
+    ("maxpool_2x2s2_pack4", (4, 9, 9), _layer("MaxPool", "p", ["data"], kernel=2, stride=2, padding=1), ["p"]),
+    ("maxpool_2x2s2_pack8", (8, 9, 9), _layer("MaxPool", "p", ["data"], kernel=2, stride=2, padding=1), ["p"]),
+    ("maxpool_3x3s1", (8, 7, 9), _layer("MaxPool", "p", ["data"], kernel=3, stride=1, padding=1), ["p"]),
+    ("maxpool_5x3_dilated", (4, 15, 14), _layer("MaxPool", "p", ["data"], kernel_h=5, kernel_w=3, stride_h=2, stride_w=3,
+                                                 padding_h=2, padding_w=1, dilation_h=2, dilation_w=1), ["p"]),
+    ("upsample_bilinear_x2", (8, 5, 7), _layer("Upsample", "u", ["data"], stride="2.000000", align_corner="false",
+                                               upsample_mode="bilinear"), ["u"]),
+    ("upsample_bilinear_x3_pack4", (12, 4, 3), _layer("Upsample", "u", ["data"], stride="3.000000",
+                                                     upsample_mode="bilinear"), ["u"]),
+    ("upsample_nearest_x2", (16, 6, 5), _layer("Upsample", "u", ["data"], stride="2.000000", upsample_mode="nearest"), ["u"]),
+    ("shuffle_crop_concat", (24, 6, 5),
+     _layer("ChannelShuffle", "s", ["data"], groups=3) + _layer("Crop", "c1", ["s"], start=0, end=8, axis=1) +
+     _layer("Crop", "c2", ["s"], start=8, end=20, axis=1) + _layer("Crop", "c3", ["s"], start=20, end=24, axis=1) +
+     _layer("Concat", "cat", ["c3", "c1", "c2"], axis=1) + _layer("ChannelShuffle", "s2", ["cat"], groups=2),
+     ["s", "c1", "c2", "c3", "cat", "s2"]),
+    ("crop_unaligned", (12, 4, 4), _layer("Crop", "c", ["data"], start=3, end=10, axis=1) +
+     _layer("Concat", "cat", ["c", "data"], axis=1), ["c", "cat"]),
+    ("shortcut", (16, 5, 5), _layer("MaxPool", "p", ["data"], kernel=3, stride=1, padding=1) +
+     "ShortCut {\n name: add\n input: \"p, data\"\n output: add\n}\n", ["add"]),
+]
+
+
+@pytest.mark.parametrize("case", GLUE_CASES, ids=[c[0] for c in GLUE_CASES])
+def test_glue_layer_against_the_reference(ref, tmp_path, case):
+    name, (c, h, w), body, outs = case
+    path = str(tmp_path / (name + ".otter"))
+    with open(path, "w") as f:
+        f.write(_otter(c, h, w, body))
+    rng = np.random.default_rng(sum(map(ord, name)))
+    x = rng.normal(0, 1, (2, c, h, w)).astype(np.float32)
+    x[:, :, 0, :] -= 3.0  # a border where every tap is negative: zero padding and -inf padding then differ
+    net = hostnet.Net(lightmode=False)
+    net.load_otter(path, initial=True)
+    rnet = ref.net(path, use_packing=name not in UNPACKED_REFERENCE)
+    for o in outs:
+        got = net.eval({"data": x}, o)
+        for i in range(2):
+            want = rnet.run("data", x[i:i + 1], [o])[0][o]
+            np.testing.assert_array_equal(got[i:i + 1], want, err_msg="%s blob %s image %d" % (name, o, i))
+
+
+def test_concat_of_mixed_packs_is_the_plain_concatenation(tmp_path):
+    """4 + 8 + 12 channels (elempack 4, 8, 4): against numpy."""
+    path = str(tmp_path / "cat.otter")
+    body = (_layer("Crop", "a", ["data"], start=20, end=24, axis=1) + _layer("Crop", "b", ["data"], start=0, end=8, axis=1) +
+            _layer("Crop", "c", ["data"], start=8, end=20, axis=1) + _layer("Concat", "cat", ["a", "b", "c"], axis=1))
+    with open(path, "w") as f:
+        f.write(_otter(24, 5, 7, body))
+    x = np.random.default_rng(3).normal(0, 1, (3, 24, 5, 7)).astype(np.float32)
+    net = hostnet.Net()
+    net.load_otter(path, initial=True)
+    np.testing.assert_array_equal(net.eval({"data": x}, "cat"), np.concatenate([x[:, 20:24], x[:, 0:8], x[:, 8:20]], 1))
+
+
+def test_bilinear_upsample_of_an_unpackable_blob_is_refused(tmp_path):
+    path = str(tmp_path / "u.otter")
+    with open(path, "w") as f:
+        f.write(_otter(6, 4, 4, _layer("Upsample", "u", ["data"], stride="2.000000", upsample_mode="bilinear")))
+    net = hostnet.Net()
+    net.load_otter(path, initial=True)
+    with pytest.raises(hostnet.HostError):
+        net.eval({"data": np.zeros((1, 6, 4, 4), np.float32)}, "u")

@@ -197,6 +197,50 @@ def build_c0(hip, capi, rng):
                 shape=(N, C, H, W))
 
 
+def build_det(hip, capi, rng, batch=16):
+    """The reference's own int8 detection model description (benchmark/nanodet-plus-m-1.5x_416_int8_fused.otter, a data
+    file kept under tests/golden) read by Net::load_otter, with synthetic int8 weights written as an ncnn .bin and read by
+    Net::load_weight: 110 int8 convolutions and the fp32 glue between them, from the image to the four head blobs."""
+    import tempfile
+    from tensor_amd import hostnet, modelfile
+    otter = os.path.join(ROOT, "tests", "golden", "nanodet-plus-m-1.5x_416_int8_fused.otter")
+    net = hostnet.Net()
+    net.load_otter(otter)
+    layers = net.describe()
+    blob, _ = modelfile.synthetic_int8_weights(layers, rng)
+    tmp = tempfile.mkdtemp(prefix="otter_det_")
+    bin_path = os.path.join(tmp, "nanodet_int8.bin")
+    with open(bin_path, "wb") as f:
+        f.write(blob)
+    net.load_weight(bin_path, ncnn=True)
+    x = rng.uniform(0, 1, (batch, 3, 416, 416)).astype(np.float32)
+    sess = net.session("data_1", x, "conv_95,conv_100,conv_105,conv_110")
+    n_layers = sum(l[0] not in ("Input", "Split", "NanodetPlusDetectionOutput") for l in layers)
+    # algorithmic work per image: convolution MACs; bytes = every layer's output written once and read once per
+    # consumer (int8 where the convolution requantizes, fp32 elsewhere) + the image
+    alias = {t: l[2][0] for l in layers if l[0] == "Split" for t in l[3]}
+    readers = {}
+    for l in layers:
+        if l[0] != "Split":
+            for b in l[2]:
+                readers[alias.get(b, b)] = readers.get(alias.get(b, b), 0) + 1
+    macs = 0
+    act_bytes = 4 * 3 * 416 * 416
+    for typ, _name, _bottoms, tops, c, (_, C, H, W) in layers:
+        if typ in ("Input", "Split", "NanodetPlusDetectionOutput"):
+            continue
+        esz = 1 if (c and c["int8_scale_term"] > 100) else 4
+        act_bytes += C * H * W * esz * (1 + max(1, readers.get(tops[0], 1)))
+        if c:
+            macs += c["K"] * (c["C"] // c["groups"]) * c["kh"] * c["kw"] * H * W
+    return dict(name="det", step=sess.run, ops=2.0 * macs * batch, launches=n_layers, images=batch,
+                dom_ops=2.0 * macs * batch, dom_bytes=float(act_bytes) * batch,
+                bound="hbm", workload="nanodet-plus-m-1.5x int8 (the reference's .otter description, synthetic ncnn .bin "
+                "weights), %dx3x416x416 fp32 in, through otter::Net: 110 int8 convolutions + %d fp32 glue layers, to the "
+                "four head blobs" % (batch, n_layers - 110), dom_kernel="whole network (all kernels of one forward pass)",
+                dom_fn=None, x=x, params=[], shape=(batch, 3, 416, 416), otter=otter, bin=bin_path, _keep=(net, sess))
+
+
 def build_copy(hip, capi, rng):
     """Calibration workload for the rocprofv3 FETCH_SIZE / WRITE_SIZE counters: a plain device copy of 256 MiB."""
     torch = hip.torch
@@ -271,6 +315,14 @@ def cpu_baseline(wl, budget_s=15.0):
                     sample="%d images, scalar C restatement" % n_img)
     if name == "copy":
         return None
+    if name == "det":
+        # the reference's own Net on the same two files, one image at a time, in a child process
+        import subprocess
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--det-cpu-child", wl["otter"], wl["bin"]],
+                           capture_output=True, text=True, timeout=300)
+        if r.returncode != 0:
+            raise RuntimeError("det CPU child failed (%d): %s" % (r.returncode, r.stderr[-200:]))
+        return json.loads(r.stdout.strip().splitlines()[-1])
     if name == "c4":
         # the reference layer by layer in a child process (a crash or hang in it must not take the GPU figures along)
         import subprocess
@@ -339,6 +391,25 @@ def c4_cpu_child():
                                  "included")))
 
 
+def det_cpu_child(otter, bin_path):
+    """Times the compiled reference's Net (load_otter + load_weight, then Extractor::extract of the four heads) on a
+    few images, one at a time as the reference runs them."""
+    from oracle import binding
+    R = binding.Ref()
+    net = R.net(otter, bin_path)
+    rng = np.random.default_rng(1)
+    heads = ["conv_95", "conv_100", "conv_105", "conv_110"]
+    best = None
+    for _ in range(6):
+        x = rng.uniform(0, 1, (1, 3, 416, 416)).astype(np.float32)
+        t0 = time.perf_counter()
+        net.run("data_1", x, heads)
+        t = time.perf_counter() - t0
+        best = t if best is None else min(best, t)
+    print(json.dumps(dict(value=1.0 / best, unit="images/s", cores=R.num_threads(), kind="reference",
+                          sample="6 single images through the reference's Net (same .otter and .bin), min")))
+
+
 def measured_traffic(name):
     """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 --pmc summary
     (profiles/hbm_traffic.json: FETCH_SIZE / WRITE_SIZE scaled by a copy-kernel calibration); None if not profiled."""
@@ -381,6 +452,10 @@ def main():
     if "--c4-cpu-child" in sys.argv:
         c4_cpu_child()
         return
+    if "--det-cpu-child" in sys.argv:
+        i = sys.argv.index("--det-cpu-child")
+        det_cpu_child(sys.argv[i + 1], sys.argv[i + 2])
+        return
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
@@ -408,16 +483,20 @@ def main():
         builders["c4"] = lambda r: mobilenet.build_bench(hip, capi, r)
     except ImportError:
         pass
+    builders["det"] = lambda r: build_det(hip, capi, r)
     if a.workload not in builders:
         print("unknown workload %s (have %s)" % (a.workload, sorted(builders)), file=sys.stderr)
         sys.exit(2)
 
     wl = builders[a.workload](np.random.default_rng(0))
-    unit = "images/s" if wl["name"] == "c4" else ("GB/s" if "bytes" in wl else "TOPS")
+    unit = "images/s" if wl["name"] in ("c4", "det") else ("GB/s" if "bytes" in wl else "TOPS")
     res = measure(wl, timer, a.steps, a.warmup, unit)
     if wl["name"] == "c4":
         value = wl["images"] / (res["ms_per_step"] * 1e-3)
         metric = "MobileNetV2-style int8 net images/sec b64"
+    elif wl["name"] == "det":
+        value = wl["images"] / (res["ms_per_step"] * 1e-3)
+        metric = "int8 detection model (reference .otter description) images/sec b16"
     elif unit == "TOPS":
         value = res["tops"]
         metric = "int8 conv TOPS"
@@ -438,13 +517,13 @@ def main():
             line["cpu_baseline"] = {"error": str(e)[:200]}
     if not a.no_also:
         also = []
-        for name in ("c1s1", "c1s2", "c2", "c0", "c4"):
+        for name in ("c1s1", "c1s2", "c2", "c0", "c4", "det"):
             if name == a.workload or name not in builders:
                 continue
             w2 = builders[name](np.random.default_rng(0))
             r2 = measure(w2, timer, max(10, a.steps // 2), a.warmup, "")
             entry = dict(name=name, **r2)
-            if name == "c4":
+            if name in ("c4", "det"):
                 entry["images_per_s"] = w2["images"] / (r2["ms_per_step"] * 1e-3)
             if not a.no_cpu and name != "c4":
                 try:

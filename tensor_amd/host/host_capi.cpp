@@ -100,6 +100,25 @@ int otter_host_net_set_conv(void* net, const char* layer_name, const int8_t* wei
     }
 }
 
+// Calibration aid: while `on`, an int8-output convolution (int8_scale_term > 100) runs as its fp32-output twin
+// (int8_scale_term - 100: same weights and input scale, dequantize + activation instead of requantize), so that a
+// calibrator can look at the values its output scale has to cover. `on` = 0 restores the layer.
+int otter_host_net_conv_fp32_probe(void* net, const char* layer_name, int on) {
+    try {
+        Net* n = static_cast<Net*>(net);
+        auto* L = dynamic_cast<ConvolutionLayer*>(n->layer_by_name(layer_name));
+        if (!L) return fail(std::string("no Convolution layer named ") + layer_name);
+        if (on && L->int8_scale_term > 100) L->int8_scale_term -= 100;
+        else if (!on && L->int8_scale_term > 0 && L->int8_scale_term < 100 && L->top_blob_int8_scales.defined()) L->int8_scale_term += 100;
+        else return 0;
+        const int rc = L->create_pipeline(n->option);
+        if (rc) return fail(std::string("create_pipeline: ") + otter_hip_last_error());
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+
 int otter_host_net_get_scale_in(void* net, const char* layer_name, float* out) {
     auto* L = dynamic_cast<ConvolutionLayer*>(static_cast<Net*>(net)->layer_by_name(layer_name));
     if (!L || !L->scale_in_data.defined()) return fail("no such layer / pipeline not built");
@@ -161,7 +180,8 @@ int otter_host_net_run(void* net, const char* in_name, const void* x, int x_is_i
 }
 
 // A session keeps the input resident on the device and runs passes without synchronising, so that a caller can time
-// a stream of passes with its own events.
+// a stream of passes with its own events. out_name may list several blobs separated by commas (the heads of a
+// detection network): a pass extracts every one of them from the same Extractor, the fetch returns the last.
 struct otter_host_session {
     Net* net;
     std::string in_name, out_name;
@@ -189,8 +209,14 @@ int otter_host_session_pass(void* session) {
         auto* s = static_cast<otter_host_session*>(session);
         Extractor ex = s->net->create_extractor();
         if (ex.input(s->in_name, s->in)) return fail("no such input blob");
-        const int rc = ex.extract(s->out_name, s->out, 1);
-        if (rc) return fail("forward failed with code " + std::to_string(rc) + ": " + otter_hip_last_error());
+        size_t pos = 0;
+        while (pos <= s->out_name.size()) {
+            size_t e = s->out_name.find(',', pos);
+            if (e == std::string::npos) e = s->out_name.size();
+            const int rc = ex.extract(s->out_name.substr(pos, e - pos), s->out, 1);
+            if (rc) return fail("forward failed with code " + std::to_string(rc) + ": " + otter_hip_last_error());
+            pos = e + 1;
+        }
         return 0;
     } catch (const std::exception& e) {
         return fail(e.what());
@@ -263,8 +289,8 @@ int otter_host_net_load_weight(void* net, const char* path, int ncnn) {
     }
 }
 
-// One line per layer, "type name bottoms tops" and for a convolution its shape as load_model will ask for it:
-// "Convolution conv_1 data_1 conv_1 K C groups kh kw bias_term int8_scale_term".
+// One line per layer, "type name bottoms tops N C H W" (the logical shape of its first top blob) and for a convolution
+// its weights as load_model will ask for them: "... K C groups kh kw bias_term int8_scale_term".
 long otter_host_net_describe(void* net, char* buf, size_t capacity) {
     try {
         const std::string out = static_cast<Net*>(net)->describe();

@@ -1364,6 +1364,7 @@ std::string Net::describe() const {
             return s.empty() ? std::string("-") : s;
         };
         o << l->type() << ' ' << l->name << ' ' << join(l->bottoms) << ' ' << join(l->tops);
+        for (int d = 0; d < 4; ++d) o << ' ' << (l->top_shapes.empty() ? 0 : l->top_shapes[0][d]);
         if (const auto* c = dynamic_cast<const ConvolutionLayer*>(l))
             o << ' ' << c->out_channels << ' ' << c->in_channels << ' ' << c->groups << ' ' << c->kernel_height << ' '
               << c->kernel_width << ' ' << c->bias_term << ' ' << c->int8_scale_term;

@@ -253,7 +253,7 @@ public:
     int load_weight(const Initializer& initializer);
     Extractor create_extractor() const;
     const std::vector<std::string> blob_names() const;
-    std::string describe() const;  // one line per layer: type, name, bottoms, tops, convolution shape
+    std::string describe() const;  // one line per layer: type, name, bottoms, tops, top shape, convolution weights
     int find_blob_index_by_name(const std::string& name) const;
     Layer* layer_by_name(const std::string& name) const;
     size_t layer_count() const { return layers_.size(); }

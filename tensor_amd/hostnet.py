@@ -13,7 +13,7 @@ EXPORTS = ["otter_host_last_error", "otter_host_net_create", "otter_host_net_des
            "otter_host_net_set_inner_product", "otter_host_net_run", "otter_host_session_create",
            "otter_host_session_pass", "otter_host_session_fetch", "otter_host_session_destroy",
            "otter_host_functional_chain", "otter_host_net_load_otter", "otter_host_net_load_weight",
-           "otter_host_net_describe", "otter_host_net_eval", "otter_host_otter_dump", "otter_host_ncnn_read"]
+           "otter_host_net_describe", "otter_host_net_conv_fp32_probe", "otter_host_net_eval", "otter_host_otter_dump", "otter_host_ncnn_read"]
 
 
 def load_cdll():
@@ -66,6 +66,10 @@ class Net:
             self.h, name.encode(), wq.ctypes.data_as(C.c_void_p), b.ctypes.data_as(f32p) if b is not None else None,
             ws.ctypes.data_as(f32p), C.c_int(ws.size), C.c_float(in_scale), C.c_float(top_scale)))
 
+    def conv_fp32_probe(self, name, on):
+        """While on, an int8-output convolution runs as its fp32-output twin (calibration aid)."""
+        self._check(self.lib.otter_host_net_conv_fp32_probe(self.h, name.encode(), int(on)))
+
     def scale_in(self, name, k):
         out = np.empty(k, np.float32)
         self._check(self.lib.otter_host_net_get_scale_in(self.h, name.encode(), out.ctypes.data_as(C.c_void_p)))
@@ -107,8 +111,8 @@ class Net:
         self._check(self.lib.otter_host_net_load_weight(self.h, os.fsencode(path), int(ncnn)))
 
     def describe(self):
-        """[(type, name, [bottom blobs], [top blobs], conv_shape or None)], conv_shape = dict(K, C, groups, kh, kw,
-        bias_term, int8_scale_term)."""
+        """[(type, name, [bottom blobs], [top blobs], conv or None, top shape (N, C, H, W))], conv = dict(K, C, groups,
+        kh, kw, bias_term, int8_scale_term)."""
         buf = C.create_string_buffer(1 << 22)
         n = self.lib.otter_host_net_describe(self.h, buf, C.c_size_t(len(buf)))
         if n < 0:
@@ -117,9 +121,10 @@ class Net:
         for line in buf.value.decode().splitlines():
             f = line.split(" ")
             conv = None
-            if len(f) > 4:
-                conv = dict(zip(("K", "C", "groups", "kh", "kw", "bias_term", "int8_scale_term"), map(int, f[4:11])))
-            out.append((f[0], f[1], [] if f[2] == "-" else f[2].split(","), [] if f[3] == "-" else f[3].split(","), conv))
+            if len(f) > 8:
+                conv = dict(zip(("K", "C", "groups", "kh", "kw", "bias_term", "int8_scale_term"), map(int, f[8:15])))
+            out.append((f[0], f[1], [] if f[2] == "-" else f[2].split(","), [] if f[3] == "-" else f[3].split(","), conv,
+                        tuple(map(int, f[4:8]))))
         return out
 
     def eval(self, inputs, out_name):

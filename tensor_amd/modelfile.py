@@ -54,7 +54,7 @@ def synthetic_int8_weights(layers, rng, bottom_scale=24.0):
     small bias, and one activation scale for every blob. Returns (bytes, {layer name: dict of what was written})."""
     blob = b""
     written = {}
-    for typ, name, _bottoms, _tops, c in layers:
+    for typ, name, _bottoms, _tops, c, _shape in layers:
         if typ != "Convolution":
             continue
         if not c["int8_scale_term"]:

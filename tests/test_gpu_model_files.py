@@ -30,7 +30,7 @@ def detector(ref, tmp_path_factory):
     net.load_weight(path, ncnn=True)
     rnet = ref.net(NANODET, path)
     alias = {}  # blobs of the automatic Split layers -> the blob they share
-    for typ, _name, bottoms, tops, _conv in layers:
+    for typ, _name, bottoms, tops, _conv, _shape in layers:
         if typ == "Split":
             for t in tops:
                 alias[t] = bottoms[0]
@@ -58,7 +58,7 @@ def test_every_layer_against_the_reference_on_the_reference_inputs(detector):
     blobs["data_1"] = x
     inexact = []
     n_int8 = 0
-    for typ, name, bottoms, tops, _conv in real:
+    for typ, name, bottoms, tops, _conv, _shape in real:
         got = net.eval({b: blobs[alias.get(b, b)] for b in bottoms}, tops[0])
         want = blobs[tops[0]]
         assert got.shape == want.shape and got.dtype == want.dtype, (typ, name)

@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from tensor_amd import hostnet, modelfile
+from tensor_amd import calibration, hostnet, modelfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN = os.path.join(HERE, "golden")
@@ -99,3 +99,12 @@ def test_conv_record_layout():
     assert np.frombuffer(rec[:4], np.uint32)[0] == 0x000D4B38
     rec1 = modelfile.conv_record(wq, None, np.ones(2, np.float32), 3.0, 4.0, 1)
     assert len(rec1) == 4 + 12 + 8 + 4
+
+
+def test_quantize_weights_definition():
+    w = np.array([[[[0.5, -1.0]]], [[[0.2, 0.1]]], [[[0.0, 0.0]]]], np.float32)
+    wq, ws = calibration.quantize_weights(w)
+    np.testing.assert_array_equal(wq.reshape(3, 2), [[64, -127], [127, 64], [0, 0]])  # 63.5 rounds away from zero
+    np.testing.assert_allclose(ws, [127.0, 635.0, 127.0])
+    wq1, ws1 = calibration.quantize_weights(w, per_channel=False)
+    assert ws1.shape == (1,) and wq1.reshape(-1)[1] == -127 and wq1.reshape(-1)[2] == 25

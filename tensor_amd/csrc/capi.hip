@@ -366,7 +366,7 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     case 2: {
         // set_tile(-2, s): force the strip height; set_tile(-3, s): same, on the vector-ALU kernels
         const int dw_shift = (h->force_tm == -2 || h->force_tm == -3) ? h->force_tn : -1;
-        const int epi = pick_epilogue(ep, g.K);
+        const int epi = dw_mfma_epilogue(ep, g.K);
         const bool mfma = h->w_dw_mfma && h->force_tm != -3 && dw_mfma_applicable(g, ep, epi, h->so_positive);
         // the (image group, channel group) index rides on grid.y: run a very large batch in slices
         const int per = 32768 / (g.C / 8);

@@ -117,7 +117,7 @@ struct Epilogue {
 };
 
 // which epilogue code a kernel instance carries
-enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3 };
+enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3, EPI_F32_P8 = 4 /* depthwise only */ };
 
 // The fast epilogues need: activation in {none, ReLU, clip, LeakyReLU with a slope in [0, 1]}, and (I8_P8) int8
 // output in Byte8 with K % 8 == 0 or (F32_P4) fp32 output in Float4 with K % 4 == 0.

@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
         si[t] = *reinterpret_cast<const v4i*>(ep.scale_in + ch + 4 * t);
         bi[t] = *reinterpret_cast<const v4i*>(ep.bias + ch + 4 * t);
         so[t] = v4i{0, 0, 0, 0};
-        if constexpr (EPI != EPI_F32_P4) so[t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
+        if constexpr (EPI != EPI_F32_P4 && EPI != EPI_F32_P8) so[t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
         // the bias is the fma's vector operand in every row: keep it resident (the compiler would otherwise re-copy
         // it from scalar registers row after row)
 #pragma unroll
@@ -209,6 +209,11 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
                       : DW_OOB;
         s_out = (unsigned)(n0 * (g.C / 4) + 2 * o) * OHW * 16u;
         row_bytes = (unsigned)g.OW * 16u;
+    } else if constexpr (EPI == EPI_F32_P8) {  // Float8: [N][C/8][OH*OW][8 floats]; a lane's sets are the pixel's halves
+        v_out = st_ok ? (unsigned)di * (unsigned)C8 * OHW * 32u + (unsigned)ox * 32u + (S == 1 ? 0u : (unsigned)(q & 1) * 16u)
+                      : DW_OOB;
+        s_out = (unsigned)(n0 * C8 + o) * OHW * 32u;
+        row_bytes = (unsigned)g.OW * 32u;
     } else {  // Byte8: [N][C/8][OH*OW][8 bytes]
         v_out = st_ok ? (unsigned)di * (unsigned)C8 * OHW * 8u + (unsigned)ox * 8u + (S == 1 ? 0u : (unsigned)(q & 1) * 4u)
                       : DW_OOB;
@@ -236,12 +241,12 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
     __builtin_amdgcn_sched_barrier(0);
 
     auto epilogue_store = [&](unsigned v_o, unsigned s_row, bool row_ok) {
-        if constexpr (EPI == EPI_F32_P4) {
+        if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P8) {
 #pragma unroll
             for (int t = 0; t < T; ++t) {
                 const v4i res = dw_dequant4(ep, cur[t], si[t], bi[t]);
-                // the second set's channels 4..7 are the next Float4 pack: one plane further
-                const unsigned vo_t = (t == 0 || !row_ok) ? v_o : v_o + OHW * 16u;
+                // the second set's channels 4..7: the next Float4 pack is one plane further, in Float8 they follow
+                const unsigned vo_t = (t == 0 || !row_ok) ? v_o : v_o + (EPI == EPI_F32_P4 ? OHW * 16u : 16u);
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, res), rout, (int)vo_t, (int)s_row, 0);
             }
         } else {
@@ -310,12 +315,21 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
     }
 }
 
+// the epilogue code of a depthwise layer: the common rule, plus fp32 output in the depthwise default layout Float8
+int dw_mfma_epilogue(const Epilogue& ep, int K) {
+    const int epi = pick_epilogue(ep, K);
+    const bool clamp_act = ep.act == 0 || ep.act == 1 || ep.act == 3 || (ep.act == 2 && ep.lrelu);
+    if (epi == EPI_GENERIC && clamp_act && ep.out_kind == OTTER_HIP_OUT_F32 && ep.out_layout == OTTER_HIP_F32_P8 && K % 8 == 0)
+        return EPI_F32_P8;
+    return epi;
+}
+
 // true when this layer / batch can take the matrix-core kernel (the caller falls back to the vector kernels otherwise)
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive) {
     if (epi == EPI_I8_P8_NONNEG && !scale_out_positive) return false;  // the clamp is moved past the output scale
     if (!(g.kh == 3 && g.kw == 3 && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2))) return false;
     if (g.ph > 1 || g.pw > 1 || g.C % 8 != 0 || g.C != g.K) return false;
-    if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4) return false;
+    if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4 && epi != EPI_F32_P8) return false;
     const size_t in_bytes = (size_t)g.N * g.C * g.H * g.W;
     const size_t out_bytes = (size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1);
     return in_bytes < ((size_t)1 << 31) && out_bytes < ((size_t)1 << 31);  // 32-bit buffer offsets
@@ -361,7 +375,7 @@ hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const 
     if (wpb == 4 && per_cu >= 2 && per_cu <= 4) lds_reserve = (unsigned)(160 * 1024 / per_cu) / 1024 * 1024;
     if (lds_reserve > 64 * 1024) lds_reserve = 64 * 1024;  // the default limit of dynamic LDS; still two per CU
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
-    const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1));
+    const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 || epi == EPI_F32_P8 ? 4 : 1));
 #define OHIP_DWM(S_, E_) \
     do {                                                                                                               \
         if (g.W & 1)                                                                                                   \
@@ -375,6 +389,7 @@ hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const 
     do {                                                              \
         if (epi == EPI_I8_P8_NONNEG) OHIP_DWM(S_, EPI_I8_P8_NONNEG);  \
         else if (epi == EPI_I8_P8) OHIP_DWM(S_, EPI_I8_P8);           \
+        else if (epi == EPI_F32_P8) OHIP_DWM(S_, EPI_F32_P8);         \
         else OHIP_DWM(S_, EPI_F32_P4);                                \
     } while (0)
     if (g.sh == 1) OHIP_DWM_E(1);

@@ -26,6 +26,7 @@ hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void*
 // conv_dw.hip
 size_t dw_mfma_weight_bytes(int C, int stride);
 void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t* dst);
+int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
                             int strip_shift, hipStream_t stream);

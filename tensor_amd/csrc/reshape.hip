@@ -105,10 +105,37 @@ __global__ void __launch_bounds__(256) channel_shuffle_kernel(const float* __res
     dst[i] = src[packed_off(d.n, cs, d.y, d.x, C, H, W, ps)];
 }
 
+// groups == 2 on elempack 8 (the ShuffleNetV2 block of the detection model): output pack q interleaves source channels
+// 4q..4q+3 of the first half with the same four of the second half -- two 16-byte reads, two 16-byte writes per pixel
+__global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                                  int C, int HW, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // (n, output pack, pixel)
+    if (i >= total) return;
+    const int px = (int)(i % HW);
+    const size_t r = i / HW;
+    const int packs = C / 8;
+    const int q = (int)(r % packs);
+    const size_t n = r / packs;
+    const int half = C / 2;
+    const int c0 = 4 * q, c1 = half + 4 * q;  // first source channel of each half
+    const float* base = src + n * (size_t)C * HW;
+    const float4 a = *reinterpret_cast<const float4*>(base + ((size_t)(c0 / 8) * HW + px) * 8 + c0 % 8);
+    const float4 b = *reinterpret_cast<const float4*>(base + ((size_t)(c1 / 8) * HW + px) * 8 + c1 % 8);
+    float4* o = reinterpret_cast<float4*>(dst + (n * (size_t)C * HW) + ((size_t)q * HW + px) * 8);
+    o[0] = make_float4(a.x, b.x, a.y, b.y);
+    o[1] = make_float4(a.z, b.z, a.w, b.w);
+}
+
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
                                hipStream_t stream) {
     const size_t total = (size_t)N * C * H * W;
     if (total == 0) return hipSuccess;
+    if (groups == 2 && ps == 8 && pd == 8 && C % 16 == 0) {
+        const size_t units = total / 8;
+        hipLaunchKernelGGL(channel_shuffle2_p8_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, src, dst, C,
+                           H * W, units);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(channel_shuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd,
                        N, C, H, W, groups, total);
     return hipGetLastError();

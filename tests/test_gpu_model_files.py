@@ -135,6 +135,8 @@ GLUE_CASES = [
      _layer("Crop", "c2", ["s"], start=8, end=20, axis=1) + _layer("Crop", "c3", ["s"], start=20, end=24, axis=1) +
      _layer("Concat", "cat", ["c3", "c1", "c2"], axis=1) + _layer("ChannelShuffle", "s2", ["cat"], groups=2),
      ["s", "c1", "c2", "c3", "cat", "s2"]),
+    ("shuffle_groups2_pack8", (48, 7, 9), _layer("ChannelShuffle", "s", ["data"], groups=2), ["s"]),
+    ("shuffle_groups4", (16, 3, 5), _layer("ChannelShuffle", "s", ["data"], groups=4), ["s"]),
     ("crop_unaligned", (12, 4, 4), _layer("Crop", "c", ["data"], start=3, end=10, axis=1) +
      _layer("Concat", "cat", ["c", "data"], axis=1), ["c", "cat"]),
     ("shortcut", (16, 5, 5), _layer("MaxPool", "p", ["data"], kernel=3, stride=1, padding=1) +

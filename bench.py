@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 convolution path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c0|c4] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c0|c4|det] [--no-cpu] [--no-also]
 
-Prints ONE JSON line. The headline workload is BASELINE.json configs[3] (the MFMA-bound case the metric's
+Prints ONE JSON line. The headline workload is the fourth benchmark configuration (the MFMA-bound case the metric's
 "int8 conv TOPS (% MFMA peak)" is quoted on): four chained int8-in/int8-out 3x3 convolutions 128->128 at
 56x56, batch 64, fused requantize+ReLU. One step = the four layers back to back on device-resident int8
 activations. The other single-GPU configurations (depthwise c1 at stride 1 and 2 with its HBM roofline, the
@@ -465,7 +465,7 @@ def main():
     ap.add_argument("--no-also", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1:
-        print("bench.py: this build runs on one GPU only (batch sharding is described in DESIGN.md); "
+        print("bench.py: this build runs on one GPU only (the path shards by batch: images are independent); "
               "--gpus %d is not supported" % a.gpus, file=sys.stderr)
         sys.exit(2)
     if int(os.environ.get("WORLD_SIZE", "1")) > 1:

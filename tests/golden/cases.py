@@ -2,7 +2,8 @@
 
 Every case stays inside what the reference itself executes correctly in packed mode (groups == 1 or
 depthwise with C % 8 == 0, batch looped, no C % 8 != 0 with K % 4 != 0); the shapes it crashes or hangs on
-are listed in DESIGN.md and are never sent to the compiled reference.
+(packed C=3 K=4 1x1, grouped non-depthwise, depthwise with C % 8 != 0, unpacked depthwise) are never sent to the
+compiled reference.
 """
 
 # name, C, K, kernel, stride, pad, dilation, groups, H, W, N, in_is_int8, int8_out, bias, activation, act_params

@@ -97,7 +97,7 @@ def main():
             G[tag + "/q"] = R.requantize(acc, si, so, bias, act, ap, packing)
     # ---- dequantize: bitwise, with the magnitudes where fma and mul+add part ways -------------------
     for C, packing in ((8, True), (4, True), (8, False)):
-        acc = rng.integers(-2000000, 2000000, size=(2, C, 8, 8)).astype(np.int32)  # H*W % 4 == 0: see DESIGN.md
+        acc = rng.integers(-2000000, 2000000, size=(2, C, 8, 8)).astype(np.int32)  # H*W % 4 == 0: the reference's unpacked dequantize leaves a ragged tail unwritten
         si = rng.uniform(1e-6, 1e-5, C).astype(np.float32)
         bias = rng.normal(0, 1, C).astype(np.float32)
         for j, b in enumerate((None, bias)):

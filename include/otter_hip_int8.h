@@ -135,7 +135,8 @@ int otter_hip_conv_forward(const otter_hip_conv_t* handle, const void* in, int i
                            void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
- * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel. For tests and profiling. */
+ * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
+ * blob). For tests and profiling. */
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, int n, int in_h, int in_w,
                                int out_layout);
 

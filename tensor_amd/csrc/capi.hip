@@ -52,6 +52,7 @@ struct otter_hip_conv {
     bool depthwise = false;
     int8_t* w_raw = nullptr;     // [K, C/g, kh, kw]           (direct kernel)
     int8_t* w_igemm = nullptr;   // MFMA lane order            (groups == 1, C % 8 == 0)
+    int8_t* w_stem = nullptr;    // MFMA lane order of the few-channel 3x3 kernel (C <= 5, K <= 64)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
     int8_t* w_dw_mfma = nullptr; // block-diagonal MFMA operands (depthwise 3x3, C % 8 == 0)
     bool so_positive = true;     // every output scale is finite and > 0
@@ -140,6 +141,7 @@ int otter_hip_conv_destroy(otter_hip_conv_t* h) {
     if (!h) return OTTER_HIP_OK;
     (void)hipFree(h->w_raw);
     (void)hipFree(h->w_igemm);
+    (void)hipFree(h->w_stem);
     (void)hipFree(h->w_dw);
     (void)hipFree(h->w_dw_mfma);
     (void)hipFree(h->scale_in);
@@ -214,6 +216,11 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             igemm_pack_weights(wpad.data(), K, cp, d.kernel_h, d.kernel_w, wp.data());
             if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
             h->c_pad = cp;
+            if (C <= 5 && K <= 64 && d.kernel_h == 3 && d.kernel_w == 3) {  // an image stem: see conv_stem.hip
+                std::vector<int8_t> wsv(stem_packed_weight_bytes(K));
+                stem_pack_weights(weight, K, C, wsv.data());
+                if ((rc = upload<int8_t>(&h->w_stem, wsv.data(), wsv.size(), wsv.size(), 0))) break;
+            }
         }
     } while (0);
     if (rc != OTTER_HIP_OK) {
@@ -287,7 +294,12 @@ static Epilogue make_epilogue(const otter_hip_conv* h, int out_layout) {
     return ep;
 }
 
-// 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS
+// the few-channel 3x3 kernel takes the blob as the caller holds it (unpacked fp32 or int8): no quantize / pad pass
+static bool use_stem(const otter_hip_conv* h, int in_layout, const ConvGeom& g_in, const Epilogue& ep) {
+    return h->w_stem && h->force_tm == 0 && conv_stem_applicable(g_in, ep, in_layout);
+}
+
+// 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS, 4 few-channel 3x3 (image stem)
 static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g, const Epilogue& ep) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
@@ -303,8 +315,9 @@ static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom&
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int out_layout) {
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
-    if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
     ConvGeom g = make_geom(h->d, n, in_h, in_w);
+    if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) return 4;
+    if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
     if (h->c_pad) l = OTTER_HIP_I8_P8, g.C = h->c_pad;
     return pick_kernel(h, l, g, make_epilogue(h, out_layout));
 }
@@ -331,6 +344,12 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
     if ((size_t)n * g.C * in_h * in_w >= (1ull << 31) || (size_t)n * g.K * g.OH * g.OW >= (1ull << 31))
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
     if (n == 0) return OTTER_HIP_OK;
+
+    if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) {
+        OHIP_CHECK(run_conv_stem(in, layout_elem(in_layout) == 0, h->w_stem, out, g, make_epilogue(h, out_layout), h->in_scale,
+                                 d.in_round_mode, stream));
+        return OTTER_HIP_OK;
+    }
 
     // (1) quantize_to_int8 when the blob is not int8 yet (Tensor/ConvolutionLayer.cpp:770-775)
     const int8_t* xq = (const int8_t*)in;

@@ -56,6 +56,13 @@ hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, fl
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream);
 
+// conv_stem.hip: 3x3 convolution of a blob with at most 5 channels, straight from the unpacked fp32 / int8 blob
+size_t stem_packed_weight_bytes(int K);
+void stem_pack_weights(const int8_t* w, int K, int C, int8_t* dst);
+bool conv_stem_applicable(const ConvGeom& g, const Epilogue& ep, int in_layout);
+hipError_t run_conv_stem(const void* x, bool in_f32, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                         const float* in_scale, int in_round, hipStream_t stream);
+
 // reshape.hip: fp32 layout glue (pack = elempack of the layout on that side)
 hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
                              int H, int W, hipStream_t stream);

@@ -302,6 +302,35 @@ def test_leaky_relu_fast_epilogues(hip, oracle, C, K, k, s, p, g, N, H, W, kind)
             assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("C,K,s,p,N,H,W,in_i8,act,int8_out", [
+    (3, 32, 2, 1, 3, 30, 46, False, 3, True),    # the MobileNetV2 stem: fp32 image, ReLU6, int8 out
+    (3, 24, 2, 1, 2, 33, 21, False, 2, False),   # the detection model's stem: LeakyReLU, fp32 out, 1.5 tiles of channels
+    (1, 16, 1, 0, 2, 9, 19, False, 0, True),     # one channel, no padding
+    (4, 40, 1, 1, 2, 12, 17, True, 1, True),     # int8 planar input, 2.5 tiles
+    (5, 64, 2, 0, 1, 15, 16, True, 0, False),    # the widest reduction (45 of 64 bytes), 4 tiles
+    (3, 8, 1, 1, 5, 8, 8, False, 1, False),      # half a tile
+])
+def test_few_channel_3x3_stem_kernel(hip, oracle, C, K, s, p, N, H, W, in_i8, act, int8_out):
+    """3x3 on a blob with at most 5 channels goes straight from the unpacked blob (quantized on the way) to the
+    packed output; the same layer forced through the channel-padded copy and the generic kernel must agree bit for
+    bit, and both equal the oracle."""
+    rng = np.random.default_rng(1000 * C + K)
+    x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W, in_i8=in_i8)
+    kw = dict(stride=s, pad=p, bias=bias, top_scale=11.0, act=act, act_p0=0.1,
+              out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+    want = oracle.conv_layer_forward(x, wq, ws, 25.0, stride=(s, s), pad=(p, p), bias=bias, top_scale=11.0,
+                                     int8_out=int8_out, act_type=act, act_params=[0.1] if act == 2 else None)
+    out, kind = run_conv(hip, oracle, x, wq, ws, 25.0, **kw)
+    assert kind == 4
+    via_copy, kind2 = run_conv(hip, oracle, x, wq, ws, 25.0, tile=(-4, 0), **kw)
+    assert kind2 == 1
+    if int8_out:
+        np.testing.assert_array_equal(out, want)
+    else:
+        assert_f32_close(out, want)
+    np.testing.assert_array_equal(out, via_copy)
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

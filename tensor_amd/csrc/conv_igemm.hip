@@ -55,8 +55,9 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     }
     const int mt0 = blockIdx.y * (TM / 16);  // first 16-row tile of this workgroup
     const int OHW = g.OH * g.OW;
-    const long total_pix = (long)g.N * OHW;
-    const long tile_base = (long)pt * TN;
+    // 32-bit pixel indices: the C ABI refuses tensors of 2^31 elements or more, and a 64-bit division costs ~4x
+    const unsigned total_pix = (unsigned)g.N * (unsigned)OHW;
+    const unsigned tile_base = (unsigned)pt * TN;
     const int C8 = g.C / 8;
     const int HW = g.H * g.W;
 
@@ -64,14 +65,14 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     const int p_l = tid % TN;
     const int j0 = tid / TN;
     constexpr int J_STEP = 256 / TN > 0 ? 256 / TN : 1;
-    const long gp = tile_base + p_l;
+    const unsigned gp = tile_base + p_l;
     const bool pvalid = gp < total_pix;
     int iy0 = 0, ix0 = 0;
     const int8_t* xn = x;
     if (pvalid) {
-        const int n = (int)(gp / OHW);
-        const int pix = (int)(gp % OHW);
-        const int oy = pix / g.OW, ox = pix % g.OW;
+        const int n = (int)(gp / (unsigned)OHW);
+        const int pix = (int)(gp - (unsigned)n * (unsigned)OHW);
+        const int oy = (int)((unsigned)pix / (unsigned)g.OW), ox = pix - oy * g.OW;
         iy0 = oy * g.sh - g.ph;
         ix0 = ox * g.sw - g.pw;
         xn = x + (size_t)n * C8 * HW * 8;
@@ -150,6 +151,12 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     // ---- epilogue -----------------------------------------------------------------------------------
     // (no `continue` / early exits inside the unrolled loops: the accumulator array must stay in registers)
     const int gq = lane >> 4;
+    // image and pixel of this lane's first column; the other columns are 16, 32, ... pixels further: one division per
+    // lane instead of one per column (a 32-bit division is ~20 vector instructions)
+    const unsigned gp0 = tile_base + wn * (TN / WN) + (lane & 15);
+    const unsigned n0 = gp0 / (unsigned)OHW;
+    const unsigned pix0 = gp0 - n0 * (unsigned)OHW;
+    const bool wide = (unsigned)OHW >= 16u * FN;  // then a column is at most one image further than the first
 #pragma unroll
     for (int ip = 0; ip < FM / 2; ++ip) {
         const int tpair = (mt0 + wm * FM) / 2 + ip;
@@ -159,7 +166,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         if constexpr (EPI != EPI_GENERIC) epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
-            const long gpo = tile_base + wn * (TN / WN) + j * 16 + (lane & 15);
+            const unsigned gpo = gp0 + j * 16;
             int a8[8];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -167,8 +174,14 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                 a8[4 + e] = acc[2 * ip + 1][j][e];
             }
             if (ch_ok && gpo < total_pix) {
-                const int n = (int)(gpo / OHW);
-                const int pix = (int)(gpo % OHW);
+                unsigned nn = n0, pp = pix0 + j * 16;
+                if (wide) {
+                    if (pp >= (unsigned)OHW) pp -= (unsigned)OHW, ++nn;
+                } else {
+                    nn = gpo / (unsigned)OHW;
+                    pp = gpo - nn * (unsigned)OHW;
+                }
+                const int n = (int)nn, pix = (int)pp;
                 if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
                     epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
                                                              elem_offset(8, n, ch0, pix, g.K, OHW), a8);

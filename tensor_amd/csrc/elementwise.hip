@@ -110,14 +110,15 @@ struct CopyOp {
 template <typename TI, typename TO, int SP, int DP, int V, class Op>
 __global__ void __launch_bounds__(256) ew_kernel(const TI* __restrict__ src, TO* __restrict__ dst, int N, int C, int HW,
                                                  Op op) {
-    const int cv_count = C / V;
-    const size_t total = (size_t)N * cv_count * HW;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (size_t)gridDim.x * blockDim.x) {
-        const int pix = (int)(idx % HW);
-        const size_t r = idx / HW;
-        const int cv = (int)(r % cv_count);
+    // 32-bit indices (the C ABI refuses tensors of 2^31 elements or more): 64-bit divisions would cost more vector
+    // instructions than the operation itself
+    const unsigned cv_count = (unsigned)(C / V);
+    const unsigned total = (unsigned)N * cv_count * (unsigned)HW;
+    for (unsigned idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const unsigned r = idx / (unsigned)HW;
+        const int pix = (int)(idx - r * (unsigned)HW);
         const int n = (int)(r / cv_count);
+        const int cv = (int)(r - (unsigned)n * cv_count);
         TI in[V];
         TO out[V];
         Access<TI, SP, V>::load(src, n, cv * V, pix, C, HW, in);
@@ -162,13 +163,13 @@ template <typename T>
 __global__ void __launch_bounds__(256) pad_pack8_kernel(const T* __restrict__ src, int sp, int8_t* __restrict__ dst, int N,
                                                         int C, int Cp, int HW, const float* __restrict__ scale,
                                                         int round_mode) {
-    const size_t total = (size_t)N * (Cp / 8) * HW;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const unsigned total = (unsigned)N * (unsigned)(Cp / 8) * (unsigned)HW;
+    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
-    const int pix = (int)(idx % HW);
-    const size_t r = idx / HW;
-    const int o = (int)(r % (Cp / 8));
-    const int n = (int)(r / (Cp / 8));
+    const unsigned r = idx / (unsigned)HW;
+    const int pix = (int)(idx - r * (unsigned)HW);
+    const int n = (int)(r / (unsigned)(Cp / 8));
+    const int o = (int)(r - (unsigned)n * (unsigned)(Cp / 8));
     int q[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {

@@ -17,17 +17,19 @@ __device__ __forceinline__ size_t packed_off(int n, int c, int y, int x, int C, 
 struct DstIndex {
     int n, c, y, x;
 };
-__device__ __forceinline__ DstIndex dst_index(size_t i, int c0, int cnt, int H, int W, int p) {
+// (32-bit arithmetic throughout: the C ABI refuses tensors of 2^31 elements or more)
+__device__ __forceinline__ DstIndex dst_index(unsigned i, int c0, int cnt, int H, int W, int p) {
     DstIndex d;
-    const int e = (int)(i % p);
-    i /= p;
-    d.x = (int)(i % W);
-    i /= W;
-    d.y = (int)(i % H);
-    i /= H;
-    const int packs = cnt / p;
-    d.c = c0 + (int)(i % packs) * p + e;
-    d.n = (int)(i / packs);
+    unsigned r = i / (unsigned)p;
+    const int e = (int)(i - r * (unsigned)p);
+    unsigned t = r / (unsigned)W;
+    d.x = (int)(r - t * (unsigned)W);
+    r = t / (unsigned)H;
+    d.y = (int)(t - r * (unsigned)H);
+    const unsigned packs = (unsigned)(cnt / p);
+    t = r / packs;
+    d.c = c0 + (int)(r - t * packs) * p + e;
+    d.n = (int)t;
     return d;
 }
 
@@ -36,18 +38,20 @@ __device__ __forceinline__ DstIndex dst_index(size_t i, int c0, int cnt, int H, 
 template <bool ALIGNED>
 __global__ void __launch_bounds__(256) copy_channels_kernel(const float* __restrict__ src, int Cs, int ps, int cs0,
                                                             float* __restrict__ dst, int Cd, int pd, int cd0, int cnt,
-                                                            int N, int H, int W, size_t total) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                            int N, int H, int W, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     DstIndex d;
     if (ALIGNED) {
         d = dst_index(i, cd0, cnt, H, W, pd);
     } else {  // channel-major enumeration; the writes of a packed destination are strided then
-        size_t r = i;
-        d.x = (int)(r % W), r /= W;
-        d.y = (int)(r % H), r /= H;
-        d.c = cd0 + (int)(r % cnt);
-        d.n = (int)(r / cnt);
+        unsigned r = i / (unsigned)W;
+        d.x = (int)(i - r * (unsigned)W);
+        unsigned t = r / (unsigned)H;
+        d.y = (int)(r - t * (unsigned)H);
+        r = t / (unsigned)cnt;
+        d.c = cd0 + (int)(t - r * (unsigned)cnt);
+        d.n = (int)r;
     }
     dst[packed_off(d.n, d.c, d.y, d.x, Cd, H, W, pd)] = src[packed_off(d.n, d.c - cd0 + cs0, d.y, d.x, Cs, H, W, ps)];
 }
@@ -56,21 +60,21 @@ __global__ void __launch_bounds__(256) copy_channels_kernel(const float* __restr
 // destination range starts and ends on a destination pack boundary
 __global__ void __launch_bounds__(256) copy_channels4_kernel(const float* __restrict__ src, int Cs, int ps, int cs0,
                                                              float* __restrict__ dst, int Cd, int pd, int cd0, int cnt,
-                                                             int N, int H, int W, size_t total4) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                             int N, int H, int W, unsigned total4) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total4) return;
     // quads of the destination range in memory order: (n, pack, y, x, quad within the pack)
-    size_t r = i;
-    const int qd = pd / 4;
-    const int q = (int)(r % qd);
-    r /= qd;
-    const int x = (int)(r % W);
-    r /= W;
-    const int y = (int)(r % H);
-    r /= H;
-    const int packs = cnt / pd;
-    const int c = cd0 + (int)(r % packs) * pd + 4 * q;
-    const int n = (int)(r / packs);
+    const unsigned qd = (unsigned)(pd / 4);
+    unsigned r = i / qd;
+    const int q = (int)(i - r * qd);
+    unsigned t = r / (unsigned)W;
+    const int x = (int)(r - t * (unsigned)W);
+    r = t / (unsigned)H;
+    const int y = (int)(t - r * (unsigned)H);
+    const unsigned packs = (unsigned)(cnt / pd);
+    t = r / packs;
+    const int c = cd0 + (int)(r - t * packs) * pd + 4 * q;
+    const int n = (int)t;
     const float4 v = *reinterpret_cast<const float4*>(src + packed_off(n, c - cd0 + cs0, y, x, Cs, H, W, ps));
     *reinterpret_cast<float4*>(dst + packed_off(n, c, y, x, Cd, H, W, pd)) = v;
 }
@@ -83,21 +87,21 @@ hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* d
     if (whole && ps % 4 == 0 && pd % 4 == 0 && cs0 % 4 == 0) {
         const size_t total4 = total / 4;
         hipLaunchKernelGGL(copy_channels4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, src, Cs, ps,
-                           cs0, dst, Cd, pd, cd0, cnt, N, H, W, total4);
+                           cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total4);
     } else if (whole) {
         hipLaunchKernelGGL(copy_channels_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, Cs,
-                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, total);
+                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total);
     } else {
         hipLaunchKernelGGL(copy_channels_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, Cs,
-                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, total);
+                           ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total);
     }
     return hipGetLastError();
 }
 
 // Tensor/ChannelShuffleKernel.cpp:19-55: input seen as [n, g, C/g, ...], output as [n, C/g, g, ...]
 __global__ void __launch_bounds__(256) channel_shuffle_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst,
-                                                              int pd, int N, int C, int H, int W, int groups, size_t total) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                              int pd, int N, int C, int H, int W, int groups, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const DstIndex d = dst_index(i, 0, C, H, W, pd);
     const int cpg = C / groups;
@@ -108,14 +112,14 @@ __global__ void __launch_bounds__(256) channel_shuffle_kernel(const float* __res
 // groups == 2 on elempack 8 (the ShuffleNetV2 block of the detection model): output pack q interleaves source channels
 // 4q..4q+3 of the first half with the same four of the second half -- two 16-byte reads, two 16-byte writes per pixel
 __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                                  int C, int HW, size_t total) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // (n, output pack, pixel)
+                                                                  int C, int HW, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;  // (n, output pack, pixel)
     if (i >= total) return;
-    const int px = (int)(i % HW);
-    const size_t r = i / HW;
-    const int packs = C / 8;
-    const int q = (int)(r % packs);
+    const unsigned r = i / (unsigned)HW;
+    const int px = (int)(i - r * (unsigned)HW);
+    const unsigned packs = (unsigned)(C / 8);
     const size_t n = r / packs;
+    const int q = (int)(r - (unsigned)n * packs);
     const int half = C / 2;
     const int c0 = 4 * q, c1 = half + 4 * q;  // first source channel of each half
     const float* base = src + n * (size_t)C * HW;
@@ -133,11 +137,11 @@ hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int
     if (groups == 2 && ps == 8 && pd == 8 && C % 16 == 0) {
         const size_t units = total / 8;
         hipLaunchKernelGGL(channel_shuffle2_p8_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, src, dst, C,
-                           H * W, units);
+                           H * W, (unsigned)units);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(channel_shuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd,
-                       N, C, H, W, groups, total);
+                       N, C, H, W, groups, (unsigned)total);
     return hipGetLastError();
 }
 
@@ -147,8 +151,8 @@ hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int
 // (Tensor/Pool.cpp:974, which pad the blob with zeros first).
 __global__ void __launch_bounds__(256) maxpool_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
                                                       int N, int C, int H, int W, int OH, int OW, int kh, int kw, int sh,
-                                                      int sw, int ph, int pw, int dh, int dw, float pad_value, size_t total) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                      int sw, int ph, int pw, int dh, int dw, float pad_value, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const DstIndex d = dst_index(i, 0, C, OH, OW, pd);
     float m = -__builtin_inff();
@@ -169,7 +173,7 @@ hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int 
     const size_t total = (size_t)N * C * OH * OW;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
-                       W, OH, OW, kh, kw, sh, sw, ph, pw, dh, dw, pad_value, total);
+                       W, OH, OW, kh, kw, sh, sw, ph, pw, dh, dw, pad_value, (unsigned)total);
     return hipGetLastError();
 }
 
@@ -192,8 +196,8 @@ __device__ __forceinline__ void linear_coeff(int in_size, int out_size, int d, i
 // count is a multiple of 4.
 __global__ void __launch_bounds__(256) upsample_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
                                                        int N, int C, int H, int W, int OH, int OW, int mode,
-                                                       int align_corner, size_t total) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                       int align_corner, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const DstIndex d = dst_index(i, 0, C, OH, OW, pd);
     if (mode == 1) {
@@ -220,7 +224,7 @@ hipError_t run_upsample(const float* src, int ps, float* dst, int pd, int N, int
     const size_t total = (size_t)N * C * OH * OW;
     if (total == 0) return hipSuccess;
     hipLaunchKernelGGL(upsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
-                       W, OH, OW, mode, align_corner, total);
+                       W, OH, OW, mode, align_corner, (unsigned)total);
     return hipGetLastError();
 }
 

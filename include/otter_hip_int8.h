@@ -183,6 +183,13 @@ int otter_hip_repack(const void* src, int src_layout, int n, int c, int h, int w
  * blobs in the same layout. */
 int otter_hip_eltwise_add(const float* a, const float* b, float* out, size_t count, void* stream);
 
+/* The same sum and, in the same pass, what the int8 convolution that reads it would compute first: its
+ * quantize_to_int8 of the fp32 bottom blob (ConvolutionLayer::forward_int8, Tensor/ConvolutionLayer.cpp:770-775),
+ * q = float2int8(out * scale) written as Byte8. a, b, out in `layout` (OTTER_HIP_F32_P4 or _P8), c % 8 == 0;
+ * scale = the consumer's bottom_blob_int8_scales[0], round_mode = its input rounding primitive. */
+int otter_hip_eltwise_add_quantize(const float* a, const float* b, int layout, int n, int c, int h, int w, float scale,
+                                   int round_mode, float* out, int8_t* q, void* stream);
+
 /* ReluLayer / LReluLayer / Relu6Layer / SigmoidLayer::forward_inplace (Tensor/ReluLayer.cpp, LReluLayer.cpp:45-,
  * Relu6Layer.cpp:29-100) on a device blob; activation_type as in otter_hip_conv_desc. */
 int otter_hip_activation(float* x, size_t count, int activation_type, float activation_param0, void* stream);

@@ -489,6 +489,19 @@ int otter_hip_eltwise_add(const float* a, const float* b, float* out, size_t cou
     return OTTER_HIP_OK;
 }
 
+int otter_hip_eltwise_add_quantize(const float* a, const float* b, int layout, int n, int c, int h, int w, float scale,
+                                   int round_mode, float* out, int8_t* q, void* stream) {
+    if (!a || !b || !out || !q) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_eltwise_add_quantize: null");
+    if (layout != OTTER_HIP_F32_P4 && layout != OTTER_HIP_F32_P8)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_eltwise_add_quantize: Float4 or Float8 blobs expected");
+    if (n < 0 || c < 8 || c % 8 || h < 1 || w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_eltwise_add_quantize: the channel count must be a multiple of 8");
+    if ((size_t)n * c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_eltwise_add_quantize: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_eltwise_add_quantize(a, b, layout_pack(layout), out, q, n, c, h * w, scale, round_mode, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_activation(float* x, size_t count, int activation_type, float activation_param0, void* stream) {
     if (!x) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_activation: null");
     if (activation_type < 0 || activation_type > 4)

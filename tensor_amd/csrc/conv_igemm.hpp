@@ -52,6 +52,8 @@ hipError_t run_repack(const void* src, int sp, void* dst, int dp, int elem_bytes
 // glue.hip
 hipError_t run_eltwise_add(const float* a, const float* b, float* out, size_t n, hipStream_t stream);
 hipError_t run_activation(float* x, size_t n, int act, float p0, hipStream_t stream);
+hipError_t run_eltwise_add_quantize(const float* a, const float* b, int pack, float* out, int8_t* q, int N, int C, int HW,
+                                    float scale, int round_mode, hipStream_t stream);
 hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, float* out, hipStream_t stream);
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream);

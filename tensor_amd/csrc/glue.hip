@@ -114,6 +114,65 @@ hipError_t run_eltwise_add(const float* a, const float* b, float* out, size_t n,
     return hipGetLastError();
 }
 
+// out = a + b and, in the same pass, the int8 blob a following int8 convolution would make of it
+// (ConvolutionLayer::forward_int8 quantizes an fp32 bottom blob first, Tensor/ConvolutionLayer.cpp:770-775):
+// q = float2int8(out * scale) into Byte8. One thread per (image, channel octet, pixel); P = elempack of a, b and out.
+template <int P>
+__global__ void __launch_bounds__(256) eltwise_add_quantize_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                   float* __restrict__ out, int8_t* __restrict__ q, int C8,
+                                                                   int HW, float scale, float half, unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const unsigned r = i / (unsigned)HW;
+    const unsigned pix = i - r * (unsigned)HW;  // r = image * C8 + octet
+    float s[8];
+    if constexpr (P == 8) {
+        const size_t o = (size_t)i * 8;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float4 x = *reinterpret_cast<const float4*>(a + o + 4 * h), y = *reinterpret_cast<const float4*>(b + o + 4 * h);
+            const float4 z = make_float4(__fadd_rn(x.x, y.x), __fadd_rn(x.y, y.y), __fadd_rn(x.z, y.z), __fadd_rn(x.w, y.w));
+            *reinterpret_cast<float4*>(out + o + 4 * h) = z;
+            s[4 * h] = z.x, s[4 * h + 1] = z.y, s[4 * h + 2] = z.z, s[4 * h + 3] = z.w;
+        }
+    } else {  // Float4: the octet's two packs are the planes 2r and 2r+1
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const size_t o = ((size_t)(2 * r + h) * HW + pix) * 4;
+            const float4 x = *reinterpret_cast<const float4*>(a + o), y = *reinterpret_cast<const float4*>(b + o);
+            const float4 z = make_float4(__fadd_rn(x.x, y.x), __fadd_rn(x.y, y.y), __fadd_rn(x.z, y.z), __fadd_rn(x.w, y.w));
+            *reinterpret_cast<float4*>(out + o) = z;
+            s[4 * h] = z.x, s[4 * h + 1] = z.y, s[4 * h + 2] = z.z, s[4 * h + 3] = z.w;
+        }
+    }
+    int v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float t = __fmul_rn(s[e], scale);
+        const int k = (int)__fadd_rn(t, __builtin_copysignf(half, t));
+        v[e] = min(max(k, -127), 127) & 0xff;
+    }
+    ohip_v2i pk;
+    pk[0] = v[0] | (v[1] << 8) | (v[2] << 16) | (v[3] << 24);
+    pk[1] = v[4] | (v[5] << 8) | (v[6] << 16) | (v[7] << 24);
+    reinterpret_cast<ohip_v2i*>(q)[i] = pk;
+}
+
+hipError_t run_eltwise_add_quantize(const float* a, const float* b, int pack, float* out, int8_t* q, int N, int C, int HW,
+                                    float scale, int round_mode, hipStream_t stream) {
+    const size_t total = (size_t)N * (C / 8) * HW;
+    if (total == 0) return hipSuccess;
+    const float half = round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (pack == 8)
+        hipLaunchKernelGGL(eltwise_add_quantize_kernel<8>, grid, block, 0, stream, a, b, out, q, C / 8, HW, scale, half,
+                           (unsigned)total);
+    else
+        hipLaunchKernelGGL(eltwise_add_quantize_kernel<4>, grid, block, 0, stream, a, b, out, q, C / 8, HW, scale, half,
+                           (unsigned)total);
+    return hipGetLastError();
+}
+
 hipError_t run_activation(float* x, size_t n, int act, float p0, hipStream_t stream) {
     if (n == 0 || act == 0) return hipSuccess;
     hipLaunchKernelGGL(activation_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, n, act, p0);

@@ -94,6 +94,7 @@ int otter_host_net_set_conv(void* net, const char* layer_name, const int8_t* wei
         if (L->int8_scale_term > 100) L->top_blob_int8_scales = f32_vec(ts.data(), (int)ts.size());
         const int rc = L->create_pipeline(n->option);
         if (rc) return fail(std::string("create_pipeline: ") + otter_hip_last_error());
+        n->invalidate_plan();
         return 0;
     } catch (const std::exception& e) {
         return fail(e.what());

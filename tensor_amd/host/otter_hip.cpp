@@ -153,6 +153,10 @@ struct Tensor::Storage {
     void* dev = nullptr;
     size_t bytes = 0;
     bool host_valid = false, dev_valid = false;
+    std::shared_ptr<Storage> q8;  // the blob's own int8 quantization, if its producer made one
+    std::vector<int64_t> q8_sizes;
+    float q8_scale = 0.f;
+    int q8_round = 0;
     ~Storage() {
         std::free(host);
         if (dev) pool().put(bytes, dev);
@@ -247,6 +251,22 @@ Tensor Tensor::view(const std::vector<int64_t>& sizes) const {
     t.sizes_ = s;
     OTTER_CHECK(t.numel() == numel(), "view: size mismatch");
     return t;
+}
+
+void Tensor::attach_quantized(const Tensor& q, float scale, int round_mode) {
+    OTTER_CHECK(defined() && q.defined() && q.scalar_type() == ScalarType::Byte8, "attach_quantized: a Byte8 blob expected");
+    st_->q8 = q.st_;
+    st_->q8_sizes = q.sizes_;
+    st_->q8_scale = scale;
+    st_->q8_round = round_mode;
+}
+
+bool Tensor::quantized_twin(float scale, int round_mode, Tensor& q) const {
+    if (!defined() || !st_->q8 || st_->q8_scale != scale || st_->q8_round != round_mode) return false;
+    q.st_ = st_->q8;
+    q.sizes_ = st_->q8_sizes;
+    q.dtype_ = ScalarType::Byte8;
+    return true;
 }
 
 Tensor Tensor::packing(int p) const {
@@ -534,6 +554,11 @@ int ConvolutionLayer::create_pipeline(const NetOption& opt) {
     return -1;  // fp32 convolution: outside the accelerated path
 }
 
+// which rounding primitive the reference's quantize of this layer's input ends in (Tensor/QuantizeX86.cpp:402)
+int ConvolutionLayer::input_round_mode(const NetOption& opt) const {
+    return (opt.use_packing_layout && in_channels % 8 == 0) ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT;
+}
+
 // Tensor/ConvolutionLayer.cpp:666-752: scale_in on the host (true division), weights re-laid-out once
 int ConvolutionLayer::create_pipeline_int8(const NetOption& opt) {
     OTTER_CHECK(weight_data_int8_scales.defined() && bottom_blob_int8_scales.defined(),
@@ -554,7 +579,7 @@ int ConvolutionLayer::create_pipeline_int8(const NetOption& opt) {
     // which rounding primitive the reference's routing ends in (Tensor/QuantizeX86.cpp:402,1177-1179,1729)
     const bool pk = opt.use_packing_layout;
     const bool dw8 = in_channels == groups && groups == out_channels && in_channels % 8 == 0;
-    d.in_round_mode = (pk && in_channels % 8 == 0) ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT;
+    d.in_round_mode = input_round_mode(opt);
     d.out_round_mode = (pk && (dw8 || out_channels % 4 == 0)) ? OTTER_HIP_ROUND_SSE : OTTER_HIP_ROUND_EXACT;
     if (handle_) {
         otter_hip_conv_destroy(handle_);
@@ -573,8 +598,13 @@ int ConvolutionLayer::forward(const Tensor& bottom, Tensor& top, const NetOption
 }
 
 // Tensor/ConvolutionLayer.cpp:754-847, whole batch in one launch
-int ConvolutionLayer::forward_int8(const Tensor& bottom, Tensor& top, const NetOption& opt) const {
-    if (!handle_ || !bottom.defined() || bottom.dim() != 4) return -1;
+int ConvolutionLayer::forward_int8(const Tensor& bottom_in, Tensor& top, const NetOption& opt) const {
+    if (!handle_ || !bottom_in.defined() || bottom_in.dim() != 4) return -1;
+    // the producer may already have quantized this blob with this layer's scale (see Net::plan_fused_quantize)
+    Tensor bottom = bottom_in, twin;
+    if (base_of(bottom_in.scalar_type()) == ScalarType::Float && in_channels % 8 == 0 &&
+        bottom_in.quantized_twin(bottom_blob_int8_scales.data_ptr<float>()[0], input_round_mode(opt), twin))
+        bottom = twin;
     const int in_layout = hip_layout_of(bottom.scalar_type());
     if (in_layout < 0 || base_of(bottom.scalar_type()) == ScalarType::Int) return -1;
     const int N = (int)bottom.size(0), H = (int)bottom.size(2), W = (int)bottom.size(3);
@@ -776,6 +806,21 @@ public:
             if (base_of(b[i].scalar_type()) != ScalarType::Float || b[i].channels() != acc.channels()) return -1;
             Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
             Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
+            const bool last = i + 1 == b.size();
+            if (last && fuse_scale > 0.f && acc.dim() == 4 && acc.channels() % 8 == 0 && (acc.elempack() == 4 || acc.elempack() == 8)) {
+                // the readers are int8 convolutions: hand them the quantized blob along with the sum
+                Tensor q = Tensor::empty_device({acc.size(0), acc.channels() / 8, acc.size(2), acc.size(3)}, ScalarType::Byte8);
+                if (otter_hip_eltwise_add_quantize((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(),
+                                                   hip_layout_of(acc.scalar_type()), (int)acc.size(0), (int)acc.channels(),
+                                                   (int)acc.size(2), (int)acc.size(3), fuse_scale, fuse_round,
+                                                   (float*)out.device_ptr(), (int8_t*)q.device_ptr(), nullptr))
+                    return -1;
+                out.mark_device_written();
+                q.mark_device_written();
+                out.attach_quantized(q, fuse_scale, fuse_round);
+                acc = out;
+                continue;
+            }
             if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
                                       (size_t)acc.numel() * acc.elempack(), nullptr))
                 return -1;
@@ -786,6 +831,8 @@ public:
         return 0;
     }
     std::string type() const override { return "Eltwise"; }
+    float fuse_scale = 0.f;  // > 0: also quantize the sum with this scale (set by Net::plan_fused_quantize)
+    int fuse_round = 0;
 };
 
 class SplitLayer : public Layer {  // Tensor/SplitLayer.cpp: every top shares the bottom blob
@@ -1375,6 +1422,7 @@ std::string Net::describe() const {
 
 // Tensor/Net.cpp:588-611: every layer reads its tensors from the stream in order, then builds its pipeline
 int Net::load_weight(const Initializer& initializer) {
+    planned_ = false;
     for (Layer* l : layers_) {
         int rc = l->load_model(initializer);
         if (rc) return rc;
@@ -1431,7 +1479,43 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
     return 0;
 }
 
-Extractor Net::create_extractor() const { return Extractor(this, blobs_.size()); }
+// An Eltwise sum that feeds int8 convolutions is quantized by each of them before anything else happens; when they
+// agree on the scale and the rounding primitive, the Eltwise layer does it on the way (one pass over the blob instead
+// of two, one launch less per reader). Readers behind the automatic Split layers count.
+void Net::plan_fused_quantize() const {
+    for (Layer* l : layers_) {
+        auto* e = dynamic_cast<EltwiseLayer*>(l);
+        if (!e) continue;
+        e->fuse_scale = 0.f;
+        std::vector<int> pending(e->tops.begin(), e->tops.end());
+        float scale = 0.f;
+        int round = 0;
+        bool agree = true;
+        while (!pending.empty()) {
+            const int b = pending.back();
+            pending.pop_back();
+            for (int ci : blobs_[b].consumers) {
+                const Layer* c = layers_[ci];
+                if (c->type() == "Split") {
+                    pending.insert(pending.end(), c->tops.begin(), c->tops.end());
+                } else if (const auto* conv = dynamic_cast<const ConvolutionLayer*>(c)) {
+                    if (!conv->int8_scale_term || !conv->bottom_blob_int8_scales.defined() || conv->in_channels % 8) continue;
+                    const float s = conv->bottom_blob_int8_scales.data_ptr<float>()[0];
+                    const int r = conv->input_round_mode(option);
+                    if (scale != 0.f && (s != scale || r != round)) agree = false;
+                    scale = s, round = r;
+                }
+            }
+        }
+        if (agree && scale > 0.f) e->fuse_scale = scale, e->fuse_round = round;
+    }
+    planned_ = true;
+}
+
+Extractor Net::create_extractor() const {
+    if (!planned_) plan_fused_quantize();
+    return Extractor(this, blobs_.size());
+}
 
 Extractor::Extractor(const Net* net, size_t blob_count) : option(net->option), net_(net), blob_tensors_(blob_count) {}
 

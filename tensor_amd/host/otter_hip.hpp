@@ -72,6 +72,11 @@ public:
     bool on_device() const;         // a valid device copy exists
     void mark_device_written();     // the device copy is now the fresh one
 
+    // An fp32 blob may carry its own int8 quantization (Byte8, made by the layer that produced the blob in the same
+    // pass): a convolution whose input scale and rounding primitive match reads that instead of quantizing again.
+    void attach_quantized(const Tensor& q, float scale, int round_mode);
+    bool quantized_twin(float scale, int round_mode, Tensor& q) const;
+
 private:
     struct Storage;
     std::shared_ptr<Storage> st_;
@@ -198,6 +203,8 @@ public:
     // when set, forward() produces fp32 even if int8_scale_term > 100 is absent etc.; -1 = the reference's rule
     int force_out_layout = -1;
 
+    int input_round_mode(const NetOption& opt) const;
+
 private:
     int create_pipeline_int8(const NetOption& opt);
     int forward_int8(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const;
@@ -252,6 +259,10 @@ public:
     int load_weight(FILE* f, WeightType type = WeightType::Otter);
     int load_weight(const Initializer& initializer);
     Extractor create_extractor() const;
+    // Tells every Eltwise layer whose sum is read by int8 convolutions which scale to quantize it with on the way
+    // (runs by itself before the first pass after the convolutions' scales changed).
+    void plan_fused_quantize() const;
+    void invalidate_plan() { planned_ = false; }
     const std::vector<std::string> blob_names() const;
     std::string describe() const;  // one line per layer: type, name, bottoms, tops, top shape, convolution weights
     int find_blob_index_by_name(const std::string& name) const;
@@ -270,6 +281,7 @@ private:
     std::vector<Layer*> layers_;
     std::vector<Blob> blobs_;
     std::vector<LayerOption> layer_options_;
+    mutable bool planned_ = false;
 };
 
 class Extractor {

@@ -93,6 +93,44 @@ def test_net_residual_block_with_auto_split(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("same_scale", [True, False], ids=["readers_agree", "readers_disagree"])
+def test_sum_feeding_int8_convolutions_is_quantized_on_the_way(oracle, same_scale):
+    """An Eltwise sum read by int8 convolutions (here two, behind an automatic Split, plus a second Eltwise that needs
+    the fp32 sum itself) carries its own quantization when the readers agree on the input scale; whether they do or
+    not, every blob equals the oracle's layer-by-layer computation."""
+    rng = np.random.default_rng(17)
+    C, K = 24, 16
+    x = rng.uniform(-1, 1, (3, C, 9, 11)).astype(np.float32)
+    wp, sp = _qweights(rng, C, C, 1)
+    wa, sa = _qweights(rng, K, C, 3)
+    wb, sb = _qweights(rng, C, C, 1)
+    bp, ba, bb = (rng.normal(0, 0.1, n).astype(np.float32) for n in (C, K, C))
+    in_p = np.float32(127) / np.abs(x).max()
+    net = hostnet.Net(lightmode=False)
+    net.add_layer(type="Input", name="data", batchsize=3, channel=C, height=9, width=11)
+    net.add_layer(type="Convolution", name="p", input="data", out_channels=C, kernel=1, int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="sum", input="data,p")
+    net.add_layer(type="Convolution", name="a", input="sum", out_channels=K, kernel=3, padding=1, int8_scale_term=102,
+                  activation="Relu")
+    net.add_layer(type="Convolution", name="b", input="sum", out_channels=C, kernel=1, int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="sum2", input="sum,b")
+    net.compile()
+    yp = oracle.conv_layer_forward(x, wp, sp, in_p, bias=bp)
+    s1 = yp + x
+    in_a = np.float32(127) / np.abs(s1).max()
+    in_b = in_a if same_scale else np.float32(in_a * 0.75)
+    net.set_conv("p", wp, bp, sp, in_p)
+    net.set_conv("a", wa, ba, sa, in_a, 9.0)
+    net.set_conv("b", wb, bb, sb, in_b)
+    ya = oracle.conv_layer_forward(s1, wa, sa, in_a, pad=(1, 1), bias=ba, top_scale=9.0, int8_out=True, act_type=1)
+    yb = oracle.conv_layer_forward(s1, wb, sb, in_b, bias=bb)
+    np.testing.assert_allclose(net.run("data", x, "sum"), s1, rtol=1e-5, atol=1e-30)
+    np.testing.assert_array_equal(net.run("data", x, "a"), ya)
+    np.testing.assert_allclose(net.run("data", x, "b"), yb, rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(net.run("data", x, "sum2"), s1 + yb, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.gpu
 def test_functional_api_matches_oracle(oracle):
     rng = np.random.default_rng(8)
     for (C, K, k, s, p, g, i8) in [(16, 16, 3, 1, 1, 1, True), (32, 32, 3, 2, 1, 32, True), (8, 12, 1, 1, 0, 1, False)]:

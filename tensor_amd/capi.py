@@ -67,7 +67,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_workspace_bytes", "otter_hip_conv_forward", "otter_hip_conv_kernel_kind",
            "otter_hip_quantize", "otter_hip_dequantize", "otter_hip_requantize", "otter_hip_repack",
            "otter_hip_conv_set_tile", "otter_hip_eltwise_add", "otter_hip_activation", "otter_hip_global_avgpool",
-           "otter_hip_inner_product"]
+           "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
+           "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d"]
 
 
 def load_cdll():
@@ -150,6 +151,42 @@ class Library:
         self._check(self.lib.otter_hip_repack(self.ptr(src), src_layout, n, c, h, w, self.ptr(dst), dst_layout,
                                               self.stream()))
         return dst
+
+    # -- fp32 layout glue (device tensors in packed storage; every op takes any fp32 layout on either side) ------
+    def copy_channels(self, src, src_layout, src_c, src_c0, dst, dst_layout, dst_c, dst_c0, count, n, h, w):
+        self._check(self.lib.otter_hip_copy_channels(self.ptr(src), src_layout, src_c, src_c0, self.ptr(dst), dst_layout,
+                                                     dst_c, dst_c0, count, n, h, w, self.stream()))
+        return dst
+
+    def channel_shuffle(self, src, src_layout, shape, groups, dst_layout):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, np.float32)
+        self._check(self.lib.otter_hip_channel_shuffle(self.ptr(src), src_layout, self.ptr(dst), dst_layout, n, c, h, w,
+                                                       groups, self.stream()))
+        return dst
+
+    def maxpool2d(self, src, src_layout, shape, kernel, stride, pad, dil, out_hw, pad_value, dst_layout):
+        n, c, h, w = shape
+        dst = self.empty(n * c * out_hw[0] * out_hw[1], np.float32)
+        self._check(self.lib.otter_hip_maxpool2d(self.ptr(src), src_layout, n, c, h, w, kernel[0], kernel[1], stride[0],
+                                                 stride[1], pad[0], pad[1], dil[0], dil[1], out_hw[0], out_hw[1],
+                                                 C.c_float(pad_value), self.ptr(dst), dst_layout, self.stream()))
+        return dst
+
+    def upsample2d(self, src, src_layout, shape, out_hw, mode, align_corner, dst_layout):
+        n, c, h, w = shape
+        dst = self.empty(n * c * out_hw[0] * out_hw[1], np.float32)
+        self._check(self.lib.otter_hip_upsample2d(self.ptr(src), src_layout, n, c, h, w, out_hw[0], out_hw[1], mode,
+                                                  int(align_corner), self.ptr(dst), dst_layout, self.stream()))
+        return dst
+
+    def eltwise_add_quantize(self, a, b, layout, shape, scale, round_mode):
+        n, c, h, w = shape
+        out = self.empty(n * c * h * w, np.float32)
+        q = self.empty(n * c * h * w, np.int8)
+        self._check(self.lib.otter_hip_eltwise_add_quantize(self.ptr(a), self.ptr(b), layout, n, c, h, w, C.c_float(scale),
+                                                            round_mode, self.ptr(out), self.ptr(q), self.stream()))
+        return out, q
 
     def conv(self, **kw):
         return Conv(self, **kw)

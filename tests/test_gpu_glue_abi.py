@@ -1,0 +1,115 @@
+"""The fp32 glue entry points of the C ABI called directly, with every combination of source and destination layout
+(elempack 1, 4, 8), against numpy / torch definitions: the host layer only ever uses a few of these combinations."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tensor_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+F32 = {1: capi.F32, 4: capi.F32_P4, 8: capi.F32_P8}
+
+
+def _dev(hip, a, p):
+    return hip.to_device(capi.pack_np(a, p))
+
+
+def _host(t, p, shape):
+    return capi.unpack_np(t.cpu().numpy(), p, shape)
+
+
+@pytest.mark.parametrize("ps,pd", list(itertools.product([1, 4, 8], repeat=2)))
+def test_copy_channels_every_layout_pair(hip, ps, pd):
+    rng = np.random.default_rng(10 * ps + pd)
+    N, Cs, Cd, H, W = 3, 24, 40, 5, 7
+    src = rng.normal(0, 1, (N, Cs, H, W)).astype(np.float32)
+    base = rng.normal(0, 1, (N, Cd, H, W)).astype(np.float32)
+    for s0, d0, cnt in [(0, 0, 24), (8, 16, 16), (4, 8, 8), (3, 5, 7), (0, 39, 1)]:
+        dst = _dev(hip, base, pd)
+        hip.copy_channels(_dev(hip, src, ps), F32[ps], Cs, s0, dst, F32[pd], Cd, d0, cnt, N, H, W)
+        want = base.copy()
+        want[:, d0:d0 + cnt] = src[:, s0:s0 + cnt]
+        np.testing.assert_array_equal(_host(dst, pd, base.shape), want, err_msg=str((s0, d0, cnt)))
+
+
+@pytest.mark.parametrize("ps,pd", list(itertools.product([1, 4, 8], repeat=2)))
+@pytest.mark.parametrize("groups", [2, 3, 8])
+def test_channel_shuffle(hip, ps, pd, groups):
+    rng = np.random.default_rng(groups)
+    shape = (2, 48, 6, 5)
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    got = _host(hip.channel_shuffle(_dev(hip, x, ps), F32[ps], shape, groups, F32[pd]), pd, shape)
+    want = F.channel_shuffle(torch.from_numpy(x), groups).numpy()
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("ps,pd", [(1, 1), (4, 8), (8, 4), (8, 8), (1, 8)])
+@pytest.mark.parametrize("k,s,p,d,ceil", [((3, 3), (2, 2), (1, 1), (1, 1), False), ((2, 2), (2, 2), (0, 0), (1, 1), False),
+                                          ((3, 2), (1, 2), (1, 0), (2, 1), False), ((3, 3), (2, 2), (1, 1), (1, 1), True)])
+def test_maxpool_both_paddings(hip, ps, pd, k, s, p, d, ceil):
+    rng = np.random.default_rng(3)
+    shape = (2, 16, 11, 14)
+    x = (rng.normal(0, 1, shape) - 1.5).astype(np.float32)  # mostly negative: the padding value shows
+    t = torch.from_numpy(x)
+    want_inf = F.max_pool2d(t, k, s, p, d, ceil_mode=ceil).numpy()
+    oh, ow = want_inf.shape[2:]
+    got = _host(hip.maxpool2d(_dev(hip, x, ps), F32[ps], shape, k, s, p, d, (oh, ow), -np.inf, F32[pd]), pd, want_inf.shape)
+    np.testing.assert_array_equal(got, want_inf)
+    if not ceil and d == (1, 1):
+        # zero padding = pooling the explicitly zero-padded blob without padding
+        want_zero = F.max_pool2d(F.pad(t, (p[1], p[1], p[0], p[0])), k, s, 0, d).numpy()
+        got0 = _host(hip.maxpool2d(_dev(hip, x, ps), F32[ps], shape, k, s, p, d, (oh, ow), 0.0, F32[pd]), pd, want_zero.shape)
+        np.testing.assert_array_equal(got0, want_zero)
+
+
+@pytest.mark.parametrize("ps,pd", [(1, 1), (4, 8), (8, 8)])
+def test_upsample_against_torch(hip, ps, pd):
+    """Bilinear with half-pixel centres and nearest by floor(d * in/out) are torch's definitions too; bilinear agrees to
+    rounding (the reference's operation order is reproduced exactly, torch's differs), nearest exactly."""
+    rng = np.random.default_rng(4)
+    shape = (2, 8, 5, 7)
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    t = torch.from_numpy(x)
+    for oh, ow in [(10, 14), (15, 21), (7, 9)]:
+        got = _host(hip.upsample2d(_dev(hip, x, ps), F32[ps], shape, (oh, ow), 2, False, F32[pd]), pd, (2, 8, oh, ow))
+        want = F.interpolate(t, size=(oh, ow), mode="bilinear", align_corners=False).numpy()
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)  # torch weights the taps in another order
+        gotn = _host(hip.upsample2d(_dev(hip, x, ps), F32[ps], shape, (oh, ow), 1, False, F32[pd]), pd, (2, 8, oh, ow))
+        wantn = F.interpolate(t, size=(oh, ow), mode="nearest").numpy()
+        np.testing.assert_array_equal(gotn, wantn)
+    got = _host(hip.upsample2d(_dev(hip, x, ps), F32[ps], shape, (10, 14), 2, True, F32[pd]), pd, (2, 8, 10, 14))
+    want = F.interpolate(t, size=(10, 14), mode="bilinear", align_corners=True).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)  # torch weights the taps in another order
+
+
+@pytest.mark.parametrize("p", [4, 8])
+@pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT])
+def test_eltwise_add_quantize(hip, oracle, p, mode):
+    rng = np.random.default_rng(p)
+    shape = (3, 24, 7, 9)
+    a = rng.normal(0, 1, shape).astype(np.float32)
+    b = rng.normal(0, 1, shape).astype(np.float32)
+    b.reshape(-1)[:64] = (np.arange(64) - 32 + 0.5) / np.float32(37.5) - a.reshape(-1)[:64]  # sums on rounding ties
+    out, q = hip.eltwise_add_quantize(_dev(hip, a, p), _dev(hip, b, p), F32[p], shape, 37.5, mode)
+    s = a + b
+    np.testing.assert_array_equal(_host(out, p, shape), s)
+    want_q = oracle.quantize(s, [37.5], mode)
+    np.testing.assert_array_equal(_host(q, 8, shape), want_q)
+
+
+def test_glue_argument_errors(hip):
+    x = hip.to_device(np.zeros(8 * 16, np.float32))
+    with pytest.raises(capi.HipError):
+        hip.copy_channels(x, capi.F32, 8, 4, x, capi.F32, 8, 0, 8, 1, 4, 4)          # range beyond the source
+    with pytest.raises(capi.HipError):
+        hip.channel_shuffle(x, capi.F32, (1, 8, 4, 4), 3, capi.F32)                  # groups do not divide C
+    with pytest.raises(capi.HipError):
+        hip.upsample2d(x, capi.F32, (1, 8, 4, 4), (8, 8), 3, False, capi.F32)        # bicubic is not supported
+    with pytest.raises(capi.HipError):
+        hip.maxpool2d(x, capi.F32, (1, 8, 4, 4), (3, 3), (2, 2), (1, 1), (1, 1), (9, 9), 0.0, capi.F32)  # output too large
+    with pytest.raises(capi.HipError):
+        hip.eltwise_add_quantize(x, x, capi.F32, (1, 8, 4, 4), 1.0, capi.ROUND_SSE)  # unpacked blobs

@@ -195,10 +195,10 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             std::vector<int32_t> wm(dw_packed_weight_bytes(C, d.kernel_h, d.kernel_w) / sizeof(int32_t));
             dw_pack_weights(weight, C, d.kernel_h, d.kernel_w, wm.data());
             if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
-            if (d.kernel_h == 3 && d.kernel_w == 3 && d.stride_h == d.stride_w && (d.stride_w == 1 || d.stride_w == 2) &&
-                d.pad_w <= 1) {
-                std::vector<int8_t> wa(dw_mfma_weight_bytes(C, d.stride_w));
-                dw_mfma_pack_weights(weight, C, d.stride_w, d.pad_w, wa.data());
+            if (d.kernel_h == d.kernel_w && (d.kernel_h == 3 || d.kernel_h == 5) && d.stride_h == d.stride_w &&
+                (d.stride_w == 1 || d.stride_w == 2) && dw_mfma_window_fits(d.kernel_w, d.stride_w, d.pad_w)) {
+                std::vector<int8_t> wa(dw_mfma_weight_bytes(C, d.stride_w, d.kernel_w));
+                dw_mfma_pack_weights(weight, C, d.stride_w, d.pad_w, d.kernel_w, wa.data());
                 if ((rc = upload<int8_t>(&h->w_dw_mfma, wa.data(), wa.size(), wa.size(), 0))) break;
             }
         } else if (g == 1 && C % 8 == 0) {

@@ -30,17 +30,24 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned v4u_store __attribute__((__vector_size__(4 * sizeof(unsigned))));
 typedef unsigned v2u_store __attribute__((__vector_size__(2 * sizeof(unsigned))));
 
-// weight [C, 1, 3, 3] int8 -> A operands [C/8 octets][kernel row 3][set T][lane 64][16 bytes], T = 2 for stride 1
+// weight [C, 1, ks, ks] int8 (ks = 3 or 5) -> A operands [C/8 octets][kernel row ks][set T][lane 64][16 bytes], T = 2 for stride 1
 // (set t = channels 4t..4t+3) and 1 for stride 2. Lane (r = lane % 16, g = lane / 16) holds A[row r][16g .. 16g+15];
 // reduction byte 16g + 8e + j is (input pixel 4n-2+2g+e, channel j).
 static int dw_mfma_sets(int stride) { return stride == 1 ? 2 : 1; }
-size_t dw_mfma_weight_bytes(int C, int stride) { return (size_t)(C / 8) * 3 * dw_mfma_sets(stride) * 64 * 16; }
+size_t dw_mfma_weight_bytes(int C, int stride, int ks) { return (size_t)(C / 8) * ks * dw_mfma_sets(stride) * 64 * 16; }
 
-void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t* dst) {
+// The 8 input pixels 4n-2 .. 4n+5 of a column must cover the windows of its 4 (stride 1) or 2 (stride 2) outputs:
+// with pad_w columns of padding the window of output phase p starts at pixel slot 2 + stride*p - pad_w.
+bool dw_mfma_window_fits(int ks, int stride, int pad_w) {
+    const int phases = 4 / stride;
+    return 2 - pad_w >= 0 && (ks - 1) + 2 + stride * (phases - 1) - pad_w <= 7;
+}
+
+void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks, int8_t* dst) {
     const int T = dw_mfma_sets(stride);
-    std::fill(dst, dst + dw_mfma_weight_bytes(C, stride), (int8_t)0);
+    std::fill(dst, dst + dw_mfma_weight_bytes(C, stride, ks), (int8_t)0);
     for (int o = 0; o < C / 8; ++o)
-        for (int dy = 0; dy < 3; ++dy)
+        for (int dy = 0; dy < ks; ++dy)
             for (int t = 0; t < T; ++t)
                 for (int lane = 0; lane < 64; ++lane) {
                     const int r = lane % 16, g = lane / 16;
@@ -50,9 +57,9 @@ void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t*
                     for (int e = 0; e < 2; ++e) {
                         // input pixel 4n - 2 + 2g + e feeds output pixel (4/stride) n + p through tap dx
                         const int dx = 2 * g + e - 2 - stride * p + pad_w;
-                        if (dx < 0 || dx > 2) continue;
-                        dst[((((size_t)o * 3 + dy) * T + t) * 64 + lane) * 16 + 8 * e + c] =
-                            w[(size_t)(8 * o + c) * 9 + dy * 3 + dx];
+                        if (dx < 0 || dx >= ks) continue;
+                        dst[((((size_t)o * ks + dy) * T + t) * 64 + lane) * 16 + 8 * e + c] =
+                            w[(size_t)(8 * o + c) * ks * ks + dy * ks + dx];
                     }
                 }
 }
@@ -116,7 +123,7 @@ __device__ __forceinline__ v4i dw_dequant4(const Epilogue& ep, const v4i& acc, c
 // down `rps` output rows. The input rows live in a ring of 8 register fragments: a step computes 8/S output rows
 // from the ring and refills every slot as soon as its last reader has issued, so the loads run 5 input rows ahead of
 // the matrix instructions for the whole walk. Narrow images sit side by side in the wave (`lpi` lane columns each).
-template <int S, int EPI, bool ODDW>
+template <int S, int EPI, bool ODDW, int KS>
 __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wa,
                                                               void* __restrict__ out, ConvGeom g, Epilogue ep,
                                                               int n_strips, int rps, int col_chunks, int lpi, int ipw,
@@ -149,7 +156,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
 
     const int oy0 = strip * rps;
     const int iy0 = oy0 * S - g.ph;
-    const int rows_needed = (min(rps, g.OH - oy0) - 1) * S + 3;  // input rows this strip really reads
+    const int rows_needed = (min(rps, g.OH - oy0) - 1) * S + KS;  // input rows this strip really reads
     auto load_row = [&](int j) -> v4i {  // j: input row relative to iy0; rows outside the image or the strip read zero
         const int iy = iy0 + j;
         const bool ok = iy >= 0 && iy < g.H && j < rows_needed;  // wave-uniform
@@ -167,11 +174,11 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
 #pragma unroll
     for (int j = 0; j < RING; ++j) frag[j] = load_row(j);
 
-    v4i a[3][T];
+    v4i a[KS][T];
     {
-        const v4i* ap = reinterpret_cast<const v4i*>(wa) + (size_t)o * 3 * T * 64 + lane;
+        const v4i* ap = reinterpret_cast<const v4i*>(wa) + (size_t)o * KS * T * 64 + lane;
 #pragma unroll
-        for (int dy = 0; dy < 3; ++dy)
+        for (int dy = 0; dy < KS; ++dy)
 #pragma unroll
             for (int t = 0; t < T; ++t) a[dy][t] = ap[(dy * T + t) * 64];
     }
@@ -230,7 +237,7 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
         for (int t = 0; t < T; ++t) {
             acc[t] = v4i{0, 0, 0, 0};
 #pragma unroll
-            for (int dy = 0; dy < 3; ++dy)
+            for (int dy = 0; dy < KS; ++dy)
                 acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[dy][t], frag[(u * S + dy) % RING], acc[t], 0, 0, 0);
         }
     };
@@ -327,8 +334,8 @@ int dw_mfma_epilogue(const Epilogue& ep, int K) {
 // true when this layer / batch can take the matrix-core kernel (the caller falls back to the vector kernels otherwise)
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive) {
     if (epi == EPI_I8_P8_NONNEG && !scale_out_positive) return false;  // the clamp is moved past the output scale
-    if (!(g.kh == 3 && g.kw == 3 && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2))) return false;
-    if (g.ph > 1 || g.pw > 1 || g.C % 8 != 0 || g.C != g.K) return false;
+    if (!(g.kh == g.kw && (g.kh == 3 || g.kh == 5) && g.dh == 1 && g.dw == 1 && g.sh == g.sw && (g.sh == 1 || g.sh == 2))) return false;
+    if (g.ph > g.kh / 2 || !dw_mfma_window_fits(g.kh, g.sh, g.pw) || g.C % 8 != 0 || g.C != g.K) return false;
     if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4 && epi != EPI_F32_P8) return false;
     const size_t in_bytes = (size_t)g.N * g.C * g.H * g.W;
     const size_t out_bytes = (size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1);
@@ -376,14 +383,21 @@ hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const 
     if (lds_reserve > 64 * 1024) lds_reserve = 64 * 1024;  // the default limit of dynamic LDS; still two per CU
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 || epi == EPI_F32_P8 ? 4 : 1));
+#define OHIP_DWM_K(S_, E_, O_)                                                                                         \
+    do {                                                                                                               \
+        if (g.kh == 3)                                                                                                 \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, O_, 3>), grid, block, lds_reserve, stream, x, wa, out, g, ep, \
+                               n_strips, rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                              \
+        else                                                                                                           \
+            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, O_, 5>), grid, block, lds_reserve, stream, x, wa, out, g, ep, \
+                               n_strips, rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                              \
+    } while (0)
 #define OHIP_DWM(S_, E_) \
     do {                                                                                                               \
         if (g.W & 1)                                                                                                   \
-            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, true>), grid, block, lds_reserve, stream, x, wa, out, g, ep, n_strips, \
-                               rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
+            OHIP_DWM_K(S_, E_, true);                                                                                  \
         else                                                                                                           \
-            hipLaunchKernelGGL((conv_dw3x3_mfma_kernel<S_, E_, false>), grid, block, lds_reserve, stream, x, wa, out, g, ep, n_strips, \
-                               rps, col_chunks, lpi, ipw, in_bytes, out_bytes);                                        \
+            OHIP_DWM_K(S_, E_, false);                                                                                 \
     } while (0)
 #define OHIP_DWM_E(S_)                                                \
     do {                                                              \
@@ -395,6 +409,7 @@ hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const 
     if (g.sh == 1) OHIP_DWM_E(1);
     else OHIP_DWM_E(2);
 #undef OHIP_DWM_E
+#undef OHIP_DWM_K
 #undef OHIP_DWM
     return hipGetLastError();
 }

@@ -24,8 +24,9 @@ hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void*
                            const Epilogue& ep, hipStream_t stream);
 
 // conv_dw.hip
-size_t dw_mfma_weight_bytes(int C, int stride);
-void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int8_t* dst);
+size_t dw_mfma_weight_bytes(int C, int stride, int ks);
+bool dw_mfma_window_fits(int ks, int stride, int pad_w);
+void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks, int8_t* dst);
 int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,

@@ -278,6 +278,30 @@ def test_depthwise3x3_every_strip_height(hip, oracle, family, s, shift):
                 assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("s", [1, 2])
+@pytest.mark.parametrize("family", [-2, -3], ids=["mfma", "valu"])
+def test_depthwise5x5_and_wide_padding(hip, oracle, family, s):
+    """The matrix-core depthwise kernel also takes a 5x5 window with pad 2 (the 8 input pixels of a column cover it)
+    and a 3x3 window with pad 2; checked like the 3x3 case, forced strips included, against the oracle and against
+    the vector-ALU family."""
+    rng = np.random.default_rng(50 + s)
+    for (C, N, H, W, k, p) in [(16, 2, 19, 70, 5, 2), (8, 5, 13, 9, 5, 2), (40, 3, 9, 21, 5, 2), (24, 2, 26, 26, 5, 2),
+                               (16, 2, 11, 12, 3, 2)]:
+        x, wq, ws, bias = _rand_problem(rng, C, C, k, C, N, H, W)
+        for act, int8_out, shift in ((3, True, 0), (0, True, 1), (2, False, 2)):
+            want = oracle.conv_layer_forward(x, wq, ws, 20.0, stride=(s, s), pad=(p, p), groups=C, bias=bias,
+                                             top_scale=9.0, int8_out=int8_out, act_type=act,
+                                             act_params=[0.1] if act == 2 else None)
+            out, kind = run_conv(hip, oracle, x, wq, ws, 20.0, stride=s, pad=p, groups=C, bias=bias, top_scale=9.0,
+                                 act=act, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32,
+                                 tile=(family, shift))
+            assert kind == 2
+            if int8_out:
+                np.testing.assert_array_equal(out, want, err_msg=str((C, N, H, W, k, act)))
+            else:
+                assert_f32_close(out, want)
+
+
 @pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,kind", [
     (64, 96, 3, 1, 1, 1, 2, 14, 16, 3),     # 3x3 LDS-halo kernel
     (48, 72, 1, 1, 0, 1, 2, 13, 11, 1),     # 1x1 implicit GEMM

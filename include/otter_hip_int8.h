@@ -219,6 +219,13 @@ int otter_hip_copy_channels(const float* src, int src_layout, int src_c, int src
 int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,
                               int groups, void* stream);
 
+/* The tail of a ShuffleNetV2 unit as the reference's model files spell it -- ConcatLayer(a, b) -> ChannelShuffleLayer with
+ * 2 groups -> two CropLayers taking the first and the second half of the channels (Tensor/ConcatLayer.cpp:54-67,
+ * Tensor/ChannelShuffleKernel.cpp:19-55, Tensor/CropLayer.cpp:69-75) -- in one pass: first_half[2j+i] = (i ? b : a)[j],
+ * second_half[2j+i] = (i ? b : a)[channels_each/2 + j]. All four blobs Float8 (OTTER_HIP_F32_P8), channels_each % 8 == 0. */
+int otter_hip_shuffle2_split(const float* a, const float* b, int n, int channels_each, int h, int w, float* first_half,
+                             float* second_half, void* stream);
+
 /* MaxPoolLayer::forward (Tensor/MaxPoolLayer.cpp:123-134): max over a kernel window of the padded input; out_h /
  * out_w as MaxPoolLayer::compute_output_shape gives them (Tensor/Pool.hpp:33-50). pad_value is what a tap outside
  * the image counts as: -INFINITY in the reference's generic kernel, 0 in its packed 3x3 and 2x2 stride-2 kernels,

@@ -68,7 +68,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_quantize", "otter_hip_dequantize", "otter_hip_requantize", "otter_hip_repack",
            "otter_hip_conv_set_tile", "otter_hip_eltwise_add", "otter_hip_activation", "otter_hip_global_avgpool",
            "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
-           "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d"]
+           "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split"]
 
 
 def load_cdll():
@@ -164,6 +164,13 @@ class Library:
         self._check(self.lib.otter_hip_channel_shuffle(self.ptr(src), src_layout, self.ptr(dst), dst_layout, n, c, h, w,
                                                        groups, self.stream()))
         return dst
+
+    def shuffle2_split(self, a, b, n, channels_each, h, w):
+        c1 = self.empty(n * channels_each * h * w, np.float32)
+        c2 = self.empty(n * channels_each * h * w, np.float32)
+        self._check(self.lib.otter_hip_shuffle2_split(self.ptr(a), self.ptr(b), n, channels_each, h, w, self.ptr(c1),
+                                                      self.ptr(c2), self.stream()))
+        return c1, c2
 
     def maxpool2d(self, src, src_layout, shape, kernel, stride, pad, dil, out_hw, pad_value, dst_layout):
         n, c, h, w = shape

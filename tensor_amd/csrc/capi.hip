@@ -562,6 +562,17 @@ int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int 
     return OTTER_HIP_OK;
 }
 
+int otter_hip_shuffle2_split(const float* a, const float* b, int n, int channels_each, int h, int w, float* first_half,
+                             float* second_half, void* stream) {
+    if (!a || !b || !first_half || !second_half) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shuffle2_split: null");
+    if (n < 0 || channels_each < 8 || channels_each % 8 || h < 1 || w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shuffle2_split: each input needs a multiple of 8 channels");
+    if ((size_t)n * channels_each * 2 * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_shuffle2_split: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_shuffle2_split(a, b, first_half, second_half, n, channels_each, h * w, (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_maxpool2d(const float* src, int src_layout, int n, int c, int h, int w, int kernel_h, int kernel_w,
                         int stride_h, int stride_w, int pad_h, int pad_w, int dilation_h, int dilation_w, int out_h,
                         int out_w, float pad_value, float* dst, int dst_layout, void* stream) {

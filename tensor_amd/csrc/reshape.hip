@@ -130,6 +130,38 @@ __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* _
     o[1] = make_float4(a.z, b.z, a.w, b.w);
 }
 
+// The ShuffleNetV2 unit tail in one pass: Concat(a, b) -> ChannelShuffle(2 groups) -> the two half Crops. With Ch channels
+// in a and in b, the shuffled blob alternates a[j], b[j]; its first Ch channels are output c1, the rest c2. All four
+// blobs in elempack 8; one thread per (image, pack of the shuffled blob, pixel).
+__global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                float* __restrict__ c1, float* __restrict__ c2, int Ch, int HW,
+                                                                unsigned total) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const unsigned r = i / (unsigned)HW;
+    const int px = (int)(i - r * (unsigned)HW);
+    const unsigned packs = (unsigned)(Ch / 4);  // packs of the shuffled blob (2*Ch channels)
+    const size_t n = r / packs;
+    const int q = (int)(r - (unsigned)n * packs);
+    const int cs = 4 * q;  // first source channel, in a and in b
+    const size_t src = (n * (size_t)(Ch / 8) + cs / 8) * HW * 8 + (size_t)px * 8 + cs % 8;
+    const float4 x = *reinterpret_cast<const float4*>(a + src), y = *reinterpret_cast<const float4*>(b + src);
+    const int half_packs = Ch / 8;
+    float* dst = q < half_packs ? c1 : c2;
+    const int qd = q < half_packs ? q : q - half_packs;
+    float4* o = reinterpret_cast<float4*>(dst + (n * (size_t)half_packs + qd) * HW * 8 + (size_t)px * 8);
+    o[0] = make_float4(x.x, y.x, x.y, y.y);
+    o[1] = make_float4(x.z, y.z, x.w, y.w);
+}
+
+hipError_t run_shuffle2_split(const float* a, const float* b, float* c1, float* c2, int N, int Ch, int HW, hipStream_t stream) {
+    const size_t total = (size_t)N * (Ch / 4) * HW;
+    if (total == 0) return hipSuccess;
+    hipLaunchKernelGGL(shuffle2_split_p8_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, b, c1, c2, Ch,
+                       HW, (unsigned)total);
+    return hipGetLastError();
+}
+
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
                                hipStream_t stream) {
     const size_t total = (size_t)N * C * H * W;

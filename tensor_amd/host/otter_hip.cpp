@@ -1035,6 +1035,8 @@ public:
         return 0;
     }
     std::string type() const override { return "Crop"; }
+    int start() const { return start_; }
+    int end() const { return end_; }
 
 private:
     int start_ = -1, end_ = -1;
@@ -1065,6 +1067,7 @@ public:
         return 0;
     }
     std::string type() const override { return "ChannelShuffle"; }
+    int groups() const { return groups_; }
 
 private:
     int groups_ = 1;
@@ -1447,6 +1450,18 @@ Layer* Net::layer_by_name(const std::string& name) const {
 // Tensor/Net.cpp:350-505: lazy, recursive, memoised in the extractor's blob table
 int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt) const {
     const Layer* layer = layers_[li];
+    {
+        const auto unit = shuffle_units_.find(li);
+        if (unit != shuffle_units_.end()) {
+            const ShuffleUnit& u = unit->second;
+            // only when nothing inside the unit has been computed (or set by the caller) yet
+            if (!blobs[layers_[u.concat]->tops[0]].defined() && !blobs[layers_[u.shuffle]->tops[0]].defined() &&
+                !blobs[layer->bottoms[0]].defined()) {
+                const int rc = forward_shuffle_unit(u, blobs, opt);
+                if (rc <= 0) return rc;
+            }
+        }
+    }
     for (int b : layer->bottoms)
         if (!blobs[b].defined()) {
             int rc = forward_layer(blobs_[b].producer, blobs, opt);
@@ -1509,7 +1524,61 @@ void Net::plan_fused_quantize() const {
         }
         if (agree && scale > 0.f) e->fuse_scale = scale, e->fuse_round = round;
     }
+    // ShuffleNetV2 unit tails: Concat of two equal blobs -> ChannelShuffle(2) -> exactly the two half Crops
+    shuffle_units_.clear();
+    auto sole_reader = [&](int blob) { return blobs_[blob].consumers.size() == 1 ? blobs_[blob].consumers[0] : -1; };
+    for (size_t ci = 0; ci < layers_.size(); ++ci) {
+        const Layer* cat = layers_[ci];
+        if (cat->type() != "Concat" || cat->bottoms.size() != 2 || cat->bottom_shapes[0] != cat->bottom_shapes[1]) continue;
+        const int64_t ch = cat->bottom_shapes[0][1];
+        if (ch % 8) continue;
+        const int si = sole_reader(cat->tops[0]);
+        const auto* sh = si < 0 ? nullptr : dynamic_cast<const ChannelShuffleLayer*>(layers_[si]);
+        if (!sh || sh->groups() != 2) continue;
+        int sp = sole_reader(sh->tops[0]);
+        if (sp < 0 || layers_[sp]->type() != "Split" || layers_[sp]->tops.size() != 2) continue;
+        int lo = -1, hi = -1;
+        for (int t : layers_[sp]->tops) {
+            const int r = sole_reader(t);
+            const auto* crop = r < 0 ? nullptr : dynamic_cast<const CropLayer*>(layers_[r]);
+            if (!crop) continue;
+            if (crop->start() == 0 && crop->end() == ch) lo = r;
+            if (crop->start() == ch && (crop->end() == 2 * ch || crop->end() == -1)) hi = r;
+        }
+        if (lo < 0 || hi < 0) continue;
+        const ShuffleUnit u{(int)ci, si, lo, hi};
+        shuffle_units_[lo] = u;
+        shuffle_units_[hi] = u;
+    }
     planned_ = true;
+}
+
+// One kernel for a whole unit (otter_hip_shuffle2_split) when the blobs between its ends are not wanted by anybody else.
+int Net::forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const {
+    const Layer* cat = layers_[u.concat];
+    for (int b : cat->bottoms)
+        if (!blobs[b].defined()) {
+            const int rc = forward_layer(blobs_[b].producer, blobs, opt);
+            if (rc) return rc;
+        }
+    Tensor a = blobs[cat->bottoms[0]], b = blobs[cat->bottoms[1]];
+    if (!f32_4d(a) || !f32_4d(b) || a.channels() != b.channels() || a.channels() % 8 || a.size(0) != b.size(0) ||
+        a.size(2) != b.size(2) || a.size(3) != b.size(3))
+        return 1;  // not the shapes the plan assumed: the caller falls back to the layers one by one
+    if (a.elempack() != 8) a = a.packing(8);
+    if (b.elempack() != 8) b = b.packing(8);
+    Tensor lo = Tensor::empty_device(a.sizes(), a.scalar_type()), hi = Tensor::empty_device(a.sizes(), a.scalar_type());
+    if (otter_hip_shuffle2_split((const float*)a.device_ptr(), (const float*)b.device_ptr(), (int)a.size(0), (int)a.channels(),
+                                 (int)a.size(2), (int)a.size(3), (float*)lo.device_ptr(), (float*)hi.device_ptr(), nullptr))
+        return -1;
+    lo.mark_device_written();
+    hi.mark_device_written();
+    blobs[layers_[u.crop_lo]->tops[0]] = lo;
+    blobs[layers_[u.crop_hi]->tops[0]] = hi;
+    if (opt.lightmode)
+        for (int bb : cat->bottoms)
+            if (blobs_[bb].consumers.size() == 1) blobs[bb] = Tensor();
+    return 0;
 }
 
 Extractor Net::create_extractor() const {

@@ -282,6 +282,13 @@ private:
     std::vector<Blob> blobs_;
     std::vector<LayerOption> layer_options_;
     mutable bool planned_ = false;
+    // Concat(a, b) -> ChannelShuffle(2) -> Crop(first half) + Crop(second half), found by the plan: either Crop layer's
+    // index -> the unit; forward_layer runs the whole unit in one kernel when none of its inner blobs exists yet
+    struct ShuffleUnit {
+        int concat, shuffle, crop_lo, crop_hi;
+    };
+    mutable std::map<int, ShuffleUnit> shuffle_units_;
+    int forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
 };
 
 class Extractor {

@@ -101,6 +101,19 @@ def test_eltwise_add_quantize(hip, oracle, p, mode):
     np.testing.assert_array_equal(_host(q, 8, shape), want_q)
 
 
+def test_shuffle2_split_is_concat_shuffle_and_two_crops(hip):
+    rng = np.random.default_rng(9)
+    N, Ch, H, W = 3, 24, 5, 9
+    a = rng.normal(0, 1, (N, Ch, H, W)).astype(np.float32)
+    b = rng.normal(0, 1, (N, Ch, H, W)).astype(np.float32)
+    c1, c2 = hip.shuffle2_split(_dev(hip, a, 8), _dev(hip, b, 8), N, Ch, H, W)
+    s = F.channel_shuffle(torch.from_numpy(np.concatenate([a, b], 1)), 2).numpy()
+    np.testing.assert_array_equal(_host(c1, 8, a.shape), s[:, :Ch])
+    np.testing.assert_array_equal(_host(c2, 8, a.shape), s[:, Ch:])
+    with pytest.raises(capi.HipError):
+        hip.shuffle2_split(_dev(hip, a[:, :12], 4), _dev(hip, b[:, :12], 4), N, 12, H, W)
+
+
 def test_glue_argument_errors(hip):
     x = hip.to_device(np.zeros(8 * 16, np.float32))
     with pytest.raises(capi.HipError):

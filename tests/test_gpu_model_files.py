@@ -137,6 +137,12 @@ GLUE_CASES = [
      ["s", "c1", "c2", "c3", "cat", "s2"]),
     ("shuffle_groups2_pack8", (48, 7, 9), _layer("ChannelShuffle", "s", ["data"], groups=2), ["s"]),
     ("shuffle_groups4", (16, 3, 5), _layer("ChannelShuffle", "s", ["data"], groups=4), ["s"]),
+    ("shufflenet_unit_tail", (32, 6, 7),
+     _layer("Crop", "a", ["data"], start=0, end=16, axis=1) + _layer("Crop", "b", ["data"], start=16, end=32, axis=1) +
+     _layer("MaxPool", "bp", ["b"], kernel=3, stride=1, padding=1) + _layer("Concat", "cat", ["a", "bp"], axis=1) +
+     _layer("ChannelShuffle", "s", ["cat"], groups=2) + _layer("Crop", "lo", ["s"], start=0, end=16, axis=1) +
+     _layer("Crop", "hi", ["s"], start=16, end=32, axis=1) + _layer("MaxPool", "out", ["hi"], kernel=3, stride=1, padding=1),
+     ["lo", "hi", "out", "s", "cat"]),   # lo / hi / out run the unit in one kernel, s / cat layer by layer
     ("crop_unaligned", (12, 4, 4), _layer("Crop", "c", ["data"], start=3, end=10, axis=1) +
      _layer("Concat", "cat", ["c", "data"], axis=1), ["c", "cat"]),
     ("shortcut", (16, 5, 5), _layer("MaxPool", "p", ["data"], kernel=3, stride=1, padding=1) +

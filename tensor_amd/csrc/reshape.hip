@@ -133,9 +133,11 @@ __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* _
 // The ShuffleNetV2 unit tail in one pass: Concat(a, b) -> ChannelShuffle(2 groups) -> the two half Crops. With Ch channels
 // in a and in b, the shuffled blob alternates a[j], b[j]; its first Ch channels are output c1, the rest c2. All four
 // blobs in elempack 8; one thread per (image, pack of the shuffled blob, pixel).
+// q2 (optional): the Byte8 quantization of c2 with `scale`, for an int8 convolution that reads c2 next.
 __global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                                float* __restrict__ c1, float* __restrict__ c2, int Ch, int HW,
-                                                                unsigned total) {
+                                                                float* __restrict__ c1, float* __restrict__ c2,
+                                                                int8_t* __restrict__ q2, float scale, float half, int Ch,
+                                                                int HW, unsigned total) {
     const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const unsigned r = i / (unsigned)HW;
@@ -152,13 +154,28 @@ __global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __r
     float4* o = reinterpret_cast<float4*>(dst + (n * (size_t)half_packs + qd) * HW * 8 + (size_t)px * 8);
     o[0] = make_float4(x.x, y.x, x.y, y.y);
     o[1] = make_float4(x.z, y.z, x.w, y.w);
+    if (q2 != nullptr && q >= half_packs) {
+        const float v[8] = {x.x, y.x, x.y, y.y, x.z, y.z, x.w, y.w};
+        int k[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float t = __fmul_rn(v[e], scale);
+            k[e] = min(max((int)__fadd_rn(t, __builtin_copysignf(half, t)), -127), 127) & 0xff;
+        }
+        ohip_v2i pk;
+        pk[0] = k[0] | (k[1] << 8) | (k[2] << 16) | (k[3] << 24);
+        pk[1] = k[4] | (k[5] << 8) | (k[6] << 16) | (k[7] << 24);
+        *reinterpret_cast<ohip_v2i*>(q2 + (n * (size_t)half_packs + qd) * HW * 8 + (size_t)px * 8) = pk;
+    }
 }
 
-hipError_t run_shuffle2_split(const float* a, const float* b, float* c1, float* c2, int N, int Ch, int HW, hipStream_t stream) {
+hipError_t run_shuffle2_split(const float* a, const float* b, float* c1, float* c2, int8_t* q2, float scale, int round_mode,
+                              int N, int Ch, int HW, hipStream_t stream) {
     const size_t total = (size_t)N * (Ch / 4) * HW;
     if (total == 0) return hipSuccess;
-    hipLaunchKernelGGL(shuffle2_split_p8_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, b, c1, c2, Ch,
-                       HW, (unsigned)total);
+    const float half = round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    hipLaunchKernelGGL(shuffle2_split_p8_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, b, c1, c2, q2,
+                       scale, half, Ch, HW, (unsigned)total);
     return hipGetLastError();
 }
 

@@ -1546,7 +1546,22 @@ void Net::plan_fused_quantize() const {
             if (crop->start() == ch && (crop->end() == 2 * ch || crop->end() == -1)) hi = r;
         }
         if (lo < 0 || hi < 0) continue;
-        const ShuffleUnit u{(int)ci, si, lo, hi};
+        // int8 convolutions reading the second half (the unit's next branch) and agreeing on the scale
+        float hs = 0.f;
+        int hr = 0;
+        bool agree = true;
+        for (int rc : blobs_[layers_[hi]->tops[0]].consumers) {
+            const auto* conv = dynamic_cast<const ConvolutionLayer*>(layers_[rc]);
+            if (!conv || !conv->int8_scale_term || !conv->bottom_blob_int8_scales.defined() || conv->in_channels % 8) {
+                agree = false;
+                continue;
+            }
+            const float sc = conv->bottom_blob_int8_scales.data_ptr<float>()[0];
+            const int r = conv->input_round_mode(option);
+            if (hs != 0.f && (sc != hs || r != hr)) agree = false;
+            hs = sc, hr = r;
+        }
+        const ShuffleUnit u{(int)ci, si, lo, hi, agree && hs > 0.f ? hs : 0.f, hr};
         shuffle_units_[lo] = u;
         shuffle_units_[hi] = u;
     }
@@ -1568,11 +1583,18 @@ int Net::forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, 
     if (a.elempack() != 8) a = a.packing(8);
     if (b.elempack() != 8) b = b.packing(8);
     Tensor lo = Tensor::empty_device(a.sizes(), a.scalar_type()), hi = Tensor::empty_device(a.sizes(), a.scalar_type());
+    Tensor hq;
+    if (u.hi_scale > 0.f) hq = Tensor::empty_device(a.sizes(), ScalarType::Byte8);
     if (otter_hip_shuffle2_split((const float*)a.device_ptr(), (const float*)b.device_ptr(), (int)a.size(0), (int)a.channels(),
-                                 (int)a.size(2), (int)a.size(3), (float*)lo.device_ptr(), (float*)hi.device_ptr(), nullptr))
+                                 (int)a.size(2), (int)a.size(3), (float*)lo.device_ptr(), (float*)hi.device_ptr(),
+                                 hq.defined() ? (int8_t*)hq.device_ptr() : nullptr, u.hi_scale, u.hi_round, nullptr))
         return -1;
     lo.mark_device_written();
     hi.mark_device_written();
+    if (hq.defined()) {
+        hq.mark_device_written();
+        hi.attach_quantized(hq, u.hi_scale, u.hi_round);
+    }
     blobs[layers_[u.crop_lo]->tops[0]] = lo;
     blobs[layers_[u.crop_hi]->tops[0]] = hi;
     if (opt.lightmode)

@@ -286,6 +286,8 @@ private:
     // index -> the unit; forward_layer runs the whole unit in one kernel when none of its inner blobs exists yet
     struct ShuffleUnit {
         int concat, shuffle, crop_lo, crop_hi;
+        float hi_scale;  // > 0: the second half is read by int8 convolutions with this input scale ...
+        int hi_round;    // ... and this rounding primitive: quantize it on the way
     };
     mutable std::map<int, ShuffleUnit> shuffle_units_;
     int forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;

@@ -110,6 +110,10 @@ def test_shuffle2_split_is_concat_shuffle_and_two_crops(hip):
     s = F.channel_shuffle(torch.from_numpy(np.concatenate([a, b], 1)), 2).numpy()
     np.testing.assert_array_equal(_host(c1, 8, a.shape), s[:, :Ch])
     np.testing.assert_array_equal(_host(c2, 8, a.shape), s[:, Ch:])
+    c1, c2, q2 = hip.shuffle2_split(_dev(hip, a, 8), _dev(hip, b, 8), N, Ch, H, W, scale=41.0, round_mode=capi.ROUND_SSE)
+    np.testing.assert_array_equal(_host(c2, 8, a.shape), s[:, Ch:])
+    t = s[:, Ch:] * np.float32(41.0)
+    np.testing.assert_array_equal(_host(q2, 8, a.shape), np.clip(np.trunc(t + np.copysign(np.float32(0.5), t)), -127, 127))
     with pytest.raises(capi.HipError):
         hip.shuffle2_split(_dev(hip, a[:, :12], 4), _dev(hip, b[:, :12], 4), N, 12, H, W)
 

@@ -222,11 +222,13 @@ int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int 
 /* The tail of a ShuffleNetV2 unit as the reference's model files spell it -- ConcatLayer(a, b) -> ChannelShuffleLayer with
  * 2 groups -> two CropLayers taking the first and the second half of the channels (Tensor/ConcatLayer.cpp:54-67,
  * Tensor/ChannelShuffleKernel.cpp:19-55, Tensor/CropLayer.cpp:69-75) -- in one pass: first_half[2j+i] = (i ? b : a)[j],
- * second_half[2j+i] = (i ? b : a)[channels_each/2 + j]. All four blobs Float8 (OTTER_HIP_F32_P8), channels_each % 8 == 0.
+ * second_half[2j+i] = (i ? b : a)[channels_each/2 + j]. The outputs are Float8 (OTTER_HIP_F32_P8), a and b each Float4 or
+ * Float8; channels_each % 8 == 0.
  * second_half_q (may be NULL): the Byte8 quantization of second_half, float2int8(v * scale) with round_mode, for the int8
  * convolution that reads that half next (its quantize_to_int8, Tensor/ConvolutionLayer.cpp:770-775). */
-int otter_hip_shuffle2_split(const float* a, const float* b, int n, int channels_each, int h, int w, float* first_half,
-                             float* second_half, int8_t* second_half_q, float scale, int round_mode, void* stream);
+int otter_hip_shuffle2_split(const float* a, int a_layout, const float* b, int b_layout, int n, int channels_each, int h,
+                             int w, float* first_half, float* second_half, int8_t* second_half_q, float scale,
+                             int round_mode, void* stream);
 
 /* MaxPoolLayer::forward (Tensor/MaxPoolLayer.cpp:123-134): max over a kernel window of the padded input; out_h /
  * out_w as MaxPoolLayer::compute_output_shape gives them (Tensor/Pool.hpp:33-50). pad_value is what a tap outside

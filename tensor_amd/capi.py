@@ -165,11 +165,11 @@ class Library:
                                                        groups, self.stream()))
         return dst
 
-    def shuffle2_split(self, a, b, n, channels_each, h, w, scale=None, round_mode=0):
+    def shuffle2_split(self, a, b, n, channels_each, h, w, scale=None, round_mode=0, a_layout=F32_P8, b_layout=F32_P8):
         c1 = self.empty(n * channels_each * h * w, np.float32)
         c2 = self.empty(n * channels_each * h * w, np.float32)
         q2 = self.empty(n * channels_each * h * w, np.int8) if scale is not None else None
-        self._check(self.lib.otter_hip_shuffle2_split(self.ptr(a), self.ptr(b), n, channels_each, h, w, self.ptr(c1),
+        self._check(self.lib.otter_hip_shuffle2_split(self.ptr(a), a_layout, self.ptr(b), b_layout, n, channels_each, h, w, self.ptr(c1),
                                                       self.ptr(c2), self.ptr(q2) if q2 is not None else None,
                                                       C.c_float(scale or 0.0), round_mode, self.stream()))
         return (c1, c2, q2) if scale is not None else (c1, c2)

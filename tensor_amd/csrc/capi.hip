@@ -562,15 +562,18 @@ int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int 
     return OTTER_HIP_OK;
 }
 
-int otter_hip_shuffle2_split(const float* a, const float* b, int n, int channels_each, int h, int w, float* first_half,
-                             float* second_half, int8_t* second_half_q, float scale, int round_mode, void* stream) {
+int otter_hip_shuffle2_split(const float* a, int a_layout, const float* b, int b_layout, int n, int channels_each, int h,
+                             int w, float* first_half, float* second_half, int8_t* second_half_q, float scale,
+                             int round_mode, void* stream) {
     if (!a || !b || !first_half || !second_half) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shuffle2_split: null");
+    if ((a_layout != OTTER_HIP_F32_P4 && a_layout != OTTER_HIP_F32_P8) || (b_layout != OTTER_HIP_F32_P4 && b_layout != OTTER_HIP_F32_P8))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shuffle2_split: Float4 or Float8 inputs expected");
     if (n < 0 || channels_each < 8 || channels_each % 8 || h < 1 || w < 1)
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shuffle2_split: each input needs a multiple of 8 channels");
     if ((size_t)n * channels_each * 2 * h * w >= (1ull << 31))
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_shuffle2_split: tensor exceeds 2^31 elements");
-    OHIP_CHECK(run_shuffle2_split(a, b, first_half, second_half, second_half_q, scale, round_mode, n, channels_each, h * w,
-                                  (hipStream_t)stream));
+    OHIP_CHECK(run_shuffle2_split(a, layout_pack(a_layout), b, layout_pack(b_layout), first_half, second_half, second_half_q,
+                                  scale, round_mode, n, channels_each, h * w, (hipStream_t)stream));
     return OTTER_HIP_OK;
 }
 

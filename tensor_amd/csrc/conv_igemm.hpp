@@ -71,8 +71,8 @@ hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* d
                              int H, int W, hipStream_t stream);
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
                                hipStream_t stream);
-hipError_t run_shuffle2_split(const float* a, const float* b, float* c1, float* c2, int8_t* q2, float scale, int round_mode,
-                              int N, int Ch, int HW, hipStream_t stream);
+hipError_t run_shuffle2_split(const float* a, int pa, const float* b, int pb, float* c1, float* c2, int8_t* q2, float scale,
+                              int round_mode, int N, int Ch, int HW, hipStream_t stream);
 hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int kh,
                        int kw, int sh, int sw, int ph, int pw, int dh, int dw, float pad_value, hipStream_t stream);
 hipError_t run_upsample(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int mode,

@@ -132,12 +132,12 @@ __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* _
 
 // The ShuffleNetV2 unit tail in one pass: Concat(a, b) -> ChannelShuffle(2 groups) -> the two half Crops. With Ch channels
 // in a and in b, the shuffled blob alternates a[j], b[j]; its first Ch channels are output c1, the rest c2. All four
-// blobs in elempack 8; one thread per (image, pack of the shuffled blob, pixel).
+// outputs in elempack 8, inputs in elempack 4 or 8 each; one thread per (image, pack of the shuffled blob, pixel).
 // q2 (optional): the Byte8 quantization of c2 with `scale`, for an int8 convolution that reads c2 next.
 __global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                                 float* __restrict__ c1, float* __restrict__ c2,
                                                                 int8_t* __restrict__ q2, float scale, float half, int Ch,
-                                                                int HW, unsigned total) {
+                                                                int HW, int pa, int pb, unsigned total) {
     const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const unsigned r = i / (unsigned)HW;
@@ -146,8 +146,10 @@ __global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __r
     const size_t n = r / packs;
     const int q = (int)(r - (unsigned)n * packs);
     const int cs = 4 * q;  // first source channel, in a and in b
-    const size_t src = (n * (size_t)(Ch / 8) + cs / 8) * HW * 8 + (size_t)px * 8 + cs % 8;
-    const float4 x = *reinterpret_cast<const float4*>(a + src), y = *reinterpret_cast<const float4*>(b + src);
+    // a and b may each be Float4 or Float8 (pa, pb): four consecutive channels are contiguous in both
+    const size_t sa = ((n * (size_t)(Ch / pa) + cs / pa) * HW + px) * pa + cs % pa;
+    const size_t sb = ((n * (size_t)(Ch / pb) + cs / pb) * HW + px) * pb + cs % pb;
+    const float4 x = *reinterpret_cast<const float4*>(a + sa), y = *reinterpret_cast<const float4*>(b + sb);
     const int half_packs = Ch / 8;
     float* dst = q < half_packs ? c1 : c2;
     const int qd = q < half_packs ? q : q - half_packs;
@@ -169,13 +171,13 @@ __global__ void __launch_bounds__(256) shuffle2_split_p8_kernel(const float* __r
     }
 }
 
-hipError_t run_shuffle2_split(const float* a, const float* b, float* c1, float* c2, int8_t* q2, float scale, int round_mode,
-                              int N, int Ch, int HW, hipStream_t stream) {
+hipError_t run_shuffle2_split(const float* a, int pa, const float* b, int pb, float* c1, float* c2, int8_t* q2, float scale,
+                              int round_mode, int N, int Ch, int HW, hipStream_t stream) {
     const size_t total = (size_t)N * (Ch / 4) * HW;
     if (total == 0) return hipSuccess;
     const float half = round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
     hipLaunchKernelGGL(shuffle2_split_p8_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, b, c1, c2, q2,
-                       scale, half, Ch, HW, (unsigned)total);
+                       scale, half, Ch, HW, pa, pb, (unsigned)total);
     return hipGetLastError();
 }
 

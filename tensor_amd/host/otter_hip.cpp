@@ -1580,12 +1580,14 @@ int Net::forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, 
     if (!f32_4d(a) || !f32_4d(b) || a.channels() != b.channels() || a.channels() % 8 || a.size(0) != b.size(0) ||
         a.size(2) != b.size(2) || a.size(3) != b.size(3))
         return 1;  // not the shapes the plan assumed: the caller falls back to the layers one by one
-    if (a.elempack() != 8) a = a.packing(8);
-    if (b.elempack() != 8) b = b.packing(8);
-    Tensor lo = Tensor::empty_device(a.sizes(), a.scalar_type()), hi = Tensor::empty_device(a.sizes(), a.scalar_type());
+    if (a.elempack() == 1) a = a.packing(8);
+    if (b.elempack() == 1) b = b.packing(8);
+    const std::vector<int64_t> out_sizes = {a.size(0), a.channels() / 8, a.size(2), a.size(3)};
+    Tensor lo = Tensor::empty_device(out_sizes, ScalarType::Float8), hi = Tensor::empty_device(out_sizes, ScalarType::Float8);
     Tensor hq;
-    if (u.hi_scale > 0.f) hq = Tensor::empty_device(a.sizes(), ScalarType::Byte8);
-    if (otter_hip_shuffle2_split((const float*)a.device_ptr(), (const float*)b.device_ptr(), (int)a.size(0), (int)a.channels(),
+    if (u.hi_scale > 0.f) hq = Tensor::empty_device(out_sizes, ScalarType::Byte8);
+    if (otter_hip_shuffle2_split((const float*)a.device_ptr(), hip_layout_of(a.scalar_type()), (const float*)b.device_ptr(),
+                                 hip_layout_of(b.scalar_type()), (int)a.size(0), (int)a.channels(),
                                  (int)a.size(2), (int)a.size(3), (float*)lo.device_ptr(), (float*)hi.device_ptr(),
                                  hq.defined() ? (int8_t*)hq.device_ptr() : nullptr, u.hi_scale, u.hi_round, nullptr))
         return -1;

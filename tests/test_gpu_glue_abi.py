@@ -114,6 +114,9 @@ def test_shuffle2_split_is_concat_shuffle_and_two_crops(hip):
     np.testing.assert_array_equal(_host(c2, 8, a.shape), s[:, Ch:])
     t = s[:, Ch:] * np.float32(41.0)
     np.testing.assert_array_equal(_host(q2, 8, a.shape), np.clip(np.trunc(t + np.copysign(np.float32(0.5), t)), -127, 127))
+    c1, c2 = hip.shuffle2_split(_dev(hip, a, 4), _dev(hip, b, 8), N, Ch, H, W, a_layout=capi.F32_P4)
+    np.testing.assert_array_equal(_host(c1, 8, a.shape), s[:, :Ch])
+    np.testing.assert_array_equal(_host(c2, 8, a.shape), s[:, Ch:])
     with pytest.raises(capi.HipError):
         hip.shuffle2_split(_dev(hip, a[:, :12], 4), _dev(hip, b[:, :12], 4), N, 12, H, W)
 

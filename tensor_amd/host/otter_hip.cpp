@@ -1606,7 +1606,12 @@ int Net::forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, 
 }
 
 Extractor Net::create_extractor() const {
-    if (!planned_) plan_fused_quantize();
+    {
+        // extractors may be created from several threads over one const Net: plan once, under a lock
+        static std::mutex plan_mutex;
+        std::lock_guard<std::mutex> lock(plan_mutex);
+        if (!planned_) plan_fused_quantize();
+    }
     return Extractor(this, blobs_.size());
 }
 

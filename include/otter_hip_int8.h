@@ -134,6 +134,16 @@ size_t otter_hip_conv_workspace_bytes(const otter_hip_conv_t* handle, int in_lay
 int otter_hip_conv_forward(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h, int in_w,
                            void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same forward for a layer with an fp32 result (out_kind F32, K % 8 == 0) whose top blob is read by int8
+ * convolutions next: besides `out`, writes what each of those readers would compute first, its quantize_to_int8 of the
+ * blob (Tensor/ConvolutionLayer.cpp:770-775), out_q = float2int8(out * q_scale) as Byte8 [N][K/8][OH*OW][8].
+ * q_scale = the readers' bottom_blob_int8_scales[0], q_round_mode = their input rounding primitive. The implicit-GEMM
+ * kernel writes out_q from its own epilogue (Float4 output, clamp-type activation); every other case runs the
+ * quantize pass after the convolution, with the same result. */
+int otter_hip_conv_forward_twin(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h,
+                                int in_w, void* out, int out_layout, void* out_q, float q_scale, int q_round_mode,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
  * blob). For tests and profiling. */

@@ -322,8 +322,11 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, 
     return pick_kernel(h, l, g, make_epilogue(h, out_layout));
 }
 
-int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
-                           void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream_) {
+// the convolution; `twin` (or null) receives the Byte8 quantization of an fp32 result, from the convolution's own
+// epilogue where that kernel can write it and from a quantize pass after it otherwise
+static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w, void* out,
+                        int out_layout, void* workspace, size_t workspace_bytes, void* stream_, int8_t* twin,
+                        float twin_scale, int twin_round) {
     if (!h || !in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: null");
     if (!valid_layout(in_layout) || !valid_layout(out_layout))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: unknown layout");
@@ -345,10 +348,18 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
     if (n == 0) return OTTER_HIP_OK;
 
+    // the twin as a pass of its own, for the kernels that do not write it
+    auto quantize_twin = [&]() -> int {
+        if (twin)
+            OHIP_CHECK(run_quantize_by((const float*)out, layout_pack(out_layout), twin, 8, n, g.K, g.OH * g.OW, twin_scale,
+                                       twin_round, stream));
+        return OTTER_HIP_OK;
+    };
+
     if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) {
         OHIP_CHECK(run_conv_stem(in, layout_elem(in_layout) == 0, h->w_stem, out, g, make_epilogue(h, out_layout), h->in_scale,
                                  d.in_round_mode, stream));
-        return OTTER_HIP_OK;
+        return quantize_twin();
     }
 
     // (1) quantize_to_int8 when the blob is not int8 yet (Tensor/ConvolutionLayer.cpp:770-775)
@@ -375,10 +386,16 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         xq = (const int8_t*)workspace;
     }
 
-    const Epilogue ep = make_epilogue(h, out_layout);
+    Epilogue ep = make_epilogue(h, out_layout);
+    const int kind = pick_kernel(h, q_layout, g, ep);
+    if (twin && kind == 1 && g.K % 8 == 0 && pick_epilogue(ep, g.K) == EPI_F32_P4) {
+        ep.twin = twin, ep.twin_scale = twin_scale;
+        ep.twin_half = twin_round == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+        twin = nullptr;  // written by the convolution itself
+    }
 
     // (2)+(3)+(4) convolution with the fused epilogue
-    switch (pick_kernel(h, q_layout, g, ep)) {
+    switch (kind) {
     case 3:
         OHIP_CHECK(run_conv3x3_halo(xq, h->w_igemm, out, g, ep, h->force_tm < 0 ? h->force_tn : 0, stream));
         break;
@@ -408,7 +425,25 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
         OHIP_CHECK(run_conv_direct(xq, layout_pack(q_layout), h->w_raw, out, g, ep, stream));
         break;
     }
-    return OTTER_HIP_OK;
+    return quantize_twin();
+}
+
+int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
+                           void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream) {
+    return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, nullptr, 0.f,
+                        0);
+}
+
+int otter_hip_conv_forward_twin(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
+                                void* out, int out_layout, void* out_q, float q_scale, int q_round_mode, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+    if (!h || !out_q) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_twin: null");
+    if (h->d.out_kind != OTTER_HIP_OUT_F32 || h->d.out_channels % 8)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_twin: needs an fp32 output with K % 8 == 0");
+    if (q_round_mode != OTTER_HIP_ROUND_SSE && q_round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_twin: unknown rounding mode");
+    return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, (int8_t*)out_q,
+                        q_scale, q_round_mode);
 }
 
 // -----------------------------------------------------------------------------------------------------

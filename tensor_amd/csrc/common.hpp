@@ -114,6 +114,10 @@ struct Epilogue {
     float round_half;      // 0.5f (ROUND_SSE) or 0.49999997f (ROUND_EXACT)
     bool so_positive;      // every output scale is finite and > 0 (lets the int8 epilogue clamp after rounding)
     bool lrelu;            // LeakyReLU with a slope in [0, 1]: v = max(v, v * act_p0), applied by the fast epilogues
+    // fp32 output only: also write the Byte8 quantization of the result, q = float2int8(v * twin_scale), for an int8
+    // convolution that reads this blob next (null: no twin). Honoured by the implicit-GEMM Float4 epilogue.
+    int8_t* twin = nullptr;
+    float twin_scale = 0.f, twin_half = 0.5f;
 };
 
 // which epilogue code a kernel instance carries
@@ -300,19 +304,27 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
     *reinterpret_cast<ohip_v2i*>(out + elem) = pk;
 }
 
-// dequantize (+clamp activation) 4 channels and store one Float4 element
-__device__ __forceinline__ void epi4_store_f32p4(float* __restrict__ out, const Epilogue& ep, const float* si,
-                                                 const float* bi, size_t elem, int a0, int a1, int a2, int a3) {
+// dequantize (+clamp activation) 4 channels and store one Float4 element; returns the four bytes of the blob's int8
+// twin (float2int8(v * twin_scale)) when the epilogue carries one
+__device__ __forceinline__ unsigned epi4_store_f32p4(float* __restrict__ out, const Epilogue& ep, const float* si,
+                                                     const float* bi, size_t elem, int a0, int a1, int a2, int a3) {
     const int a[4] = {a0, a1, a2, a3};
     ohip_v4i r;
+    unsigned q = 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)a[e], si[e], bi[e]);
         v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
         if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
         r[e] = __float_as_int(v);
+        if (ep.twin != nullptr) {  // wave-uniform
+            const float t = __fmul_rn(v, ep.twin_scale);
+            const int k = (int)__fadd_rn(t, __builtin_copysignf(ep.twin_half, t));
+            q |= (unsigned)(min(max(k, -127), 127) & 0xff) << (8 * e);
+        }
     }
     *reinterpret_cast<ohip_v4i*>(out + elem) = r;
+    return q;
 }
 
 }  // namespace ohip

@@ -39,6 +39,9 @@ hipError_t run_conv_dw(const int8_t* x, const int32_t* wmask, void* out, const C
 // elementwise.hip
 hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,
                         int n_scales, int round_mode, hipStream_t stream);
+// one scale for every channel, passed by value
+hipError_t run_quantize_by(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, float scale, int round_mode,
+                           hipStream_t stream);
 hipError_t run_pad_pack8(const void* src, bool src_is_float, int sp, int8_t* dst, int N, int C, int Cp, int HW,
                          const float* scale, int round_mode, hipStream_t stream);
 hipError_t run_dequantize(const int32_t* src, int sp, float* dst, int dp, int N, int C, int HW, const float* scale,

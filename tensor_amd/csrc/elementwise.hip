@@ -47,14 +47,15 @@ struct Access {
 };
 
 struct QuantOp {
-    const float* scales;
+    const float* scales;  // null: `scale` for every channel
     int n_scales;
     int round_mode;
+    float scale;
     template <int V>
     __device__ __forceinline__ void operator()(const float (&in)[V], int8_t (&out)[V], int c0) const {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-            float s = n_scales == 1 ? scales[0] : scales[c0 + j];
+            float s = scales == nullptr ? scale : (n_scales == 1 ? scales[0] : scales[c0 + j]);
             out[j] = (int8_t)float2int8_rt(__fmul_rn(in[j], s), round_mode);
         }
     }
@@ -203,7 +204,13 @@ hipError_t run_pad_pack8(const void* src, bool src_is_float, int sp, int8_t* dst
 
 hipError_t run_quantize(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, const float* scales,
                         int n_scales, int round_mode, hipStream_t stream) {
-    QuantOp op{scales, n_scales, round_mode};
+    QuantOp op{scales, n_scales, round_mode, 0.f};
+    return dispatch_ew<float, int8_t, QuantOp>(src, sp, dst, dp, N, C, HW, op, stream);
+}
+
+hipError_t run_quantize_by(const float* src, int sp, int8_t* dst, int dp, int N, int C, int HW, float scale, int round_mode,
+                           hipStream_t stream) {
+    QuantOp op{nullptr, 1, round_mode, scale};
     return dispatch_ew<float, int8_t, QuantOp>(src, sp, dst, dp, N, C, HW, op, stream);
 }
 

@@ -621,9 +621,20 @@ int ConvolutionLayer::forward_int8(const Tensor& bottom_in, Tensor& top, const N
         Tensor ws;
         const size_t ws_bytes = otter_hip_conv_workspace_bytes(handle_, in_layout, N, H, W);
         if (ws_bytes) ws = Tensor::empty_device({(int64_t)ws_bytes}, ScalarType::Byte);
-        const int rc = otter_hip_conv_forward(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
-                                              ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
-        if (rc) return rc;
+        int rc;
+        if (fuse_scale > 0.f && out_layout == OTTER_HIP_F32_P4 && out_channels % 8 == 0) {
+            Tensor q = Tensor::empty_device({N, out_channels / 8, oh, ow}, ScalarType::Byte8);
+            rc = otter_hip_conv_forward_twin(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
+                                             q.device_ptr(), fuse_scale, fuse_round, ws_bytes ? ws.device_ptr() : nullptr,
+                                             ws_bytes, nullptr);
+            if (rc) return rc;
+            q.mark_device_written();
+            top.attach_quantized(q, fuse_scale, fuse_round);
+        } else {
+            rc = otter_hip_conv_forward(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
+                                        ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
+            if (rc) return rc;
+        }
         top.mark_device_written();
     } catch (const Error&) {
         return -100;
@@ -1494,15 +1505,18 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
     return 0;
 }
 
-// An Eltwise sum that feeds int8 convolutions is quantized by each of them before anything else happens; when they
-// agree on the scale and the rounding primitive, the Eltwise layer does it on the way (one pass over the blob instead
-// of two, one launch less per reader). Readers behind the automatic Split layers count.
+// An fp32 blob -- an Eltwise sum, or the dequantized result of an int8 convolution that something else reads as fp32
+// too -- that feeds int8 convolutions is quantized by each of them before anything else happens; when they agree on
+// the scale and the rounding primitive, its producer does it on the way (one pass over the blob instead of two, one
+// launch less per reader). Readers behind the automatic Split layers count.
 void Net::plan_fused_quantize() const {
     for (Layer* l : layers_) {
         auto* e = dynamic_cast<EltwiseLayer*>(l);
-        if (!e) continue;
-        e->fuse_scale = 0.f;
-        std::vector<int> pending(e->tops.begin(), e->tops.end());
+        auto* pc = dynamic_cast<ConvolutionLayer*>(l);
+        if (pc && (!pc->int8_scale_term || pc->int8_scale_term > 100)) pc = nullptr;  // fp32 results only
+        if (!e && !pc) continue;
+        (e ? e->fuse_scale : pc->fuse_scale) = 0.f;
+        std::vector<int> pending(l->tops.begin(), l->tops.end());
         float scale = 0.f;
         int round = 0;
         bool agree = true;
@@ -1522,7 +1536,10 @@ void Net::plan_fused_quantize() const {
                 }
             }
         }
-        if (agree && scale > 0.f) e->fuse_scale = scale, e->fuse_round = round;
+        if (agree && scale > 0.f) {
+            if (e) e->fuse_scale = scale, e->fuse_round = round;
+            else pc->fuse_scale = scale, pc->fuse_round = round;
+        }
     }
     // ShuffleNetV2 unit tails: Concat of two equal blobs -> ChannelShuffle(2) -> exactly the two half Crops
     shuffle_units_.clear();

@@ -202,6 +202,10 @@ public:
     Tensor weight_data_int8_scales, bottom_blob_int8_scales, top_blob_int8_scales, scale_in_data;
     // when set, forward() produces fp32 even if int8_scale_term > 100 is absent etc.; -1 = the reference's rule
     int force_out_layout = -1;
+    // > 0: an fp32 top blob is also quantized with this scale, for the int8 convolutions that read it next (set by
+    // Net::plan_fused_quantize)
+    float fuse_scale = 0.f;
+    int fuse_round = 0;
 
     int input_round_mode(const NetOption& opt) const;
 

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from cases import LAYER_CASES
-from gpu_util import ACT, run_conv
+from gpu_util import ACT, host_scale_in, run_conv
 from oracle.binding import ROUND_EXACT, ROUND_SSE
 from tensor_amd import capi
 
@@ -353,6 +353,38 @@ def test_few_channel_3x3_stem_kernel(hip, oracle, C, K, s, p, N, H, W, in_i8, ac
     else:
         assert_f32_close(out, want)
     np.testing.assert_array_equal(out, via_copy)
+
+
+@pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,act,kind", [
+    (96, 24, 1, 1, 0, 1, 3, 14, 13, 0, 1),     # pointwise project, ragged pixel tile: twin from the epilogue
+    (32, 16, 1, 1, 0, 1, 2, 9, 9, 1, 1),
+    (144, 40, 1, 2, 0, 1, 2, 9, 9, 3, 1),      # K % 32 != 0
+    (64, 64, 3, 1, 1, 1, 1, 10, 12, 1, 3),     # halo kernel: quantize pass behind it
+    (16, 16, 3, 1, 1, 16, 2, 9, 9, 0, 2),      # depthwise
+    (24, 24, 1, 1, 0, 1, 1, 5, 5, 4, 1),       # sigmoid: generic epilogue, quantize pass
+])
+@pytest.mark.parametrize("round_mode", [capi.ROUND_SSE, capi.ROUND_EXACT], ids=["sse", "exact"])
+def test_forward_twin_equals_forward_then_quantize(hip, oracle, C, K, k, s, p, g, N, H, W, act, kind, round_mode):
+    """otter_hip_conv_forward_twin: the fp32 blob is bit-identical to otter_hip_conv_forward's, and the Byte8 twin
+    is bit-identical to the oracle's quantize_to_int8 of that blob, whichever kernel produced it."""
+    rng = np.random.default_rng(C + K * 5 + k + act)
+    x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W)
+    in_scale = 20.0
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=in_scale, out_scale=None,
+                    stride=(s, s), pad=(p, p), dil=(1, 1), groups=g, act=act, act_p0=0.0, out_kind=capi.OUT_F32,
+                    out_round=0, in_round=oracle.quantize_round_mode(C, True))
+    xd = hip.to_device(capi.pack_np(x, 8))
+    assert conv.kernel_kind(capi.I8_P8, N, H, W, capi.F32_P4) == kind
+    plain = conv.forward(xd, capi.I8_P8, N, H, W, capi.F32_P4).cpu().numpy()
+    q_scale = 127.0 / max(float(np.abs(plain).max()), 1e-6) * 1.3   # some values saturate
+    out, q = conv.forward_twin(xd, capi.I8_P8, N, H, W, q_scale, round_mode, capi.F32_P4)
+    hip.torch.cuda.synchronize()
+    oh, ow = conv.out_hw(H, W)
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint32), plain.view(np.uint32))
+    y = capi.unpack_np(plain, 4, (N, K, oh, ow))
+    want = oracle.quantize(y, np.float32(q_scale), round_mode)
+    np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), 8, (N, K, oh, ow)), want)
+    conv.close()
 
 
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):

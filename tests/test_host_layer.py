@@ -131,6 +131,44 @@ def test_sum_feeding_int8_convolutions_is_quantized_on_the_way(oracle, same_scal
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("k", [1, 3], ids=["pointwise_producer", "3x3_producer"])
+@pytest.mark.parametrize("same_scale", [True, False], ids=["readers_agree", "readers_disagree"])
+def test_fp32_convolution_feeding_int8_convolutions_is_quantized_on_the_way(oracle, same_scale, k):
+    """The MobileNetV2 pattern at the head of a residual chain: a project convolution whose fp32 result is read by the
+    shortcut sum and by the next expand convolutions. The producer writes the readers' quantization itself when they
+    agree on the scale; every blob equals the oracle's layer-by-layer computation either way."""
+    rng = np.random.default_rng(23 + k)
+    C, K = 24, 32
+    x = rng.uniform(-1, 1, (3, C, 9, 11)).astype(np.float32)
+    wp, sp = _qweights(rng, C, C, k)
+    wa, sa = _qweights(rng, K, C, 1)
+    wb, sb = _qweights(rng, C, C, 1)
+    bp, ba, bb = (rng.normal(0, 0.1, n).astype(np.float32) for n in (C, K, C))
+    in_p = np.float32(127) / np.abs(x).max()
+    net = hostnet.Net(lightmode=False)
+    net.add_layer(type="Input", name="data", batchsize=3, channel=C, height=9, width=11)
+    net.add_layer(type="Convolution", name="p", input="data", out_channels=C, kernel=k, padding=k // 2,
+                  int8_scale_term=2)
+    net.add_layer(type="Convolution", name="a", input="p", out_channels=K, kernel=1, int8_scale_term=102,
+                  activation="Relu6")
+    net.add_layer(type="Convolution", name="b", input="p", out_channels=C, kernel=1, int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="sum", input="p,b")
+    net.compile()
+    yp = oracle.conv_layer_forward(x, wp, sp, in_p, pad=(k // 2, k // 2), bias=bp)
+    in_a = np.float32(127) / np.abs(yp).max() * np.float32(1.2)
+    in_b = in_a if same_scale else np.float32(in_a * 0.75)
+    net.set_conv("p", wp, bp, sp, in_p)
+    net.set_conv("a", wa, ba, sa, in_a, 9.0)
+    net.set_conv("b", wb, bb, sb, in_b)
+    ya = oracle.conv_layer_forward(yp, wa, sa, in_a, bias=ba, top_scale=9.0, int8_out=True, act_type=3)
+    yb = oracle.conv_layer_forward(yp, wb, sb, in_b, bias=bb)
+    np.testing.assert_allclose(net.run("data", x, "p"), yp, rtol=1e-5, atol=1e-30)
+    np.testing.assert_array_equal(net.run("data", x, "a"), ya)
+    np.testing.assert_allclose(net.run("data", x, "b"), yb, rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(net.run("data", x, "sum"), yp + yb, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.gpu
 def test_functional_api_matches_oracle(oracle):
     rng = np.random.default_rng(8)
     for (C, K, k, s, p, g, i8) in [(16, 16, 3, 1, 1, 1, True), (32, 32, 3, 2, 1, 32, True), (8, 12, 1, 1, 0, 1, False)]:

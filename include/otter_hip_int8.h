@@ -96,8 +96,13 @@ typedef struct {
     int pad_h, pad_w;
     int dilation_h, dilation_w;
     int groups;
-    int activation_type;     /* 0 none, 1 ReLU, 2 LeakyReLU, 3 clip [0,6], 4 sigmoid
-                                (Tensor/ConvolutionLayer.cpp:113-122, Tensor/QuantizeX86.hpp:72-106) */
+    int activation_type;     /* 0 none, 1 ReLU, 2 LeakyReLU, 3 clip [0,6], 4 sigmoid, 5 mish
+                                (Tensor/ConvolutionLayer.cpp:113-122, Tensor/QuantizeX86.hpp:72-106; the layer's
+                                option strings select 1-4, mish exists in the requantize function only). 4 and 5
+                                are evaluated with the device's exp / log / tanh: the reference's values come
+                                from polynomial approximations and an approximate-reciprocal instruction, so an
+                                int8 result may differ from it by one step where the scaled value is at a
+                                rounding tie. */
     float activation_param0; /* LeakyReLU slope */
     int out_kind;            /* otter_hip_out_kind */
     int out_round_mode;      /* otter_hip_round_mode used when out_kind is I8 */

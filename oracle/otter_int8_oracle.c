@@ -10,8 +10,12 @@
  *          where that library exists, and with golden vectors it produced (tests/golden/) everywhere else,
  *          including adversarial near-tie values; _conv_int32 additionally against an independent numpy
  *          int64 einsum (exact integer arithmetic, order independent).
- *   otter_oracle_activation types 4 (sigmoid) and 5 (mish): PARITY UNPINNED -- the reference evaluates them
- *          with -ffast-math polynomial approximations (Tensor/QuantizeX86.hpp:38-58); libm is used here.
+ *   otter_oracle_activation types 4 (sigmoid) and 5 (mish): the reference evaluates them with polynomial
+ *          exp / log (Tensor/QuantizeX86.hpp:38-58) and, built with -Ofast, an approximate-reciprocal instruction
+ *          plus one Newton step for the division, so its own value depends on the CPU model; libm is used here.
+ *          Pinned to that bound: against vectors written by the compiled reference
+ *          (tests/test_activation_golden.py), int8 results equal but for at most one step at rounding ties
+ *          (fewer than 0.2 % of the values), fp32 results within a relative 1e-5.
  *   x86 overflow artefact: for |v| >= 2^31 (or NaN) cvttps2dq returns INT_MIN, so the reference yields -127
  *          for a huge *positive* value. Restated here for completeness; callers keep to |v| < 2^31.
  *

@@ -164,7 +164,7 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: channels not divisible by groups");
     if (d.out_kind < OTTER_HIP_OUT_I32 || d.out_kind > OTTER_HIP_OUT_I8)
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: bad out_kind");
-    if (d.activation_type < 0 || d.activation_type > 4)
+    if (d.activation_type < 0 || d.activation_type > 5)
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_create: activation type not supported");
     if (d.out_kind == OTTER_HIP_OUT_I8 && (!out_scale || (n_out_scale != 1 && n_out_scale != d.out_channels)))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_create: int8 output needs 1 or K output scales");
@@ -496,7 +496,7 @@ int otter_hip_requantize(const int32_t* src, int src_layout, int n, int c, int h
     if (!bias) n_bias = 0;
     if (n_bias != 0 && n_bias != 1 && n_bias != c)
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_requantize: need 0, 1 or C biases");
-    if (activation_type < 0 || activation_type > 4)
+    if (activation_type < 0 || activation_type > 5)
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_requantize: activation type not supported");
     OHIP_CHECK(run_requantize(src, layout_pack(src_layout), dst, layout_pack(dst_layout), n, c, h * w, scale_in,
                               n_scale_in, scale_out, n_scale_out, bias, n_bias, activation_type, activation_param0,
@@ -539,7 +539,7 @@ int otter_hip_eltwise_add_quantize(const float* a, const float* b, int layout, i
 
 int otter_hip_activation(float* x, size_t count, int activation_type, float activation_param0, void* stream) {
     if (!x) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_activation: null");
-    if (activation_type < 0 || activation_type > 4)
+    if (activation_type < 0 || activation_type > 5)
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_activation: activation type not supported");
     OHIP_CHECK(run_activation(x, count, activation_type, activation_param0, (hipStream_t)stream));
     return OTTER_HIP_OK;

@@ -74,6 +74,8 @@ __device__ __forceinline__ float activate(float v, int act, float p0) {
         return fminf(fmaxf(v, 0.f), 6.f);
     case 4:
         return 1.f / (1.f + __expf(-v));
+    case 5:  // mish: reachable through the standalone requantize only (no option string of the layer selects it)
+        return __fmul_rn(v, tanhf(logf(__expf(v) + 1.f)));
     default:
         return v;
     }

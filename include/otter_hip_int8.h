@@ -149,6 +149,18 @@ int otter_hip_conv_forward_twin(const otter_hip_conv_t* handle, const void* in, 
                                 int in_w, void* out, int out_layout, void* out_q, float q_scale, int q_round_mode,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* The tail of a residual block in one call: an int8 convolution with an fp32 result followed by the Eltwise sum with
+ * the block's shortcut (Tensor/ConvolutionLayer.cpp:754-847, then Tensor/EltwiseLayer.cpp:48-80), out =
+ * activation(convolution) + residual, both in out_layout, same shape. With out_q (or null; needs K % 8 == 0) also the
+ * quantize_to_int8 of the sum for the int8 convolutions that read it, as in otter_hip_conv_forward_twin. The
+ * convolution's own result is not stored anywhere: use this only when the Eltwise layer is its sole reader. The
+ * implicit-GEMM kernel adds (and quantizes) in its epilogue (Float4 output, clamp-type activation); every other case
+ * runs the separate passes behind the convolution, with the same result. */
+int otter_hip_conv_forward_residual(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h,
+                                    int in_w, const float* residual, void* out, int out_layout, void* out_q,
+                                    float q_scale, int q_round_mode, void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
  * blob). For tests and profiling. */

@@ -69,7 +69,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_set_tile", "otter_hip_eltwise_add", "otter_hip_activation", "otter_hip_global_avgpool",
            "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
-           "otter_hip_conv_forward_twin"]
+           "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual"]
 
 
 def load_cdll():
@@ -265,6 +265,21 @@ class Conv:
             self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout, self.L.ptr(q), C.c_float(q_scale),
             q_round_mode, self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes),
             self.L.stream()))
+        return out, q
+
+    def forward_residual(self, x, in_layout, n, h, w, residual, q_scale=None, q_round_mode=ROUND_SSE, out_layout=None):
+        """activation(convolution) + residual, and with q_scale the Byte8 quantization of that sum
+        (otter_hip_conv_forward_residual). Returns (sum, q or None)."""
+        out_layout = self.default_out_layout() if out_layout is None else out_layout
+        oh, ow = self.out_hw(h, w)
+        out = self.L.empty(n * self.K * oh * ow, layout_dtype(out_layout))
+        q = self.L.empty(n * self.K * oh * ow, np.int8) if q_scale is not None else None
+        ws_bytes = self.L.lib.otter_hip_conv_workspace_bytes(self.h, in_layout, n, h, w)
+        workspace = self.L.empty(ws_bytes, np.int8) if ws_bytes else None
+        self.L._check(self.L.lib.otter_hip_conv_forward_residual(
+            self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(residual), self.L.ptr(out), out_layout,
+            self.L.ptr(q) if q is not None else None, C.c_float(q_scale or 0.0), q_round_mode,
+            self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))
         return out, q
 
     def close(self):

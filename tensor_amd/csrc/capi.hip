@@ -324,9 +324,10 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, 
 
 // the convolution; `twin` (or null) receives the Byte8 quantization of an fp32 result, from the convolution's own
 // epilogue where that kernel can write it and from a quantize pass after it otherwise
+// `residual` (or null): a blob in the output's layout added to the fp32 result; the twin is then made of the sum
 static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w, void* out,
                         int out_layout, void* workspace, size_t workspace_bytes, void* stream_, int8_t* twin,
-                        float twin_scale, int twin_round) {
+                        float twin_scale, int twin_round, const float* residual = nullptr) {
     if (!h || !in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: null");
     if (!valid_layout(in_layout) || !valid_layout(out_layout))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward: unknown layout");
@@ -348,11 +349,18 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
         return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_forward: tensor exceeds 2^31 elements; split the batch");
     if (n == 0) return OTTER_HIP_OK;
 
-    // the twin as a pass of its own, for the kernels that do not write it
+    // the sum and the twin as a pass of their own, for the kernels that do not write them
     auto quantize_twin = [&]() -> int {
-        if (twin)
-            OHIP_CHECK(run_quantize_by((const float*)out, layout_pack(out_layout), twin, 8, n, g.K, g.OH * g.OW, twin_scale,
-                                       twin_round, stream));
+        float* o = (float*)out;
+        if (residual && twin && layout_pack(out_layout) != 1)
+            OHIP_CHECK(run_eltwise_add_quantize(o, residual, layout_pack(out_layout), o, twin, n, g.K, g.OH * g.OW, twin_scale,
+                                                twin_round, stream));
+        else {
+            if (residual) OHIP_CHECK(run_eltwise_add(o, residual, o, (size_t)n * g.K * g.OH * g.OW, stream));
+            if (twin)
+                OHIP_CHECK(run_quantize_by(o, layout_pack(out_layout), twin, 8, n, g.K, g.OH * g.OW, twin_scale, twin_round,
+                                           stream));
+        }
         return OTTER_HIP_OK;
     };
 
@@ -388,10 +396,11 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
 
     Epilogue ep = make_epilogue(h, out_layout);
     const int kind = pick_kernel(h, q_layout, g, ep);
-    if (twin && kind == 1 && g.K % 8 == 0 && pick_epilogue(ep, g.K) == EPI_F32_P4) {
+    if ((twin || residual) && kind == 1 && (!twin || g.K % 8 == 0) && pick_epilogue(ep, g.K) == EPI_F32_P4) {
         ep.twin = twin, ep.twin_scale = twin_scale;
         ep.twin_half = twin_round == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
-        twin = nullptr;  // written by the convolution itself
+        ep.residual = residual;
+        twin = nullptr, residual = nullptr;  // done by the convolution itself
     }
 
     // (2)+(3)+(4) convolution with the fused epilogue
@@ -432,6 +441,21 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
                            void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream) {
     return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, nullptr, 0.f,
                         0);
+}
+
+int otter_hip_conv_forward_residual(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
+                                    const float* residual, void* out, int out_layout, void* out_q, float q_scale,
+                                    int q_round_mode, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!h || !residual) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_residual: null");
+    if (h->d.out_kind != OTTER_HIP_OUT_F32)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_residual: needs an fp32 output");
+    if (out_q && h->d.out_channels % 8)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_residual: the quantized sum needs K % 8 == 0");
+    if (out_q && q_round_mode != OTTER_HIP_ROUND_SSE && q_round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_residual: unknown rounding mode");
+    if (residual == out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_residual: out must not be the residual");
+    return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, (int8_t*)out_q,
+                        q_scale, q_round_mode, residual);
 }
 
 int otter_hip_conv_forward_twin(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,

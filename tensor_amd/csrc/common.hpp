@@ -120,6 +120,9 @@ struct Epilogue {
     // convolution that reads this blob next (null: no twin). Honoured by the implicit-GEMM Float4 epilogue.
     int8_t* twin = nullptr;
     float twin_scale = 0.f, twin_half = 0.5f;
+    // fp32 output only: a blob in the output's layout that is added to the activated result (the Eltwise sum of a
+    // residual block; null: none). The twin, if any, is the quantization of the sum. Float4 epilogue only.
+    const float* residual = nullptr;
 };
 
 // which epilogue code a kernel instance carries
@@ -313,11 +316,14 @@ __device__ __forceinline__ unsigned epi4_store_f32p4(float* __restrict__ out, co
     const int a[4] = {a0, a1, a2, a3};
     ohip_v4i r;
     unsigned q = 0;
+    ohip_v4i res = {0, 0, 0, 0};
+    if (ep.residual != nullptr) res = *reinterpret_cast<const ohip_v4i*>(ep.residual + elem);  // wave-uniform
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)a[e], si[e], bi[e]);
         v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
         if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
+        if (ep.residual != nullptr) v = __fadd_rn(v, __int_as_float(res[e]));
         r[e] = __float_as_int(v);
         if (ep.twin != nullptr) {  // wave-uniform
             const float t = __fmul_rn(v, ep.twin_scale);

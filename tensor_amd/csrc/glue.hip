@@ -6,9 +6,10 @@
 
 namespace ohip {
 
-// out = a + b (Tensor/EltwiseLayer.cpp:48-80, operation sum); layouts must match, so it is a flat add
-__global__ void __launch_bounds__(256) eltwise_add_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                          float* __restrict__ out, size_t n4, size_t n) {
+// out = a + b (Tensor/EltwiseLayer.cpp:48-80, operation sum); layouts must match, so it is a flat add.
+// `out` may be `a` (every element is read and written by one thread): no __restrict__ on the two.
+__global__ void __launch_bounds__(256) eltwise_add_kernel(const float* a, const float* __restrict__ b, float* out, size_t n4,
+                                                          size_t n) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n4) {
         const float4 x = reinterpret_cast<const float4*>(a)[i], y = reinterpret_cast<const float4*>(b)[i];
@@ -117,10 +118,11 @@ hipError_t run_eltwise_add(const float* a, const float* b, float* out, size_t n,
 // out = a + b and, in the same pass, the int8 blob a following int8 convolution would make of it
 // (ConvolutionLayer::forward_int8 quantizes an fp32 bottom blob first, Tensor/ConvolutionLayer.cpp:770-775):
 // q = float2int8(out * scale) into Byte8. One thread per (image, channel octet, pixel); P = elempack of a, b and out.
+// `out` may be `a`.
 template <int P>
-__global__ void __launch_bounds__(256) eltwise_add_quantize_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                                   float* __restrict__ out, int8_t* __restrict__ q, int C8,
-                                                                   int HW, float scale, float half, unsigned total) {
+__global__ void __launch_bounds__(256) eltwise_add_quantize_kernel(const float* a, const float* __restrict__ b, float* out,
+                                                                   int8_t* __restrict__ q, int C8, int HW, float scale,
+                                                                   float half, unsigned total) {
     const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const unsigned r = i / (unsigned)HW;

@@ -593,12 +593,19 @@ int ConvolutionLayer::create_pipeline_int8(const NetOption& opt) {
 }
 
 int ConvolutionLayer::forward(const Tensor& bottom, Tensor& top, const NetOption& opt) const {
-    if (int8_scale_term) return forward_int8(bottom, top, opt);
+    if (int8_scale_term) return forward_int8(bottom, nullptr, fuse_scale, fuse_round, top, opt);
     return -1;
 }
 
-// Tensor/ConvolutionLayer.cpp:754-847, whole batch in one launch
-int ConvolutionLayer::forward_int8(const Tensor& bottom_in, Tensor& top, const NetOption& opt) const {
+int ConvolutionLayer::forward_residual(const Tensor& bottom, const Tensor& shortcut, float q_scale, int q_round, Tensor& sum,
+                                       const NetOption& opt) const {
+    if (!int8_scale_term || int8_scale_term > 100 || !shortcut.defined()) return 1;
+    return forward_int8(bottom, &shortcut, q_scale, q_round, sum, opt);
+}
+
+// Tensor/ConvolutionLayer.cpp:754-847, whole batch in one launch; with `shortcut` the Eltwise sum behind it as well
+int ConvolutionLayer::forward_int8(const Tensor& bottom_in, const Tensor* shortcut, float q_scale, int q_round, Tensor& top,
+                                   const NetOption& opt) const {
     if (!handle_ || !bottom_in.defined() || bottom_in.dim() != 4) return -1;
     // the producer may already have quantized this blob with this layer's scale (see Net::plan_fused_quantize)
     Tensor bottom = bottom_in, twin;
@@ -616,20 +623,38 @@ int ConvolutionLayer::forward_int8(const Tensor& bottom_in, Tensor& top, const N
         out_layout = int8_scale_term > 100 ? OTTER_HIP_I8 : OTTER_HIP_F32;
     if (force_out_layout >= 0) out_layout = force_out_layout;
     const ScalarType odt = scalar_type_of_layout(out_layout);
+    if (shortcut) {  // the sum is taken in the layout this layer writes: the shortcut must already have it
+        if (shortcut->scalar_type() != odt || elempack_of(odt) != 4 || shortcut->dim() != 4 || shortcut->size(0) != N ||
+            shortcut->channels() != out_channels || shortcut->size(2) != oh || shortcut->size(3) != ow)
+            return 1;
+    }
     try {
         top = Tensor::empty_device({N, out_channels / elempack_of(odt), oh, ow}, odt);
         Tensor ws;
         const size_t ws_bytes = otter_hip_conv_workspace_bytes(handle_, in_layout, N, H, W);
         if (ws_bytes) ws = Tensor::empty_device({(int64_t)ws_bytes}, ScalarType::Byte);
         int rc;
-        if (fuse_scale > 0.f && out_layout == OTTER_HIP_F32_P4 && out_channels % 8 == 0) {
+        const bool with_q = q_scale > 0.f && out_layout == OTTER_HIP_F32_P4 && out_channels % 8 == 0;
+        if (shortcut) {
+            Tensor q;
+            if (with_q) q = Tensor::empty_device({N, out_channels / 8, oh, ow}, ScalarType::Byte8);
+            rc = otter_hip_conv_forward_residual(handle_, bottom.device_ptr(), in_layout, N, H, W,
+                                                 (const float*)shortcut->device_ptr(), top.device_ptr(), out_layout,
+                                                 with_q ? q.device_ptr() : nullptr, q_scale, q_round,
+                                                 ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
+            if (rc) return rc;
+            if (with_q) {
+                q.mark_device_written();
+                top.attach_quantized(q, q_scale, q_round);
+            }
+        } else if (with_q) {
             Tensor q = Tensor::empty_device({N, out_channels / 8, oh, ow}, ScalarType::Byte8);
             rc = otter_hip_conv_forward_twin(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
-                                             q.device_ptr(), fuse_scale, fuse_round, ws_bytes ? ws.device_ptr() : nullptr,
+                                             q.device_ptr(), q_scale, q_round, ws_bytes ? ws.device_ptr() : nullptr,
                                              ws_bytes, nullptr);
             if (rc) return rc;
             q.mark_device_written();
-            top.attach_quantized(q, fuse_scale, fuse_round);
+            top.attach_quantized(q, q_scale, q_round);
         } else {
             rc = otter_hip_conv_forward(handle_, bottom.device_ptr(), in_layout, N, H, W, top.device_ptr(), out_layout,
                                         ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
@@ -1473,6 +1498,14 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
             }
         }
     }
+    {
+        const auto unit = residual_units_.find(li);
+        // only when the convolution's own result has not been computed (or set by the caller)
+        if (unit != residual_units_.end() && !blobs[layers_[unit->second.conv]->tops[0]].defined()) {
+            const int rc = forward_residual_unit(unit->second, blobs, opt);
+            if (rc <= 0) return rc;
+        }
+    }
     for (int b : layer->bottoms)
         if (!blobs[b].defined()) {
             int rc = forward_layer(blobs_[b].producer, blobs, opt);
@@ -1541,6 +1574,22 @@ void Net::plan_fused_quantize() const {
             else pc->fuse_scale = scale, pc->fuse_round = round;
         }
     }
+    // Residual block tails: Eltwise sum of two blobs, one the fp32 result of an int8 convolution read by nothing else
+    residual_units_.clear();
+    for (size_t ei = 0; ei < layers_.size(); ++ei) {
+        const auto* e = dynamic_cast<const EltwiseLayer*>(layers_[ei]);
+        if (!e || e->bottoms.size() != 2) continue;
+        int best = -1;
+        for (int k = 0; k < 2; ++k) {
+            const int b = e->bottoms[k], pi = blobs_[b].producer;
+            const auto* pc = pi < 0 ? nullptr : dynamic_cast<const ConvolutionLayer*>(layers_[pi]);
+            if (!pc || !pc->int8_scale_term || pc->int8_scale_term > 100 || pc->force_out_layout >= 0) continue;
+            if (blobs_[b].consumers.size() != 1 || pc->out_channels % 4) continue;
+            if (e->bottoms[0] == e->bottoms[1]) continue;
+            if (best < 0 || pi > blobs_[e->bottoms[best]].producer) best = k;  // the later one: the other is ready by then
+        }
+        if (best >= 0) residual_units_[(int)ei] = ResidualUnit{blobs_[e->bottoms[best]].producer, (int)ei, e->bottoms[1 - best]};
+    }
     // ShuffleNetV2 unit tails: Concat of two equal blobs -> ChannelShuffle(2) -> exactly the two half Crops
     shuffle_units_.clear();
     auto sole_reader = [&](int blob) { return blobs_[blob].consumers.size() == 1 ? blobs_[blob].consumers[0] : -1; };
@@ -1583,6 +1632,26 @@ void Net::plan_fused_quantize() const {
         shuffle_units_[hi] = u;
     }
     planned_ = true;
+}
+
+// Convolution and Eltwise sum in one launch (otter_hip_conv_forward_residual). Returns 1 when the blobs at hand do not
+// allow it; the caller then runs the layers one by one.
+int Net::forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const {
+    const auto* conv = static_cast<const ConvolutionLayer*>(layers_[u.conv]);
+    const auto* e = static_cast<const EltwiseLayer*>(layers_[u.eltwise]);
+    for (int b : {u.shortcut, conv->bottoms[0]})
+        if (!blobs[b].defined()) {
+            const int rc = forward_layer(blobs_[b].producer, blobs, opt);
+            if (rc) return rc;
+        }
+    Tensor sum;
+    const int rc = conv->forward_residual(blobs[conv->bottoms[0]], blobs[u.shortcut], e->fuse_scale, e->fuse_round, sum, opt);
+    if (rc) return rc;
+    blobs[e->tops[0]] = sum;
+    if (opt.lightmode)
+        for (int b : {u.shortcut, conv->bottoms[0]})
+            if (blobs_[b].consumers.size() == 1) blobs[b] = Tensor();
+    return 0;
 }
 
 // One kernel for a whole unit (otter_hip_shuffle2_split) when the blobs between its ends are not wanted by anybody else.

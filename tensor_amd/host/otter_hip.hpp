@@ -208,10 +208,17 @@ public:
     int fuse_round = 0;
 
     int input_round_mode(const NetOption& opt) const;
+    // This layer followed by the Eltwise sum with `shortcut` in one launch (otter_hip_conv_forward_residual), for a layer
+    // with an fp32 result whose only reader is that sum: sum = activation(convolution) + shortcut, quantized on the way
+    // with q_scale (> 0) for the int8 convolutions that read the sum. Returns 1, and does nothing, when the blobs do not
+    // have the layouts that takes (the caller then runs the two layers one after the other).
+    int forward_residual(const Tensor& bottom_blob, const Tensor& shortcut, float q_scale, int q_round, Tensor& sum,
+                         const NetOption& opt) const;
 
 private:
     int create_pipeline_int8(const NetOption& opt);
-    int forward_int8(const Tensor& bottom_blob, Tensor& top_blob, const NetOption& opt) const;
+    int forward_int8(const Tensor& bottom_blob, const Tensor* shortcut, float q_scale, int q_round, Tensor& top_blob,
+                     const NetOption& opt) const;
     otter_hip_conv* handle_ = nullptr;
 };
 
@@ -295,6 +302,15 @@ private:
     };
     mutable std::map<int, ShuffleUnit> shuffle_units_;
     int forward_shuffle_unit(const ShuffleUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
+    // The tail of a residual block, found by the plan: an Eltwise sum of two blobs, one of them the fp32 result of an
+    // int8 convolution that nothing else reads. Eltwise layer's index -> the unit; forward_layer runs convolution and
+    // sum in one launch when the convolution's result does not exist yet.
+    struct ResidualUnit {
+        int conv, eltwise;
+        int shortcut;  // blob index of the other operand
+    };
+    mutable std::map<int, ResidualUnit> residual_units_;
+    int forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
 };
 
 class Extractor {

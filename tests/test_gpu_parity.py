@@ -387,6 +387,43 @@ def test_forward_twin_equals_forward_then_quantize(hip, oracle, C, K, k, s, p, g
     conv.close()
 
 
+@pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,act,kind", [
+    (96, 24, 1, 1, 0, 1, 3, 14, 13, 0, 1),     # pointwise project of a residual block: sum from the epilogue
+    (192, 32, 1, 1, 0, 1, 2, 9, 9, 1, 1),
+    (144, 20, 1, 1, 0, 1, 2, 7, 7, 0, 1),      # K % 8 != 0: the sum alone
+    (64, 64, 3, 1, 1, 1, 1, 10, 12, 1, 3),     # halo kernel: add (+ quantize) pass behind it
+    (16, 16, 3, 1, 1, 16, 2, 9, 9, 0, 2),      # depthwise
+    (24, 24, 1, 1, 0, 1, 1, 5, 5, 4, 1),       # sigmoid: generic epilogue
+])
+@pytest.mark.parametrize("with_q", [True, False], ids=["sum_and_twin", "sum_only"])
+def test_forward_residual_equals_forward_then_add(hip, oracle, C, K, k, s, p, g, N, H, W, act, kind, with_q):
+    """otter_hip_conv_forward_residual: the sum is bit-identical to otter_hip_conv_forward's blob plus the shortcut (one
+    fp32 addition per element), and the twin to the oracle's quantize_to_int8 of that sum."""
+    rng = np.random.default_rng(C * 3 + K + k + act)
+    x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W)
+    in_scale = 20.0
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=in_scale, out_scale=None,
+                    stride=(s, s), pad=(p, p), dil=(1, 1), groups=g, act=act, act_p0=0.0, out_kind=capi.OUT_F32,
+                    out_round=0, in_round=oracle.quantize_round_mode(C, True))
+    xd = hip.to_device(capi.pack_np(x, 8))
+    assert conv.kernel_kind(capi.I8_P8, N, H, W, capi.F32_P4) == kind
+    oh, ow = conv.out_hw(H, W)
+    plain = capi.unpack_np(conv.forward(xd, capi.I8_P8, N, H, W, capi.F32_P4).cpu().numpy(), 4, (N, K, oh, ow))
+    short = (rng.normal(0, 1, plain.shape) * np.abs(plain).mean()).astype(np.float32)
+    want = plain + short
+    with_q = with_q and K % 8 == 0
+    q_scale = 127.0 / float(np.abs(want).max()) * 1.3 if with_q else None   # some values saturate
+    out, q = conv.forward_residual(xd, capi.I8_P8, N, H, W, hip.to_device(capi.pack_np(short, 4)), q_scale,
+                                   capi.ROUND_SSE, capi.F32_P4)
+    hip.torch.cuda.synchronize()
+    got = capi.unpack_np(out.cpu().numpy(), 4, (N, K, oh, ow))
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    if with_q:
+        np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), 8, (N, K, oh, ow)),
+                                      oracle.quantize(want, np.float32(q_scale), capi.ROUND_SSE))
+    conv.close()
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

@@ -169,6 +169,55 @@ def test_fp32_convolution_feeding_int8_convolutions_is_quantized_on_the_way(orac
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("k", [1, 3], ids=["pointwise_project", "3x3_project"])
+@pytest.mark.parametrize("ask_inner_first", [False, True], ids=["fused", "inner_blob_requested"])
+def test_residual_block_tail_runs_as_one_launch_with_the_same_blobs(oracle, k, ask_inner_first):
+    """A residual block: the project convolution's fp32 result is read by the Eltwise sum alone, and the sum by an
+    int8 convolution and a second sum. Convolution + sum (+ the reader's quantization) run as one launch; asking for
+    the convolution's own blob first makes the layers run one by one. Same blobs either way."""
+    rng = np.random.default_rng(31 + k)
+    C, K = 24, 16
+    x = rng.uniform(-1, 1, (3, C, 9, 11)).astype(np.float32)
+    wp, sp = _qweights(rng, C, C, k)
+    wa, sa = _qweights(rng, K, C, 1)
+    wb, sb = _qweights(rng, C, C, 1)
+    bp, ba, bb = (rng.normal(0, 0.1, n).astype(np.float32) for n in (C, K, C))
+    in_p = np.float32(127) / np.abs(x).max()
+    net = hostnet.Net(lightmode=False)
+    net.add_layer(type="Input", name="data", batchsize=3, channel=C, height=9, width=11)
+    net.add_layer(type="Convolution", name="p", input="data", out_channels=C, kernel=k, padding=k // 2,
+                  int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="sum", input="data,p")
+    net.add_layer(type="Convolution", name="a", input="sum", out_channels=K, kernel=1, int8_scale_term=102,
+                  activation="Relu")
+    net.add_layer(type="Convolution", name="b", input="sum", out_channels=C, kernel=1, int8_scale_term=2)
+    net.add_layer(type="Eltwise", name="sum2", input="b,sum")
+    net.compile()
+    yp = oracle.conv_layer_forward(x, wp, sp, in_p, pad=(k // 2, k // 2), bias=bp)
+    s1 = x + yp
+    in_a = np.float32(127) / np.abs(s1).max()
+    net.set_conv("p", wp, bp, sp, in_p)
+    net.set_conv("a", wa, ba, sa, in_a, 9.0)
+    net.set_conv("b", wb, bb, sb, in_a)
+    ya = oracle.conv_layer_forward(s1, wa, sa, in_a, bias=ba, top_scale=9.0, int8_out=True, act_type=1)
+    yb = oracle.conv_layer_forward(s1, wb, sb, in_a, bias=bb)
+
+    def last_of(names, shape, dtype):
+        """one extractor, the blobs extracted in this order; the last one comes back"""
+        s = net.session("data", x, ",".join(names))
+        s.run()
+        out = s.fetch(shape, dtype)
+        s.close()
+        return out
+
+    first = ["p"] if ask_inner_first else []
+    np.testing.assert_allclose(last_of(first + ["sum"], s1.shape, np.float32), s1, rtol=1e-5, atol=1e-30)
+    np.testing.assert_array_equal(last_of(first + ["a"], ya.shape, np.int8), ya)
+    np.testing.assert_allclose(last_of(first + ["sum2"], s1.shape, np.float32), yb + s1, rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(last_of(first + ["sum", "p"], yp.shape, np.float32), yp, rtol=1e-5, atol=1e-30)
+
+
+@pytest.mark.gpu
 def test_functional_api_matches_oracle(oracle):
     rng = np.random.default_rng(8)
     for (C, K, k, s, p, g, i8) in [(16, 16, 3, 1, 1, 1, True), (32, 32, 3, 2, 1, 32, True), (8, 12, 1, 1, 0, 1, False)]:

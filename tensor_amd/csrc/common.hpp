@@ -126,7 +126,14 @@ struct Epilogue {
 };
 
 // which epilogue code a kernel instance carries
-enum { EPI_GENERIC = 0, EPI_I8_P8 = 1, EPI_F32_P4 = 2, EPI_I8_P8_NONNEG = 3, EPI_F32_P8 = 4 /* depthwise only */ };
+enum {
+    EPI_GENERIC = 0,
+    EPI_I8_P8 = 1,
+    EPI_F32_P4 = 2,
+    EPI_I8_P8_NONNEG = 3,
+    EPI_F32_P8 = 4,       // depthwise only
+    EPI_F32_P4_FUSED = 5  // implicit GEMM only: EPI_F32_P4 plus the residual addend and / or the int8 twin
+};
 
 // The fast epilogues need: activation in {none, ReLU, clip, LeakyReLU with a slope in [0, 1]}, and (I8_P8) int8
 // output in Byte8 with K % 8 == 0 or (F32_P4) fp32 output in Float4 with K % 4 == 0.
@@ -309,27 +316,32 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
     *reinterpret_cast<ohip_v2i*>(out + elem) = pk;
 }
 
-// dequantize (+clamp activation) 4 channels and store one Float4 element; returns the four bytes of the blob's int8
-// twin (float2int8(v * twin_scale)) when the epilogue carries one
+// dequantize (+clamp activation) 4 channels and store one Float4 element. FUSED: first add the residual blob's element
+// if the epilogue carries one, and return the four bytes of the blob's int8 twin (float2int8(v * twin_scale)) if it
+// carries one
+template <bool FUSED = false>
 __device__ __forceinline__ unsigned epi4_store_f32p4(float* __restrict__ out, const Epilogue& ep, const float* si,
                                                      const float* bi, size_t elem, int a0, int a1, int a2, int a3) {
     const int a[4] = {a0, a1, a2, a3};
     ohip_v4i r;
     unsigned q = 0;
     ohip_v4i res = {0, 0, 0, 0};
-    if (ep.residual != nullptr) res = *reinterpret_cast<const ohip_v4i*>(ep.residual + elem);  // wave-uniform
+    if constexpr (FUSED)
+        if (ep.residual != nullptr) res = *reinterpret_cast<const ohip_v4i*>(ep.residual + elem);  // wave-uniform
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)a[e], si[e], bi[e]);
         v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
         if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
-        if (ep.residual != nullptr) v = __fadd_rn(v, __int_as_float(res[e]));
-        r[e] = __float_as_int(v);
-        if (ep.twin != nullptr) {  // wave-uniform
-            const float t = __fmul_rn(v, ep.twin_scale);
-            const int k = (int)__fadd_rn(t, __builtin_copysignf(ep.twin_half, t));
-            q |= (unsigned)(min(max(k, -127), 127) & 0xff) << (8 * e);
+        if constexpr (FUSED) {
+            if (ep.residual != nullptr) v = __fadd_rn(v, __int_as_float(res[e]));
+            if (ep.twin != nullptr) {  // wave-uniform
+                const float t = __fmul_rn(v, ep.twin_scale);
+                const int k = (int)__fadd_rn(t, __builtin_copysignf(ep.twin_half, t));
+                q |= (unsigned)(min(max(k, -127), 127) & 0xff) << (8 * e);
+            }
         }
+        r[e] = __float_as_int(v);
     }
     *reinterpret_cast<ohip_v4i*>(out + elem) = r;
     return q;

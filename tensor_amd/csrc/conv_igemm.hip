@@ -185,15 +185,18 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                 if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
                     epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
                                                              elem_offset(8, n, ch0, pix, g.K, OHW), a8);
-                } else if constexpr (EPI == EPI_F32_P4) {
+                } else if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P4_FUSED) {
+                    constexpr bool FUSED = EPI == EPI_F32_P4_FUSED;
                     ohip_v2i tw = {0, 0};
-                    tw[0] = (int)epi4_store_f32p4((float*)out, ep, prm.si, prm.bi, elem_offset(4, n, ch0, pix, g.K, OHW),
-                                                  a8[0], a8[1], a8[2], a8[3]);
+                    tw[0] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si, prm.bi,
+                                                         elem_offset(4, n, ch0, pix, g.K, OHW), a8[0], a8[1], a8[2], a8[3]);
                     if (ch0 + 4 < g.K)
-                        tw[1] = (int)epi4_store_f32p4((float*)out, ep, prm.si + 4, prm.bi + 4,
-                                                      elem_offset(4, n, ch0 + 4, pix, g.K, OHW), a8[4], a8[5], a8[6], a8[7]);
-                    if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
-                        *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, g.K, OHW)) = tw;
+                        tw[1] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si + 4, prm.bi + 4,
+                                                             elem_offset(4, n, ch0 + 4, pix, g.K, OHW), a8[4], a8[5], a8[6],
+                                                             a8[7]);
+                    if constexpr (FUSED)
+                        if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
+                            *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, g.K, OHW)) = tw;
                 } else {
                     epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
                                             a8[6], a8[7]);
@@ -259,6 +262,8 @@ static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, co
     case EPI_I8_P8_NONNEG:
         return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8_NONNEG>(x, wpk, out, g, ep, stream);
     case EPI_F32_P4:
+        if (ep.twin != nullptr || ep.residual != nullptr)
+            return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4_FUSED>(x, wpk, out, g, ep, stream);
         return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, stream);
     default:
         return launch_igemm_e<TM, TN, WM, WN, EPI_GENERIC>(x, wpk, out, g, ep, stream);

@@ -241,6 +241,14 @@ int otter_hip_inner_product(const float* x, int n, int in_features, const float*
 int otter_hip_copy_channels(const float* src, int src_layout, int src_c, int src_c0, float* dst, int dst_layout,
                             int dst_c, int dst_c0, int count, int n, int h, int w, void* stream);
 
+/* The same copy and, in the same pass, the copied channels of what an int8 convolution reading dst would compute
+ * first: its quantize_to_int8 of the blob (Tensor/ConvolutionLayer.cpp:770-775), dst_q = float2int8(dst * scale) as
+ * Byte8 [N][dst_c/8][H*W][8]. One call per input of a Concat layer fills the whole of dst_q. Both layouts packed
+ * (F32_P4 / F32_P8), dst_c % 8 == 0, src_c0 % 4 == 0, and the destination range made of whole packs of dst_layout. */
+int otter_hip_copy_channels_quantize(const float* src, int src_layout, int src_c, int src_c0, float* dst,
+                                     int dst_layout, int dst_c, int dst_c0, int count, int n, int h, int w,
+                                     int8_t* dst_q, float scale, int round_mode, void* stream);
+
 /* ChannelShuffleLayer::forward (Tensor/ChannelShuffleLayer.cpp:37-41, Tensor/ChannelShuffleKernel.cpp:19-55):
  * out[:, j*groups + i] = in[:, i*(C/groups) + j]. */
 int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,

@@ -69,7 +69,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_set_tile", "otter_hip_eltwise_add", "otter_hip_activation", "otter_hip_global_avgpool",
            "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
-           "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual"]
+           "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
+           "otter_hip_copy_channels_quantize"]
 
 
 def load_cdll():
@@ -158,6 +159,13 @@ class Library:
         self._check(self.lib.otter_hip_copy_channels(self.ptr(src), src_layout, src_c, src_c0, self.ptr(dst), dst_layout,
                                                      dst_c, dst_c0, count, n, h, w, self.stream()))
         return dst
+
+    def copy_channels_quantize(self, src, src_layout, src_c, src_c0, dst, dst_layout, dst_c, dst_c0, count, n, h, w, dst_q,
+                               scale, round_mode):
+        self._check(self.lib.otter_hip_copy_channels_quantize(
+            self.ptr(src), src_layout, src_c, src_c0, self.ptr(dst), dst_layout, dst_c, dst_c0, count, n, h, w,
+            self.ptr(dst_q), C.c_float(scale), round_mode, self.stream()))
+        return dst, dst_q
 
     def channel_shuffle(self, src, src_layout, shape, groups, dst_layout):
         n, c, h, w = shape

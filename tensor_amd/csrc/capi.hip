@@ -609,6 +609,25 @@ int otter_hip_copy_channels(const float* src, int src_layout, int src_c, int src
     return OTTER_HIP_OK;
 }
 
+int otter_hip_copy_channels_quantize(const float* src, int src_layout, int src_c, int src_c0, float* dst, int dst_layout,
+                                     int dst_c, int dst_c0, int count, int n, int h, int w, int8_t* dst_q, float scale,
+                                     int round_mode, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_copy_channels_quantize", src, dst, src_layout, dst_layout, src_c, dst_c)) return rc;
+    if (!dst_q) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_copy_channels_quantize: null");
+    if (n < 0 || h < 1 || w < 1 || count < 0 || src_c0 < 0 || dst_c0 < 0 || src_c0 + count > src_c || dst_c0 + count > dst_c)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_copy_channels_quantize: channel range outside the blob");
+    if (round_mode != OTTER_HIP_ROUND_SSE && round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_copy_channels_quantize: unknown rounding mode");
+    if (dst_c % 8 || !copy_channels_moves_quads(layout_pack(src_layout), src_c0, layout_pack(dst_layout), dst_c0, count))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_copy_channels_quantize: needs packed layouts on both sides, dst_c % 8 == 0, "
+                                           "src_c0 % 4 == 0 and a destination range of whole packs");
+    if ((size_t)n * src_c * h * w >= (1ull << 31) || (size_t)n * dst_c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_copy_channels_quantize: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_copy_channels(src, src_c, layout_pack(src_layout), src_c0, dst, dst_c, layout_pack(dst_layout), dst_c0,
+                                 count, n, h, w, (hipStream_t)stream, dst_q, scale, round_mode));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,
                               int groups, void* stream) {
     if (int rc = check_f32_pair("otter_hip_channel_shuffle", src, dst, src_layout, dst_layout, c, c)) return rc;

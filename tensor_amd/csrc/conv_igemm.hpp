@@ -70,8 +70,11 @@ hipError_t run_conv_stem(const void* x, bool in_f32, const int8_t* wpk, void* ou
                          const float* in_scale, int in_round, hipStream_t stream);
 
 // reshape.hip: fp32 layout glue (pack = elempack of the layout on that side)
+// q (or null): also the Byte8 quantization of the copied channels, in a blob of Cd channels; needs
+// copy_channels_moves_quads(...) and Cd % 8 == 0
 hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
-                             int H, int W, hipStream_t stream);
+                             int H, int W, hipStream_t stream, int8_t* q = nullptr, float scale = 0.f, int round_mode = 0);
+bool copy_channels_moves_quads(int ps, int cs0, int pd, int cd0, int cnt);
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
                                hipStream_t stream);
 hipError_t run_shuffle2_split(const float* a, int pa, const float* b, int pb, float* c1, float* c2, int8_t* q2, float scale,

@@ -58,9 +58,12 @@ __global__ void __launch_bounds__(256) copy_channels_kernel(const float* __restr
 
 // same, four floats per thread: both packs are multiples of 4, the source offset is a multiple of 4 and the
 // destination range starts and ends on a destination pack boundary
+// With q: also the Byte8 quantization of the copied channels, q = float2int8(v * scale), at their place in a blob of Cd
+// channels (Cd % 8 == 0): what an int8 convolution reading dst would compute first.
 __global__ void __launch_bounds__(256) copy_channels4_kernel(const float* __restrict__ src, int Cs, int ps, int cs0,
                                                              float* __restrict__ dst, int Cd, int pd, int cd0, int cnt,
-                                                             int N, int H, int W, unsigned total4) {
+                                                             int N, int H, int W, unsigned total4, int8_t* __restrict__ qdst,
+                                                             float scale, float half) {
     const unsigned i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total4) return;
     // quads of the destination range in memory order: (n, pack, y, x, quad within the pack)
@@ -77,17 +80,34 @@ __global__ void __launch_bounds__(256) copy_channels4_kernel(const float* __rest
     const int n = (int)t;
     const float4 v = *reinterpret_cast<const float4*>(src + packed_off(n, c - cd0 + cs0, y, x, Cs, H, W, ps));
     *reinterpret_cast<float4*>(dst + packed_off(n, c, y, x, Cd, H, W, pd)) = v;
+    if (qdst != nullptr) {  // uniform
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        unsigned pk = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float t = __fmul_rn(f[e], scale);
+            const int k = (int)__fadd_rn(t, __builtin_copysignf(half, t));
+            pk |= (unsigned)(min(max(k, -127), 127) & 0xff) << (8 * e);
+        }
+        *reinterpret_cast<unsigned*>(qdst + packed_off(n, c, y, x, Cd, H, W, 8)) = pk;
+    }
+}
+
+bool copy_channels_moves_quads(int ps, int cs0, int pd, int cd0, int cnt) {
+    return cd0 % pd == 0 && cnt % pd == 0 && ps % 4 == 0 && pd % 4 == 0 && cs0 % 4 == 0;
 }
 
 hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
-                             int H, int W, hipStream_t stream) {
+                             int H, int W, hipStream_t stream, int8_t* q, float scale, int round_mode) {
     const size_t total = (size_t)N * cnt * H * W;
     if (total == 0) return hipSuccess;
     const bool whole = cd0 % pd == 0 && cnt % pd == 0;
-    if (whole && ps % 4 == 0 && pd % 4 == 0 && cs0 % 4 == 0) {
+    if (q != nullptr && !copy_channels_moves_quads(ps, cs0, pd, cd0, cnt)) return hipErrorInvalidValue;
+    if (copy_channels_moves_quads(ps, cs0, pd, cd0, cnt)) {
         const size_t total4 = total / 4;
         hipLaunchKernelGGL(copy_channels4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, src, Cs, ps,
-                           cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total4);
+                           cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total4, q, scale,
+                           round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f);
     } else if (whole) {
         hipLaunchKernelGGL(copy_channels_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, Cs,
                            ps, cs0, dst, Cd, pd, cd0, cnt, N, H, W, (unsigned)total);

@@ -825,6 +825,40 @@ private:
     const char* name_;
 };
 
+// Element-wise sum of fp32 blobs of one shape (Tensor/EltwiseLayer.cpp:48-80, Tensor/ShortCutLayer.cpp), in the first
+// blob's layout. With fuse_scale > 0 the last addition also writes the int8 blob the readers would make of the sum.
+static int sum_blobs(const std::vector<Tensor>& b, float fuse_scale, int fuse_round, std::vector<Tensor>& tops) {
+    if (b.size() < 2) return -1;
+    Tensor acc = b[0];
+    for (size_t i = 1; i < b.size(); ++i) {
+        if (base_of(b[i].scalar_type()) != ScalarType::Float || b[i].channels() != acc.channels()) return -1;
+        Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
+        Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
+        const bool last = i + 1 == b.size();
+        if (last && fuse_scale > 0.f && acc.dim() == 4 && acc.channels() % 8 == 0 && (acc.elempack() == 4 || acc.elempack() == 8)) {
+            // the readers are int8 convolutions: hand them the quantized blob along with the sum
+            Tensor q = Tensor::empty_device({acc.size(0), acc.channels() / 8, acc.size(2), acc.size(3)}, ScalarType::Byte8);
+            if (otter_hip_eltwise_add_quantize((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(),
+                                               hip_layout_of(acc.scalar_type()), (int)acc.size(0), (int)acc.channels(),
+                                               (int)acc.size(2), (int)acc.size(3), fuse_scale, fuse_round,
+                                               (float*)out.device_ptr(), (int8_t*)q.device_ptr(), nullptr))
+                return -1;
+            out.mark_device_written();
+            q.mark_device_written();
+            out.attach_quantized(q, fuse_scale, fuse_round);
+            acc = out;
+            continue;
+        }
+        if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
+                                  (size_t)acc.numel() * acc.elempack(), nullptr))
+            return -1;
+        out.mark_device_written();
+        acc = out;
+    }
+    tops.assign(1, acc);
+    return 0;
+}
+
 class EltwiseLayer : public Layer {  // Tensor/EltwiseLayer.cpp: operation "Sum"
 public:
     EltwiseLayer() { support_packing = true; }
@@ -836,39 +870,9 @@ public:
         return 0;
     }
     int forward(const std::vector<Tensor>& b, std::vector<Tensor>& tops, const NetOption&) const override {
-        if (b.size() < 2) return -1;
-        Tensor acc = b[0];
-        for (size_t i = 1; i < b.size(); ++i) {
-            if (base_of(b[i].scalar_type()) != ScalarType::Float || b[i].channels() != acc.channels()) return -1;
-            Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
-            Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
-            const bool last = i + 1 == b.size();
-            if (last && fuse_scale > 0.f && acc.dim() == 4 && acc.channels() % 8 == 0 && (acc.elempack() == 4 || acc.elempack() == 8)) {
-                // the readers are int8 convolutions: hand them the quantized blob along with the sum
-                Tensor q = Tensor::empty_device({acc.size(0), acc.channels() / 8, acc.size(2), acc.size(3)}, ScalarType::Byte8);
-                if (otter_hip_eltwise_add_quantize((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(),
-                                                   hip_layout_of(acc.scalar_type()), (int)acc.size(0), (int)acc.channels(),
-                                                   (int)acc.size(2), (int)acc.size(3), fuse_scale, fuse_round,
-                                                   (float*)out.device_ptr(), (int8_t*)q.device_ptr(), nullptr))
-                    return -1;
-                out.mark_device_written();
-                q.mark_device_written();
-                out.attach_quantized(q, fuse_scale, fuse_round);
-                acc = out;
-                continue;
-            }
-            if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
-                                      (size_t)acc.numel() * acc.elempack(), nullptr))
-                return -1;
-            out.mark_device_written();
-            acc = out;
-        }
-        tops.assign(1, acc);
-        return 0;
+        return sum_blobs(b, fuse_scale, fuse_round, tops);
     }
     std::string type() const override { return "Eltwise"; }
-    float fuse_scale = 0.f;  // > 0: also quantize the sum with this scale (set by Net::plan_fused_quantize)
-    int fuse_round = 0;
 };
 
 class SplitLayer : public Layer {  // Tensor/SplitLayer.cpp: every top shares the bottom blob
@@ -1015,16 +1019,31 @@ public:
             C += t.channels();
         }
         Tensor out = empty_f32_device(b[0].size(0), C, b[0].size(2), b[0].size(3));
+        // the readers are int8 convolutions: every copy also writes its channels of the quantized blob, when all of
+        // them move whole quads of channels
+        bool with_q = fuse_scale > 0.f && C % 8 == 0 && out.elempack() % 4 == 0;
+        for (const Tensor& t : b) with_q = with_q && t.channels() % 4 == 0 && t.elempack() % 4 == 0;
+        Tensor q;
+        if (with_q) q = Tensor::empty_device({b[0].size(0), C / 8, b[0].size(2), b[0].size(3)}, ScalarType::Byte8);
         int at = 0;
         for (const Tensor& t : b) {
             const int c = (int)t.channels();
-            if (otter_hip_copy_channels((const float*)t.device_ptr(), hip_layout_of(t.scalar_type()), c, 0,
+            const int rc = with_q ? otter_hip_copy_channels_quantize(
+                                        (const float*)t.device_ptr(), hip_layout_of(t.scalar_type()), c, 0,
                                         (float*)out.device_ptr(), hip_layout_of(out.scalar_type()), (int)C, at, c,
-                                        (int)t.size(0), (int)t.size(2), (int)t.size(3), nullptr))
-                return -1;
+                                        (int)t.size(0), (int)t.size(2), (int)t.size(3), (int8_t*)q.device_ptr(), fuse_scale,
+                                        fuse_round, nullptr)
+                                  : otter_hip_copy_channels((const float*)t.device_ptr(), hip_layout_of(t.scalar_type()), c, 0,
+                                                            (float*)out.device_ptr(), hip_layout_of(out.scalar_type()), (int)C,
+                                                            at, c, (int)t.size(0), (int)t.size(2), (int)t.size(3), nullptr);
+            if (rc) return -1;
             at += c;
         }
         out.mark_device_written();
+        if (with_q) {
+            q.mark_device_written();
+            out.attach_quantized(q, fuse_scale, fuse_round);
+        }
         tops.assign(1, out);
         return 0;
     }
@@ -1118,21 +1137,11 @@ public:
     }
     int forward(const std::vector<Tensor>& b, std::vector<Tensor>& tops, const NetOption&) const override {
         if (b.size() < 2 || !f32_4d(b[0])) return -1;
-        Tensor acc = b[0];
-        for (size_t i = 1; i < b.size(); ++i) {
+        for (size_t i = 1; i < b.size(); ++i)
             // different channel counts select darknet's partial shortcut, which the reference leaves unimplemented
-            if (!f32_4d(b[i]) || b[i].channels() != acc.channels() || b[i].size(2) != acc.size(2) || b[i].size(3) != acc.size(3))
+            if (!f32_4d(b[i]) || b[i].channels() != b[0].channels() || b[i].size(2) != b[0].size(2) || b[i].size(3) != b[0].size(3))
                 return -1;
-            Tensor rhs = b[i].elempack() == acc.elempack() ? b[i] : b[i].packing(acc.elempack());
-            Tensor out = Tensor::empty_device(acc.sizes(), acc.scalar_type());
-            if (otter_hip_eltwise_add((const float*)acc.device_ptr(), (const float*)rhs.device_ptr(), (float*)out.device_ptr(),
-                                      (size_t)acc.numel() * acc.elempack(), nullptr))
-                return -1;
-            out.mark_device_written();
-            acc = out;
-        }
-        tops.assign(1, acc);
-        return 0;
+        return sum_blobs(b, fuse_scale, fuse_round, tops);
     }
     std::string type() const override { return "ShortCut"; }
 };
@@ -1538,17 +1547,16 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
     return 0;
 }
 
-// An fp32 blob -- an Eltwise sum, or the dequantized result of an int8 convolution that something else reads as fp32
-// too -- that feeds int8 convolutions is quantized by each of them before anything else happens; when they agree on
-// the scale and the rounding primitive, its producer does it on the way (one pass over the blob instead of two, one
-// launch less per reader). Readers behind the automatic Split layers count.
+// An fp32 blob that feeds int8 convolutions is quantized by each of them before anything else happens; when they agree
+// on the scale and the rounding primitive, its producer is told so (Layer::fuse_scale) and, if it is a layer that can
+// -- an element-wise sum, a channel concatenation, an int8 convolution with an fp32 result -- does it on the way (one
+// pass over the blob instead of two, one launch less per reader). Readers behind the automatic Split layers count.
 void Net::plan_fused_quantize() const {
     for (Layer* l : layers_) {
-        auto* e = dynamic_cast<EltwiseLayer*>(l);
-        auto* pc = dynamic_cast<ConvolutionLayer*>(l);
-        if (pc && (!pc->int8_scale_term || pc->int8_scale_term > 100)) pc = nullptr;  // fp32 results only
-        if (!e && !pc) continue;
-        (e ? e->fuse_scale : pc->fuse_scale) = 0.f;
+        l->fuse_scale = 0.f;
+        if (l->tops.size() != 1 || l->type() == "Split" || l->type() == "Input") continue;
+        if (const auto* pc = dynamic_cast<const ConvolutionLayer*>(l))
+            if (!pc->int8_scale_term || pc->int8_scale_term > 100) continue;  // fp32 results only
         std::vector<int> pending(l->tops.begin(), l->tops.end());
         float scale = 0.f;
         int round = 0;
@@ -1569,16 +1577,14 @@ void Net::plan_fused_quantize() const {
                 }
             }
         }
-        if (agree && scale > 0.f) {
-            if (e) e->fuse_scale = scale, e->fuse_round = round;
-            else pc->fuse_scale = scale, pc->fuse_round = round;
-        }
+        if (agree && scale > 0.f) l->fuse_scale = scale, l->fuse_round = round;
     }
-    // Residual block tails: Eltwise sum of two blobs, one the fp32 result of an int8 convolution read by nothing else
+    // Residual block tails: Eltwise / ShortCut sum of two blobs, one the fp32 result of an int8 convolution read by
+    // nothing else
     residual_units_.clear();
     for (size_t ei = 0; ei < layers_.size(); ++ei) {
-        const auto* e = dynamic_cast<const EltwiseLayer*>(layers_[ei]);
-        if (!e || e->bottoms.size() != 2) continue;
+        const Layer* e = layers_[ei];
+        if ((e->type() != "Eltwise" && e->type() != "ShortCut") || e->bottoms.size() != 2) continue;
         int best = -1;
         for (int k = 0; k < 2; ++k) {
             const int b = e->bottoms[k], pi = blobs_[b].producer;
@@ -1638,7 +1644,7 @@ void Net::plan_fused_quantize() const {
 // allow it; the caller then runs the layers one by one.
 int Net::forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const {
     const auto* conv = static_cast<const ConvolutionLayer*>(layers_[u.conv]);
-    const auto* e = static_cast<const EltwiseLayer*>(layers_[u.eltwise]);
+    const Layer* e = layers_[u.eltwise];
     for (int b : {u.shortcut, conv->bottoms[0]})
         if (!blobs[b].defined()) {
             const int rc = forward_layer(blobs_[b].producer, blobs, opt);

@@ -159,6 +159,11 @@ public:
     std::vector<int> bottoms, tops;
     std::vector<std::vector<int64_t>> bottom_shapes, top_shapes;  // logical [N,C,H,W]
     std::string name;
+    // Set by Net::plan_fused_quantize for a layer with one fp32 top blob that int8 convolutions read: fuse_scale > 0 is
+    // their common input scale, fuse_round their rounding primitive. A layer that can quantize on the way attaches the
+    // int8 blob to its top blob (Tensor::attach_quantized); one that cannot ignores the two.
+    float fuse_scale = 0.f;
+    int fuse_round = 0;
 };
 
 // Tensor/LayerRegistry.hpp:17-85: string-keyed factory; a later AddCreator overrides an earlier one
@@ -202,11 +207,6 @@ public:
     Tensor weight_data_int8_scales, bottom_blob_int8_scales, top_blob_int8_scales, scale_in_data;
     // when set, forward() produces fp32 even if int8_scale_term > 100 is absent etc.; -1 = the reference's rule
     int force_out_layout = -1;
-    // > 0: an fp32 top blob is also quantized with this scale, for the int8 convolutions that read it next (set by
-    // Net::plan_fused_quantize)
-    float fuse_scale = 0.f;
-    int fuse_round = 0;
-
     int input_round_mode(const NetOption& opt) const;
     // This layer followed by the Eltwise sum with `shortcut` in one launch (otter_hip_conv_forward_residual), for a layer
     // with an fp32 result whose only reader is that sum: sum = activation(convolution) + shortcut, quantized on the way

@@ -101,6 +101,32 @@ def test_eltwise_add_quantize(hip, oracle, p, mode):
     np.testing.assert_array_equal(_host(q, 8, shape), want_q)
 
 
+@pytest.mark.parametrize("ps,pd", list(itertools.product([4, 8], repeat=2)))
+@pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT])
+def test_copy_channels_quantize_builds_the_concat_and_its_int8_blob(hip, oracle, ps, pd, mode):
+    """A Concat of three blobs (24 + 8 + 16 channels; 4 channels from the middle of a blob at the end when the
+    destination packs allow it): the fp32 result equals numpy's, the Byte8 blob the oracle's quantize of it, rounding
+    ties included."""
+    rng = np.random.default_rng(ps * 10 + pd + mode)
+    N, H, W, scale = 2, 5, 7, 37.5
+    parts = [rng.normal(0, 1, (N, c, H, W)).astype(np.float32) for c in (24, 8, 16)]
+    parts[1].reshape(-1)[:64] = (np.arange(64) - 32 + 0.5) / np.float32(scale)   # exact ties
+    ranges = [(0, 24), (0, 8), (4, 8) if pd == 8 else (4, 4)]   # (first source channel, count)
+    Cd = sum(r[1] for r in ranges)
+    Cd += (-Cd) % 8
+    dst = hip.to_device(np.zeros(N * Cd * H * W, np.float32))
+    q = hip.to_device(np.zeros(N * Cd * H * W, np.int8))
+    want = np.zeros((N, Cd, H, W), np.float32)
+    at = 0
+    for part, (s0, cnt) in zip(parts, ranges):
+        hip.copy_channels_quantize(_dev(hip, part, ps), F32[ps], part.shape[1], s0, dst, F32[pd], Cd, at, cnt, N, H, W, q,
+                                   scale, mode)
+        want[:, at:at + cnt] = part[:, s0:s0 + cnt]
+        at += cnt
+    np.testing.assert_array_equal(_host(dst, pd, want.shape), want)
+    np.testing.assert_array_equal(_host(q, 8, want.shape), oracle.quantize(want, [scale], mode))
+
+
 def test_shuffle2_split_is_concat_shuffle_and_two_crops(hip):
     rng = np.random.default_rng(9)
     N, Ch, H, W = 3, 24, 5, 9
@@ -133,3 +159,8 @@ def test_glue_argument_errors(hip):
         hip.maxpool2d(x, capi.F32, (1, 8, 4, 4), (3, 3), (2, 2), (1, 1), (1, 1), (9, 9), 0.0, capi.F32)  # output too large
     with pytest.raises(capi.HipError):
         hip.eltwise_add_quantize(x, x, capi.F32, (1, 8, 4, 4), 1.0, capi.ROUND_SSE)  # unpacked blobs
+    q = hip.to_device(np.zeros(8 * 16, np.int8))
+    with pytest.raises(capi.HipError):
+        hip.copy_channels_quantize(x, capi.F32, 8, 0, x, capi.F32_P8, 8, 0, 8, 1, 4, 4, q, 1.0, capi.ROUND_SSE)   # unpacked source
+    with pytest.raises(capi.HipError):
+        hip.copy_channels_quantize(x, capi.F32_P4, 8, 0, x, capi.F32_P4, 12, 0, 8, 1, 2, 2, q, 1.0, capi.ROUND_SSE)  # dst_c % 8

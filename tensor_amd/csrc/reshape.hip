@@ -239,10 +239,52 @@ __global__ void __launch_bounds__(256) maxpool_kernel(const float* __restrict__ 
     dst[i] = m;
 }
 
+// the same window, four channels per thread: both layouts packed by a multiple of 4, so a channel quad of one pixel is one
+// 16-byte access on either side; threads in destination memory order (n, pack, y, x, quad within the pack)
+__global__ void __launch_bounds__(256) maxpool4_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
+                                                       int C, int H, int W, int OH, int OW, int kh, int kw, int sh, int sw,
+                                                       int ph, int pw, int dh, int dw, float pad_value, unsigned total4) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total4) return;
+    const unsigned qd = (unsigned)(pd / 4);
+    unsigned r = i / qd;
+    const int q = (int)(i - r * qd);
+    unsigned t = r / (unsigned)OW;
+    const int ox = (int)(r - t * (unsigned)OW);
+    r = t / (unsigned)OH;
+    const int oy = (int)(t - r * (unsigned)OH);
+    const unsigned packs = (unsigned)(C / pd);
+    t = r / packs;
+    const int c = (int)(r - t * packs) * pd + 4 * q;
+    const int n = (int)t;
+    const float ninf = -__builtin_inff();
+    float m[4] = {ninf, ninf, ninf, ninf};
+    for (int u = 0; u < kh; ++u) {
+        const int iy = oy * sh - ph + u * dh;
+        for (int v = 0; v < kw; ++v) {
+            const int ix = ox * sw - pw + v * dw;
+            const bool inside = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            float4 val = make_float4(pad_value, pad_value, pad_value, pad_value);
+            if (inside) val = *reinterpret_cast<const float4*>(src + packed_off(n, c, iy, ix, C, H, W, ps));
+            const float f[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (f[e] > m[e] || f[e] != f[e]) m[e] = f[e];
+        }
+    }
+    *reinterpret_cast<float4*>(dst + packed_off(n, c, oy, ox, C, OH, OW, pd)) = make_float4(m[0], m[1], m[2], m[3]);
+}
+
 hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int kh,
                        int kw, int sh, int sw, int ph, int pw, int dh, int dw, float pad_value, hipStream_t stream) {
     const size_t total = (size_t)N * C * OH * OW;
     if (total == 0) return hipSuccess;
+    if (ps % 4 == 0 && pd % 4 == 0) {
+        const size_t total4 = total / 4;
+        hipLaunchKernelGGL(maxpool4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, C, H,
+                           W, OH, OW, kh, kw, sh, sw, ph, pw, dh, dw, pad_value, (unsigned)total4);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(maxpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
                        W, OH, OW, kh, kw, sh, sw, ph, pw, dh, dw, pad_value, (unsigned)total);
     return hipGetLastError();
@@ -290,10 +332,56 @@ __global__ void __launch_bounds__(256) upsample_kernel(const float* __restrict__
     dst[i] = __fmaf_rn(r1, b1, __fmul_rn(r0, b0));
 }
 
+// the same arithmetic, four channels per thread (both layouts packed by a multiple of 4): the coefficients of a pixel are
+// computed once per channel quad, every tap is one 16-byte read
+__global__ void __launch_bounds__(256) upsample4_kernel(const float* __restrict__ src, int ps, float* __restrict__ dst, int pd,
+                                                        int C, int H, int W, int OH, int OW, int mode, int align_corner,
+                                                        unsigned total4) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total4) return;
+    const unsigned qd = (unsigned)(pd / 4);
+    unsigned r = i / qd;
+    const int q = (int)(i - r * qd);
+    unsigned t = r / (unsigned)OW;
+    const int ox = (int)(r - t * (unsigned)OW);
+    r = t / (unsigned)OH;
+    const int oy = (int)(t - r * (unsigned)OH);
+    const unsigned packs = (unsigned)(C / pd);
+    t = r / packs;
+    const int c = (int)(r - t * packs) * pd + 4 * q;
+    const int n = (int)t;
+    auto at = [&](int y, int x) { return *reinterpret_cast<const float4*>(src + packed_off(n, c, y, x, C, H, W, ps)); };
+    float4* out = reinterpret_cast<float4*>(dst + packed_off(n, c, oy, ox, C, OH, OW, pd));
+    if (mode == 1) {
+        const float hs = (float)H / (float)OH, ws = (float)W / (float)OW;
+        *out = at(min((int)(oy * hs), H - 1), min((int)(ox * ws), W - 1));
+        return;
+    }
+    int sx, sy;
+    float fx, fy;
+    linear_coeff(W, OW, ox, align_corner, sx, fx);
+    linear_coeff(H, OH, oy, align_corner, sy, fy);
+    const float a0 = 1.f - fx, a1 = fx, b0 = 1.f - fy, b1 = fy;
+    const float4 s00 = at(sy, sx), s01 = at(sy, sx + 1), s10 = at(sy + 1, sx), s11 = at(sy + 1, sx + 1);
+    auto mix = [&](float v00, float v01, float v10, float v11) {
+        const float r0 = __fmaf_rn(v01, a1, __fmul_rn(v00, a0));
+        const float r1 = __fmaf_rn(v11, a1, __fmul_rn(v10, a0));
+        return __fmaf_rn(r1, b1, __fmul_rn(r0, b0));
+    };
+    *out = make_float4(mix(s00.x, s01.x, s10.x, s11.x), mix(s00.y, s01.y, s10.y, s11.y), mix(s00.z, s01.z, s10.z, s11.z),
+                       mix(s00.w, s01.w, s10.w, s11.w));
+}
+
 hipError_t run_upsample(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int mode,
                         int align_corner, hipStream_t stream) {
     const size_t total = (size_t)N * C * OH * OW;
     if (total == 0) return hipSuccess;
+    if (ps % 4 == 0 && pd % 4 == 0 && H > 1 && W > 1) {
+        const size_t total4 = total / 4;
+        hipLaunchKernelGGL(upsample4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, C, H,
+                           W, OH, OW, mode, align_corner, (unsigned)total4);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(upsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd, N, C, H,
                        W, OH, OW, mode, align_corner, (unsigned)total);
     return hipGetLastError();

@@ -254,6 +254,13 @@ int otter_hip_copy_channels_quantize(const float* src, int src_layout, int src_c
 int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,
                               int groups, void* stream);
 
+/* The same shuffle and, in the same pass, what an int8 convolution reading dst would compute first: its
+ * quantize_to_int8 of the blob (Tensor/ConvolutionLayer.cpp:770-775), dst_q = float2int8(dst * scale) as Byte8. For the
+ * ShuffleNetV2 case only: 2 groups, F32_P8 on both sides, C % 16 == 0. */
+int otter_hip_channel_shuffle_quantize(const float* src, int src_layout, float* dst, int dst_layout, int n, int c,
+                                       int h, int w, int groups, int8_t* dst_q, float scale, int round_mode,
+                                       void* stream);
+
 /* The tail of a ShuffleNetV2 unit as the reference's model files spell it -- ConcatLayer(a, b) -> ChannelShuffleLayer with
  * 2 groups -> two CropLayers taking the first and the second half of the channels (Tensor/ConcatLayer.cpp:54-67,
  * Tensor/ChannelShuffleKernel.cpp:19-55, Tensor/CropLayer.cpp:69-75) -- in one pass: first_half[2j+i] = (i ? b : a)[j],

@@ -70,7 +70,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
-           "otter_hip_copy_channels_quantize"]
+           "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize"]
 
 
 def load_cdll():
@@ -173,6 +173,15 @@ class Library:
         self._check(self.lib.otter_hip_channel_shuffle(self.ptr(src), src_layout, self.ptr(dst), dst_layout, n, c, h, w,
                                                        groups, self.stream()))
         return dst
+
+    def channel_shuffle_quantize(self, src, shape, groups, scale, round_mode, layout=F32_P8):
+        n, c, h, w = shape
+        dst = self.empty(n * c * h * w, np.float32)
+        q = self.empty(n * c * h * w, np.int8)
+        self._check(self.lib.otter_hip_channel_shuffle_quantize(self.ptr(src), layout, self.ptr(dst), layout, n, c, h, w,
+                                                                groups, self.ptr(q), C.c_float(scale), round_mode,
+                                                                self.stream()))
+        return dst, q
 
     def shuffle2_split(self, a, b, n, channels_each, h, w, scale=None, round_mode=0, a_layout=F32_P8, b_layout=F32_P8):
         c1 = self.empty(n * channels_each * h * w, np.float32)

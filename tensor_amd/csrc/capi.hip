@@ -640,6 +640,21 @@ int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int 
     return OTTER_HIP_OK;
 }
 
+int otter_hip_channel_shuffle_quantize(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h,
+                                       int w, int groups, int8_t* dst_q, float scale, int round_mode, void* stream) {
+    if (int rc = check_f32_pair("otter_hip_channel_shuffle_quantize", src, dst, src_layout, dst_layout, c, c)) return rc;
+    if (!dst_q) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_channel_shuffle_quantize: null");
+    if (n < 0 || h < 1 || w < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_channel_shuffle_quantize: bad shape");
+    if (round_mode != OTTER_HIP_ROUND_SSE && round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_channel_shuffle_quantize: unknown rounding mode");
+    if (!channel_shuffle_can_quantize(layout_pack(src_layout), layout_pack(dst_layout), c, groups))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_channel_shuffle_quantize: needs 2 groups, F32_P8 on both sides, C % 16 == 0");
+    if ((size_t)n * c * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_channel_shuffle_quantize: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_channel_shuffle(src, 8, dst, 8, n, c, h, w, groups, (hipStream_t)stream, dst_q, scale, round_mode));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_shuffle2_split(const float* a, int a_layout, const float* b, int b_layout, int n, int channels_each, int h,
                              int w, float* first_half, float* second_half, int8_t* second_half_q, float scale,
                              int round_mode, void* stream) {

@@ -75,8 +75,10 @@ hipError_t run_conv_stem(const void* x, bool in_f32, const int8_t* wpk, void* ou
 hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
                              int H, int W, hipStream_t stream, int8_t* q = nullptr, float scale = 0.f, int round_mode = 0);
 bool copy_channels_moves_quads(int ps, int cs0, int pd, int cd0, int cnt);
+// q (or null): also the Byte8 quantization of the shuffled blob; needs channel_shuffle_can_quantize(...)
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
-                               hipStream_t stream);
+                               hipStream_t stream, int8_t* q = nullptr, float scale = 0.f, int round_mode = 0);
+bool channel_shuffle_can_quantize(int ps, int pd, int C, int groups);
 hipError_t run_shuffle2_split(const float* a, int pa, const float* b, int pb, float* c1, float* c2, int8_t* q2, float scale,
                               int round_mode, int N, int Ch, int HW, hipStream_t stream);
 hipError_t run_maxpool(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int OH, int OW, int kh,

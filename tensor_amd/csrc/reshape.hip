@@ -131,8 +131,10 @@ __global__ void __launch_bounds__(256) channel_shuffle_kernel(const float* __res
 
 // groups == 2 on elempack 8 (the ShuffleNetV2 block of the detection model): output pack q interleaves source channels
 // 4q..4q+3 of the first half with the same four of the second half -- two 16-byte reads, two 16-byte writes per pixel
+// qdst (or null): also the Byte8 quantization of the shuffled blob, for int8 convolutions that read it next
 __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* __restrict__ src, float* __restrict__ dst,
-                                                                  int C, int HW, unsigned total) {
+                                                                  int C, int HW, unsigned total, int8_t* __restrict__ qdst,
+                                                                  float scale, float half_ulp) {
     const unsigned i = blockIdx.x * 256 + threadIdx.x;  // (n, output pack, pixel)
     if (i >= total) return;
     const unsigned r = i / (unsigned)HW;
@@ -148,6 +150,20 @@ __global__ void __launch_bounds__(256) channel_shuffle2_p8_kernel(const float* _
     float4* o = reinterpret_cast<float4*>(dst + (n * (size_t)C * HW) + ((size_t)q * HW + px) * 8);
     o[0] = make_float4(a.x, b.x, a.y, b.y);
     o[1] = make_float4(a.z, b.z, a.w, b.w);
+    if (qdst != nullptr) {  // uniform
+        const float f[8] = {a.x, b.x, a.y, b.y, a.z, b.z, a.w, b.w};
+        int v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float t = __fmul_rn(f[e], scale);
+            const int k = (int)__fadd_rn(t, __builtin_copysignf(half_ulp, t));
+            v[e] = min(max(k, -127), 127) & 0xff;
+        }
+        ohip_v2i pk;
+        pk[0] = v[0] | (v[1] << 8) | (v[2] << 16) | (v[3] << 24);
+        pk[1] = v[4] | (v[5] << 8) | (v[6] << 16) | (v[7] << 24);
+        reinterpret_cast<ohip_v2i*>(qdst)[i] = pk;  // same (n, pack, pixel) order as dst
+    }
 }
 
 // The ShuffleNetV2 unit tail in one pass: Concat(a, b) -> ChannelShuffle(2 groups) -> the two half Crops. With Ch channels
@@ -201,14 +217,17 @@ hipError_t run_shuffle2_split(const float* a, int pa, const float* b, int pb, fl
     return hipGetLastError();
 }
 
+bool channel_shuffle_can_quantize(int ps, int pd, int C, int groups) { return groups == 2 && ps == 8 && pd == 8 && C % 16 == 0; }
+
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
-                               hipStream_t stream) {
+                               hipStream_t stream, int8_t* q, float scale, int round_mode) {
     const size_t total = (size_t)N * C * H * W;
     if (total == 0) return hipSuccess;
-    if (groups == 2 && ps == 8 && pd == 8 && C % 16 == 0) {
+    if (q != nullptr && !channel_shuffle_can_quantize(ps, pd, C, groups)) return hipErrorInvalidValue;
+    if (channel_shuffle_can_quantize(ps, pd, C, groups)) {
         const size_t units = total / 8;
         hipLaunchKernelGGL(channel_shuffle2_p8_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, src, dst, C,
-                           H * W, (unsigned)units);
+                           H * W, (unsigned)units, q, scale, round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(channel_shuffle_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, src, ps, dst, pd,

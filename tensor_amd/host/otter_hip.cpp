@@ -1115,6 +1115,18 @@ public:
         if (!f32_4d(b) || groups_ < 1 || b.channels() % groups_) return -1;
         top = Tensor::empty_device(b.sizes(), b.scalar_type());
         const int l = hip_layout_of(b.scalar_type());
+        if (fuse_scale > 0.f && groups_ == 2 && b.elempack() == 8 && b.channels() % 16 == 0) {
+            // the readers are int8 convolutions: hand them the quantized blob along with the shuffled one
+            Tensor q = Tensor::empty_device(b.sizes(), ScalarType::Byte8);
+            if (otter_hip_channel_shuffle_quantize((const float*)b.device_ptr(), l, (float*)top.device_ptr(), l, (int)b.size(0),
+                                                   (int)b.channels(), (int)b.size(2), (int)b.size(3), groups_,
+                                                   (int8_t*)q.device_ptr(), fuse_scale, fuse_round, nullptr))
+                return -1;
+            top.mark_device_written();
+            q.mark_device_written();
+            top.attach_quantized(q, fuse_scale, fuse_round);
+            return 0;
+        }
         if (otter_hip_channel_shuffle((const float*)b.device_ptr(), l, (float*)top.device_ptr(), l, (int)b.size(0),
                                       (int)b.channels(), (int)b.size(2), (int)b.size(3), groups_, nullptr))
             return -1;

@@ -127,6 +127,20 @@ def test_copy_channels_quantize_builds_the_concat_and_its_int8_blob(hip, oracle,
     np.testing.assert_array_equal(_host(q, 8, want.shape), oracle.quantize(want, [scale], mode))
 
 
+@pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT])
+def test_channel_shuffle_quantize(hip, oracle, mode):
+    rng = np.random.default_rng(5 + mode)
+    shape, scale = (3, 48, 6, 7), 29.5
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    x.reshape(-1)[:64] = (np.arange(64) - 32 + 0.5) / np.float32(scale)   # exact ties
+    dst, q = hip.channel_shuffle_quantize(_dev(hip, x, 8), shape, 2, scale, mode)
+    want = x.reshape(3, 2, 24, 6, 7).transpose(0, 2, 1, 3, 4).reshape(shape)
+    np.testing.assert_array_equal(_host(dst, 8, shape), want)
+    np.testing.assert_array_equal(_host(q, 8, shape), oracle.quantize(want, [scale], mode))
+    with pytest.raises(capi.HipError):
+        hip.channel_shuffle_quantize(_dev(hip, x, 8), shape, 3, scale, mode)      # the two-group kernel only
+
+
 def test_shuffle2_split_is_concat_shuffle_and_two_crops(hip):
     rng = np.random.default_rng(9)
     N, Ch, H, W = 3, 24, 5, 9

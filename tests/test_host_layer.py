@@ -218,19 +218,19 @@ def test_residual_block_tail_runs_as_one_launch_with_the_same_blobs(oracle, k, a
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("glue", ["Concat", "ShortCut"])
+@pytest.mark.parametrize("glue", ["Concat", "ShortCut", "Concat+ChannelShuffle"])
 @pytest.mark.parametrize("same_scale", [True, False], ids=["readers_agree", "readers_disagree"])
 def test_concat_and_shortcut_feeding_int8_convolutions_quantize_on_the_way(oracle, glue, same_scale):
     """Two fp32 convolution results joined by a Concat (channels) or a ShortCut (sum) and read by two int8
     convolutions: the joining layer writes the readers' int8 input itself when they agree on the scale."""
     rng = np.random.default_rng(41 + len(glue))
-    C, K = 16, 24
+    C, K = 16, 24   # 2K = 48 channels: a multiple of 16, as the quantizing shuffle needs
     x = rng.uniform(-1, 1, (2, C, 9, 11)).astype(np.float32)
     w1, s1 = _qweights(rng, K, C, 1)
     w2, s2 = _qweights(rng, K, C, 3)
     b1, b2 = (rng.normal(0, 0.1, K).astype(np.float32) for _ in range(2))
     in_x = np.float32(127) / np.abs(x).max()
-    J = 2 * K if glue == "Concat" else K
+    J = K if glue == "ShortCut" else 2 * K
     wa, sa = _qweights(rng, K, J, 1)
     wb, sb = _qweights(rng, 8, J, 3)
     ba, bb = rng.normal(0, 0.1, K).astype(np.float32), rng.normal(0, 0.1, 8).astype(np.float32)
@@ -239,13 +239,19 @@ def test_concat_and_shortcut_feeding_int8_convolutions_quantize_on_the_way(oracl
     net.add_layer(type="Convolution", name="c1", input="data", out_channels=K, kernel=1, int8_scale_term=2)
     net.add_layer(type="Convolution", name="c2", input="data", out_channels=K, kernel=3, padding=1, int8_scale_term=2,
                   activation="Relu")
-    net.add_layer(type=glue, name="j", input="c1,c2")
+    if glue == "Concat+ChannelShuffle":
+        net.add_layer(type="Concat", name="cat", input="c1,c2")
+        net.add_layer(type="ChannelShuffle", name="j", input="cat", groups=2)
+    else:
+        net.add_layer(type=glue, name="j", input="c1,c2")
     net.add_layer(type="Convolution", name="a", input="j", out_channels=K, kernel=1, int8_scale_term=102, activation="Relu6")
     net.add_layer(type="Convolution", name="b", input="j", out_channels=8, kernel=3, padding=1, int8_scale_term=2)
     net.compile()
     y1 = oracle.conv_layer_forward(x, w1, s1, in_x, bias=b1)
     y2 = oracle.conv_layer_forward(x, w2, s2, in_x, pad=(1, 1), bias=b2, act_type=1)
-    j = np.concatenate([y1, y2], axis=1) if glue == "Concat" else y1 + y2
+    j = y1 + y2 if glue == "ShortCut" else np.concatenate([y1, y2], axis=1)
+    if glue == "Concat+ChannelShuffle":
+        j = j.reshape(2, 2, K, 9, 11).transpose(0, 2, 1, 3, 4).reshape(2, 2 * K, 9, 11)
     in_a = np.float32(127) / np.abs(j).max() * np.float32(1.1)
     in_b = in_a if same_scale else np.float32(in_a * 0.8)
     net.set_conv("c1", w1, b1, s1, in_x)

@@ -249,6 +249,15 @@ int otter_hip_copy_channels_quantize(const float* src, int src_layout, int src_c
                                      int dst_layout, int dst_c, int dst_c0, int count, int n, int h, int w,
                                      int8_t* dst_q, float scale, int round_mode, void* stream);
 
+/* ConcatLayer::forward with axis 1 (Tensor/ConcatLayer.cpp:54-67) in one launch: `count` (1 to 8) blobs of one batch
+ * size and image size, src_channels[i] channels each in layout src_layouts[i], one after the other along the channel
+ * axis of dst. Packed layouts only (F32_P4 / F32_P8 on every side; otter_hip_copy_channels covers the rest). With dst_q
+ * (or NULL; needs a channel sum divisible by 8) also the quantize_to_int8 of dst that an int8 convolution reading it
+ * would compute first (Tensor/ConvolutionLayer.cpp:770-775): dst_q = float2int8(dst * scale) as Byte8. */
+int otter_hip_concat_channels(const float* const* srcs, const int* src_layouts, const int* src_channels, int count,
+                              float* dst, int dst_layout, int n, int h, int w, int8_t* dst_q, float scale,
+                              int round_mode, void* stream);
+
 /* ChannelShuffleLayer::forward (Tensor/ChannelShuffleLayer.cpp:37-41, Tensor/ChannelShuffleKernel.cpp:19-55):
  * out[:, j*groups + i] = in[:, i*(C/groups) + j]. */
 int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h, int w,

@@ -70,7 +70,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_inner_product", "otter_hip_eltwise_add_quantize", "otter_hip_copy_channels",
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
-           "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize"]
+           "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
+           "otter_hip_concat_channels"]
 
 
 def load_cdll():
@@ -166,6 +167,19 @@ class Library:
             self.ptr(src), src_layout, src_c, src_c0, self.ptr(dst), dst_layout, dst_c, dst_c0, count, n, h, w,
             self.ptr(dst_q), C.c_float(scale), round_mode, self.stream()))
         return dst, dst_q
+
+    def concat_channels(self, srcs, src_layouts, src_channels, n, h, w, dst_layout, scale=None, round_mode=ROUND_SSE):
+        """Concat over channels in one launch; with scale also the Byte8 quantization of the result."""
+        k = len(srcs)
+        total = sum(src_channels)
+        dst = self.empty(n * total * h * w, np.float32)
+        q = self.empty(n * total * h * w, np.int8) if scale is not None else None
+        ptrs = (C.c_void_p * k)(*[t.data_ptr() for t in srcs])
+        self._check(self.lib.otter_hip_concat_channels(ptrs, (C.c_int * k)(*src_layouts), (C.c_int * k)(*src_channels), k,
+                                                       self.ptr(dst), dst_layout, n, h, w,
+                                                       self.ptr(q) if q is not None else None, C.c_float(scale or 0.0),
+                                                       round_mode, self.stream()))
+        return dst, q
 
     def channel_shuffle(self, src, src_layout, shape, groups, dst_layout):
         n, c, h, w = shape

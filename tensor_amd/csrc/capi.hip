@@ -640,6 +640,38 @@ int otter_hip_channel_shuffle(const float* src, int src_layout, float* dst, int 
     return OTTER_HIP_OK;
 }
 
+int otter_hip_concat_channels(const float* const* srcs, const int* src_layouts, const int* src_channels, int count,
+                              float* dst, int dst_layout, int n, int h, int w, int8_t* dst_q, float scale, int round_mode,
+                              void* stream) {
+    if (!srcs || !src_layouts || !src_channels || !dst) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: null");
+    if (count < 1 || count > CONCAT_MAX)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_concat_channels: 1 to 8 sources (use otter_hip_copy_channels for more)");
+    if (n < 0 || h < 1 || w < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: bad shape");
+    if (!valid_layout(dst_layout) || layout_elem(dst_layout) != 0 || layout_pack(dst_layout) % 4)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: F32_P4 or F32_P8 destination expected");
+    ConcatSources cs;
+    int total = 0;
+    for (int i = 0; i < count; ++i) {
+        if (!srcs[i] || !valid_layout(src_layouts[i]) || layout_elem(src_layouts[i]) != 0 || layout_pack(src_layouts[i]) % 4 ||
+            src_channels[i] < 1 || src_channels[i] % layout_pack(src_layouts[i]))
+            return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: packed fp32 sources with whole packs expected");
+        cs.ptr[i] = srcs[i], cs.channels[i] = src_channels[i], cs.pack[i] = layout_pack(src_layouts[i]), cs.first[i] = total;
+        total += src_channels[i];
+    }
+    for (int i = count; i < CONCAT_MAX; ++i) cs.ptr[i] = nullptr, cs.channels[i] = 0, cs.pack[i] = 4, cs.first[i] = 0x7fffffff;
+    cs.count = count;
+    if (total % layout_pack(dst_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: the destination pack does not divide the channel sum");
+    if (dst_q && total % 8) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: the quantized blob needs C % 8 == 0");
+    if (dst_q && round_mode != OTTER_HIP_ROUND_SSE && round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_concat_channels: unknown rounding mode");
+    if ((size_t)n * total * h * w >= (1ull << 31))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_concat_channels: tensor exceeds 2^31 elements");
+    OHIP_CHECK(run_concat_channels(cs, dst, total, layout_pack(dst_layout), n, h, w, dst_q, scale, round_mode,
+                                   (hipStream_t)stream));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_channel_shuffle_quantize(const float* src, int src_layout, float* dst, int dst_layout, int n, int c, int h,
                                        int w, int groups, int8_t* dst_q, float scale, int round_mode, void* stream) {
     if (int rc = check_f32_pair("otter_hip_channel_shuffle_quantize", src, dst, src_layout, dst_layout, c, c)) return rc;

@@ -75,6 +75,15 @@ hipError_t run_conv_stem(const void* x, bool in_f32, const int8_t* wpk, void* ou
 hipError_t run_copy_channels(const float* src, int Cs, int ps, int cs0, float* dst, int Cd, int pd, int cd0, int cnt, int N,
                              int H, int W, hipStream_t stream, int8_t* q = nullptr, float scale = 0.f, int round_mode = 0);
 bool copy_channels_moves_quads(int ps, int cs0, int pd, int cd0, int cnt);
+// a Concat over channels in one launch (packed layouts, channel counts in multiples of 4)
+constexpr int CONCAT_MAX = 8;
+struct ConcatSources {
+    const float* ptr[CONCAT_MAX];
+    int channels[CONCAT_MAX], pack[CONCAT_MAX], first[CONCAT_MAX];  // first: destination channel of the source's channel 0
+    int count;
+};
+hipError_t run_concat_channels(const ConcatSources& srcs, float* dst, int Cd, int pd, int N, int H, int W, int8_t* q,
+                               float scale, int round_mode, hipStream_t stream);
 // q (or null): also the Byte8 quantization of the shuffled blob; needs channel_shuffle_can_quantize(...)
 hipError_t run_channel_shuffle(const float* src, int ps, float* dst, int pd, int N, int C, int H, int W, int groups,
                                hipStream_t stream, int8_t* q = nullptr, float scale = 0.f, int round_mode = 0);

@@ -93,6 +93,54 @@ __global__ void __launch_bounds__(256) copy_channels4_kernel(const float* __rest
     }
 }
 
+// A whole Concat over channels in one launch: up to CONCAT_MAX packed fp32 sources, every channel count a multiple of
+// 4, into a packed destination; one thread per channel quad of one destination pixel, in destination memory order.
+// With qdst also the Byte8 quantization of the result (Cd % 8 == 0), as in copy_channels4_kernel.
+__global__ void __launch_bounds__(256) concat_channels4_kernel(ConcatSources srcs, float* __restrict__ dst, int Cd, int pd,
+                                                               int H, int W, unsigned total4, int8_t* __restrict__ qdst,
+                                                               float scale, float half) {
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total4) return;
+    const unsigned qd = (unsigned)(pd / 4);
+    unsigned r = i / qd;
+    const int q = (int)(i - r * qd);
+    unsigned t = r / (unsigned)W;
+    const int x = (int)(r - t * (unsigned)W);
+    r = t / (unsigned)H;
+    const int y = (int)(t - r * (unsigned)H);
+    const unsigned packs = (unsigned)(Cd / pd);
+    t = r / packs;
+    const int c = (int)(r - t * packs) * pd + 4 * q;
+    const int n = (int)t;
+    int k = 0;  // the source that holds destination channel c
+#pragma unroll
+    for (int j = 1; j < CONCAT_MAX; ++j)
+        if (j < srcs.count && c >= srcs.first[j]) k = j;
+    const float4 v = *reinterpret_cast<const float4*>(srcs.ptr[k] +
+                                                      packed_off(n, c - srcs.first[k], y, x, srcs.channels[k], H, W, srcs.pack[k]));
+    *reinterpret_cast<float4*>(dst + packed_off(n, c, y, x, Cd, H, W, pd)) = v;
+    if (qdst != nullptr) {  // uniform
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        unsigned pk = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float tt = __fmul_rn(f[e], scale);
+            const int kk = (int)__fadd_rn(tt, __builtin_copysignf(half, tt));
+            pk |= (unsigned)(min(max(kk, -127), 127) & 0xff) << (8 * e);
+        }
+        *reinterpret_cast<unsigned*>(qdst + packed_off(n, c, y, x, Cd, H, W, 8)) = pk;
+    }
+}
+
+hipError_t run_concat_channels(const ConcatSources& srcs, float* dst, int Cd, int pd, int N, int H, int W, int8_t* q,
+                               float scale, int round_mode, hipStream_t stream) {
+    const size_t total4 = (size_t)N * Cd * H * W / 4;
+    if (total4 == 0) return hipSuccess;
+    hipLaunchKernelGGL(concat_channels4_kernel, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stream, srcs, dst, Cd, pd,
+                       H, W, (unsigned)total4, q, scale, round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f);
+    return hipGetLastError();
+}
+
 bool copy_channels_moves_quads(int ps, int cs0, int pd, int cd0, int cnt) {
     return cd0 % pd == 0 && cnt % pd == 0 && ps % 4 == 0 && pd % 4 == 0 && cs0 % 4 == 0;
 }

@@ -1025,6 +1025,26 @@ public:
         for (const Tensor& t : b) with_q = with_q && t.channels() % 4 == 0 && t.elempack() % 4 == 0;
         Tensor q;
         if (with_q) q = Tensor::empty_device({b[0].size(0), C / 8, b[0].size(2), b[0].size(3)}, ScalarType::Byte8);
+        bool quads = b.size() <= 8 && out.elempack() % 4 == 0;
+        for (const Tensor& t : b) quads = quads && t.elempack() % 4 == 0;
+        if (quads) {  // every blob packed: the whole layer is one launch
+            const float* ptrs[8];
+            int layouts[8], channels[8];
+            for (size_t i = 0; i < b.size(); ++i)
+                ptrs[i] = (const float*)b[i].device_ptr(), layouts[i] = hip_layout_of(b[i].scalar_type()), channels[i] = (int)b[i].channels();
+            if (otter_hip_concat_channels(ptrs, layouts, channels, (int)b.size(), (float*)out.device_ptr(),
+                                          hip_layout_of(out.scalar_type()), (int)b[0].size(0), (int)b[0].size(2),
+                                          (int)b[0].size(3), with_q ? (int8_t*)q.device_ptr() : nullptr, fuse_scale, fuse_round,
+                                          nullptr))
+                return -1;
+            out.mark_device_written();
+            if (with_q) {
+                q.mark_device_written();
+                out.attach_quantized(q, fuse_scale, fuse_round);
+            }
+            tops.assign(1, out);
+            return 0;
+        }
         int at = 0;
         for (const Tensor& t : b) {
             const int c = (int)t.channels();

@@ -127,6 +127,23 @@ def test_copy_channels_quantize_builds_the_concat_and_its_int8_blob(hip, oracle,
     np.testing.assert_array_equal(_host(q, 8, want.shape), oracle.quantize(want, [scale], mode))
 
 
+@pytest.mark.parametrize("packs", [(4, 4, 4, 4), (8, 8, 8, 8), (4, 8, 8, 4), (8, 4, 4, 8)], ids=str)
+@pytest.mark.parametrize("with_q", [False, True], ids=["plain", "quantized"])
+def test_concat_channels_in_one_launch(hip, oracle, packs, with_q):
+    """otter_hip_concat_channels: three sources (layouts packs[0..2]) into a destination of layout packs[3], equal to
+    numpy's concatenate; with a scale also the oracle's quantize of the result, rounding ties included."""
+    rng = np.random.default_rng(sum(p * (i + 1) for i, p in enumerate(packs)))
+    N, H, W, scale = 2, 5, 7, 37.5
+    parts = [rng.normal(0, 1, (N, c, H, W)).astype(np.float32) for c in (24, 8, 16)]
+    parts[1].reshape(-1)[:64] = (np.arange(64) - 32 + 0.5) / np.float32(scale)   # exact ties
+    want = np.concatenate(parts, axis=1)
+    dst, q = hip.concat_channels([_dev(hip, a, p) for a, p in zip(parts, packs)], [F32[p] for p in packs[:3]],
+                                 [a.shape[1] for a in parts], N, H, W, F32[packs[3]], scale if with_q else None, capi.ROUND_SSE)
+    np.testing.assert_array_equal(_host(dst, packs[3], want.shape), want)
+    if with_q:
+        np.testing.assert_array_equal(_host(q, 8, want.shape), oracle.quantize(want, [scale], capi.ROUND_SSE))
+
+
 @pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT])
 def test_channel_shuffle_quantize(hip, oracle, mode):
     rng = np.random.default_rng(5 + mode)
@@ -178,3 +195,7 @@ def test_glue_argument_errors(hip):
         hip.copy_channels_quantize(x, capi.F32, 8, 0, x, capi.F32_P8, 8, 0, 8, 1, 4, 4, q, 1.0, capi.ROUND_SSE)   # unpacked source
     with pytest.raises(capi.HipError):
         hip.copy_channels_quantize(x, capi.F32_P4, 8, 0, x, capi.F32_P4, 12, 0, 8, 1, 2, 2, q, 1.0, capi.ROUND_SSE)  # dst_c % 8
+    with pytest.raises(capi.HipError):
+        hip.concat_channels([x, x], [capi.F32, capi.F32_P4], [4, 4], 1, 2, 2, capi.F32_P4)   # an unpacked source
+    with pytest.raises(capi.HipError):
+        hip.concat_channels([x] * 9, [capi.F32_P4] * 9, [4] * 9, 1, 1, 1, capi.F32_P4)       # more than 8 sources

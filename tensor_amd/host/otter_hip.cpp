@@ -1045,6 +1045,8 @@ public:
             tops.assign(1, out);
             return 0;
         }
+        // one copy per input; it can quantize on the way only if every input fills whole packs of the result
+        for (const Tensor& t : b) with_q = with_q && t.channels() % out.elempack() == 0;
         int at = 0;
         for (const Tensor& t : b) {
             const int c = (int)t.channels();

@@ -176,6 +176,15 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
  * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo kernel would be picked. */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
+/* Test hook with no counterpart in the reference, host arithmetic only (no GPU needed): the launch plan of the 3x3
+ * stride-1 LDS-halo kernel for a dense layer of this shape. plan = { pixel fragments per wave, pixels per tile, tiles
+ * per image, persistent workgroups (grid.x), row blocks (grid.y), 1 if a workgroup reuses the per-lane LDS offsets of
+ * its first tile for its later tiles, LDS rows per tile, input channels per LDS stage }. Workgroup b walks tiles
+ * b, b + grid.x, ...; tile t (after the XCD swizzle t' = (t % 8) * (T / 8) + t / 8 for t < 8 * (T / 8), T = all tiles)
+ * is pixels [ (t' % tiles_per_image) * pixels_per_tile, ... ) of image t' / tiles_per_image. */
+int otter_hip_conv3x3_halo_plan(int in_channels, int out_channels, int pad, int n, int in_h, int in_w, int force_fn,
+                                int plan[8]);
+
 /* ------------------------------------------------------------------------------------------------ */
 /* standalone quantize / dequantize / requantize                                                    */
 /* ------------------------------------------------------------------------------------------------ */

@@ -170,6 +170,12 @@ class Oracle:
                                      out.ctypes.data_as(C.c_void_p))
         return out
 
+    def eltwise_add(self, a, b):
+        a, b = _f32(a), _f32(b)
+        out = np.empty_like(a)
+        self.lib.otter_oracle_eltwise_add(_p(a, _f32p), _p(b, _f32p), C.c_size_t(a.size), _p(out, _f32p))
+        return out
+
     def global_avgpool(self, x):
         x = _f32(x)
         n, c, h, w = x.shape

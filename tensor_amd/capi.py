@@ -71,7 +71,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
-           "otter_hip_concat_channels"]
+           "otter_hip_concat_channels", "otter_hip_conv3x3_halo_plan"]
 
 
 def load_cdll():

@@ -322,6 +322,19 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, 
     return pick_kernel(h, l, g, make_epilogue(h, out_layout));
 }
 
+int otter_hip_conv3x3_halo_plan(int in_channels, int out_channels, int pad, int n, int in_h, int in_w, int force_fn,
+                                int plan[8]) {
+    if (!plan || in_channels < 1 || out_channels < 1 || pad < 0 || n < 1 || in_h < 1 || in_w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv3x3_halo_plan: bad argument");
+    otter_hip_conv_desc d{};
+    d.in_channels = in_channels, d.out_channels = out_channels, d.kernel_h = d.kernel_w = 3, d.stride_h = d.stride_w = 1;
+    d.pad_h = d.pad_w = pad, d.dilation_h = d.dilation_w = 1, d.groups = 1;
+    const ConvGeom g = make_geom(d, n, in_h, in_w);
+    if (g.OH < 1 || g.OW < 1 || !conv3x3_halo_plan(g, force_fn, plan))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv3x3_halo_plan: the LDS-halo kernel does not take this shape");
+    return OTTER_HIP_OK;
+}
+
 // the convolution; `twin` (or null) receives the Byte8 quantization of an fp32 result, from the convolution's own
 // epilogue where that kernel can write it and from a quantize pass after it otherwise
 // `residual` (or null): a blob in the output's layout added to the fp32 result; the twin is then made of the sum

@@ -131,7 +131,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
         // LDS address of this lane's pixel (tap 0,0) per fragment, octet pair lane/16 of the current k-chunk; walks
         // forward by one chunk after the ninth tap and is wound back at the end of a stage
         // (kept as LDS byte offsets: a generic pointer here would turn the ds_read into a flat load).
-        // When a tile is a whole number of image rows the offsets are the same for every tile: computed once.
+        // When every tile is a whole number of image rows and the image a whole number of tiles (no ragged last
+        // tile, whose lanes past the image end would keep a clamped pixel) the offsets are the same for every
+        // tile: computed once.
         if (wg0 == (int)blockIdx.x || !tile_inv) {
 #pragma unroll
             for (int f = 0; f < FN; ++f) {
@@ -317,6 +319,19 @@ int halo_rows(int pt, int OW, int OHW) {
     return worst;
 }
 
+// The per-lane LDS offsets of a tile may be reused for the workgroup's next tile only if every tile covers the same
+// pixels relative to its first row: tiles are whole image rows AND no tile is cut short by the end of the image.
+bool halo_tile_invariant(int pt, int OW, int OHW) { return pt % OW == 0 && OHW % pt == 0; }
+
+// grid.y = row blocks of rows_per_wg / 16 sixteen-row tiles; grid.x = persistent workgroups, two resident per CU
+void halo_grid(int mpad, int tiles16_per_wg, int total_tiles, int* m_blocks, int* grid_x) {
+    *m_blocks = (mpad / 16 + tiles16_per_wg - 1) / tiles16_per_wg;
+    int gx = 512 / *m_blocks;
+    if (gx < 8) gx = 8;
+    if (gx > total_tiles) gx = total_tiles;
+    *grid_x = gx;
+}
+
 template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
 hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                          const HaloPlan& pl, hipStream_t stream) {
@@ -329,16 +344,14 @@ hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const Co
         attr_set = true;
     }
     const int mpad = igemm_padded_rows(g.K);
-    const int m_blocks = (mpad / 16 + WM * FM - 1) / (WM * FM);
     const int prm_ofs = (int)((pl.lds_bytes + 15) / 16 * 16);
     const int total_tiles = g.N * pl.tiles_per_img;
-    int grid_x = 512 / m_blocks;  // two resident workgroups per CU
-    if (grid_x < 8) grid_x = 8;
-    if (grid_x > total_tiles) grid_x = total_tiles;
+    int m_blocks, grid_x;
+    halo_grid(mpad, WM * FM, total_tiles, &m_blocks, &grid_x);
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
     hipLaunchKernelGGL(kern, dim3(grid_x, m_blocks), dim3(256), prm_ofs + 3 * WM * FM * 16 * sizeof(float), stream, x, wpk,
                        out, g, ep, mpad / 16, igemm_channel_groups(g.C), pl.r_max, pl.cb, pl.tiles_per_img, prm_ofs,
-                       total_tiles, in_bytes, (WN * FN * 16) % g.OW == 0 ? 1 : 0);
+                       total_tiles, in_bytes, halo_tile_invariant(WN * FN * 16, g.OW, g.OH * g.OW) ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -415,16 +428,33 @@ bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep) {
     return plan_halo(g, 0, &p);
 }
 
+// the launch plan as numbers, for tests of the tile walk: fragment count, pixels per tile, tiles per image, grid.x,
+// grid.y, 1 if the per-lane LDS offsets are reused across a workgroup's tiles, LDS rows per tile, channels per stage
+bool conv3x3_halo_plan(const ConvGeom& g, int force_fn, int plan[8]) {
+    HaloPlan p;
+    if (!plan_halo(g, force_fn, &p) && !plan_halo(g, 0, &p)) return false;
+    const int mpad = igemm_padded_rows(g.K);
+    const int pt = (mpad > 64 ? 32 : 64) * p.fn;
+    int m_blocks, grid_x;
+    halo_grid(mpad, mpad > 64 ? 8 : (mpad == 64 ? 4 : 2), g.N * p.tiles_per_img, &m_blocks, &grid_x);
+    plan[0] = p.fn, plan[1] = pt, plan[2] = p.tiles_per_img, plan[3] = grid_x, plan[4] = m_blocks;
+    plan[5] = halo_tile_invariant(pt, g.OW, g.OH * g.OW) ? 1 : 0, plan[6] = p.r_max, plan[7] = p.cb;
+    return true;
+}
+
 hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                             int force_fn, hipStream_t stream) {
     HaloPlan p;
     // a forced fragment count that does not fit LDS falls back to the automatic choice
     if (!plan_halo(g, force_fn, &p) && !plan_halo(g, 0, &p)) return hipErrorInvalidValue;
-    const bool wide = igemm_padded_rows(g.K) > 64;
+    const int mpad = igemm_padded_rows(g.K);
+    // the weight rows and the per-channel constants are padded to mpad rows: a workgroup must not read past them,
+    // so 32 padded rows (K <= 32) take two row fragments per wave, not four
 #define OHIP_HALO(FN_)                                                                  \
     case FN_:                                                                           \
-        return wide ? launch_halo<4, FN_, 2, 2>(x, wpk, out, g, ep, p, stream)          \
-                    : launch_halo<4, FN_, 1, 4>(x, wpk, out, g, ep, p, stream);
+        return mpad > 64    ? launch_halo<4, FN_, 2, 2>(x, wpk, out, g, ep, p, stream)  \
+               : mpad == 64 ? launch_halo<4, FN_, 1, 4>(x, wpk, out, g, ep, p, stream)  \
+                            : launch_halo<2, FN_, 1, 4>(x, wpk, out, g, ep, p, stream);
     switch (p.fn) {
         OHIP_HALO(4)
         OHIP_HALO(5)

@@ -338,7 +338,7 @@ bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool sca
     if (g.ph > g.kh / 2 || !dw_mfma_window_fits(g.kh, g.sh, g.pw) || g.C % 8 != 0 || g.C != g.K) return false;
     if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4 && epi != EPI_F32_P8) return false;
     const size_t in_bytes = (size_t)g.N * g.C * g.H * g.W;
-    const size_t out_bytes = (size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 ? 4 : 1);
+    const size_t out_bytes = (size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 || epi == EPI_F32_P8 ? 4 : 1);
     return in_bytes < ((size_t)1 << 31) && out_bytes < ((size_t)1 << 31);  // 32-bit buffer offsets
 }
 

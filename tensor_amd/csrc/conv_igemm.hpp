@@ -16,6 +16,7 @@ hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const C
 
 // conv3x3.hip
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep);
+bool conv3x3_halo_plan(const ConvGeom& g, int force_fn, int plan[8]);
 hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                             int force_fn, hipStream_t stream);
 

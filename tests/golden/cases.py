@@ -29,6 +29,18 @@ LAYER_CASES = [
     ("dw_3x3s2_nopad_i8_f32_relu",  32, 32, 3, 2, 0, 1, 32,  9,  9, 1, True,  False, True,  "Relu",  None),
 ]
 
+# The same layer with `use_packing_layout = false` (Tensor/NetOption.hpp; the unpacked sgemm_conv2d_int8_x86 route,
+# Tensor/ConvolutionMM2DInt8X86.cpp:1182-1262, scalar float2int8 in quantize / requantize). Same columns. fp32 outputs
+# keep OH*OW % 4 == 0: the reference's unpacked dequantize leaves a ragged tail unwritten
+# (Tensor/QuantizeX86.cpp:1115-1125). Depthwise is left out: the reference throws there in unpacked mode.
+UNPACKED_LAYER_CASES = [
+    ("unpacked_3x3_c8k8_i8_relu",     8,  8, 3, 1, 1, 1,  1,  8,  6, 2, True,  True,  True,  "Relu",  None),
+    ("unpacked_3x3_c16k16_f32_f32",  16, 16, 3, 1, 1, 1,  1,  8,  8, 1, False, False, True,  "",      None),
+    ("unpacked_1x1_c12k6_i8",        12,  6, 1, 1, 0, 1,  1,  7,  5, 2, True,  True,  False, "",      None),
+    ("unpacked_3x3s2_c3k8_relu6_i8",  3,  8, 3, 2, 1, 1,  1, 13, 11, 2, False, True,  True,  "Relu6", None),
+    ("unpacked_3x3_c8k20_f32_lrelu",  8, 20, 3, 1, 1, 1,  1,  6,  6, 1, False, False, True,  "LRelu", [0.1]),
+]
+
 
 def layer_options(case):
     """The reference's own option keys (Tensor/ConvolutionLayer.cpp:58-156)."""

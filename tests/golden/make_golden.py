@@ -18,7 +18,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 sys.path.insert(0, HERE)
 
 from oracle.binding import Ref, out_size  # noqa: E402
-from cases import LAYER_CASES, layer_options, make_inputs  # noqa: E402
+from cases import LAYER_CASES, UNPACKED_LAYER_CASES, layer_options, make_inputs  # noqa: E402
 
 
 def near_tie_values(rng, n):
@@ -57,6 +57,26 @@ def main():
         G[name + "/acc"] = acc
         G[name + "/out"] = out
         print("%-32s out %s %s" % (name, out.dtype, out.shape))
+    # ---- layer level, use_packing_layout = false ---------------------------------------------------------
+    for i, case in enumerate(UNPACKED_LAYER_CASES):
+        name = case[0]
+        C, K, k, s, p, d, g = case[1:8]
+        H, W = case[8], case[9]
+        t = make_inputs(case, seed=300 + i)
+        L = R.conv_layer(layer_options(case), (1, C, H, W), t["wq"], t["bias"], t["w_scales"], float(t["in_scale"]),
+                         float(t["top_scale"]), False)
+        out, _ = L.forward(t["x"])
+        G[name + "/scale_in"] = L.scale_in()
+        L.close()
+        xq = t["x"] if t["x"].dtype == np.int8 else R.quantize(t["x"], [t["in_scale"]], False)
+        acc = R.conv_int32(xq, t["wq"], (s, s), (p, p), (d, d), g, False)
+        for key, v in t.items():
+            if v is not None:
+                G[name + "/" + key] = np.asarray(v)
+        G[name + "/xq"] = xq
+        G[name + "/acc"] = acc
+        G[name + "/out"] = out
+        print("%-32s out %s %s (unpacked)" % (name, out.dtype, out.shape))
     # ---- quantize fine print -----------------------------------------------------------------------
     for C in (8, 4, 3):
         v = near_tie_values(rng, 120)

@@ -6,8 +6,10 @@ from tensor_amd import capi
 ACT = {"": 0, "Relu": 1, "LRelu": 2, "Relu6": 3}
 
 
-def in_layout_for(x, C):
+def in_layout_for(x, C, use_packing=True):
     """The layout Net::convert_layout hands to the layer (Tensor/Net.cpp:388-405)."""
+    if not use_packing:
+        return capi.I8 if x.dtype == np.int8 else capi.F32
     if x.dtype == np.int8:
         return capi.I8_P8 if C % 8 == 0 else capi.I8
     if C % 8 == 0:
@@ -27,19 +29,22 @@ def host_scale_in(w_scales, in_scale):
 
 
 def run_conv(hip, oracle, x, wq, w_scales, in_scale, *, stride=1, pad=0, dil=1, groups=1, bias=None, top_scale=1.0,
-             out_kind=capi.OUT_I32, act=0, act_p0=0.0, out_layout=None, in_layout=None, tile=None):
+             out_kind=capi.OUT_I32, act=0, act_p0=0.0, out_layout=None, in_layout=None, tile=None, use_packing=True):
     """x: NCHW numpy (fp32 or int8). Returns the NCHW numpy result of the GPU layer."""
     n, C, H, W = x.shape
     K = wq.shape[0]
     conv = hip.conv(wq=wq, scale_in=host_scale_in(np.broadcast_to(w_scales, (K,)), in_scale), bias=bias,
                     in_scale=float(in_scale), out_scale=[top_scale] if out_kind == capi.OUT_I8 else None,
                     stride=(stride, stride), pad=(pad, pad), dil=(dil, dil), groups=groups, act=act, act_p0=act_p0,
-                    out_kind=out_kind, out_round=oracle.requantize_round_mode(C, K, groups, True),
-                    in_round=oracle.quantize_round_mode(C, True))
+                    out_kind=out_kind, out_round=oracle.requantize_round_mode(C, K, groups, use_packing),
+                    in_round=oracle.quantize_round_mode(C, use_packing))
     if tile is not None:
         conv.set_tile(*tile)
-    in_layout = in_layout_for(x, C) if in_layout is None else in_layout
-    out_layout = conv.default_out_layout() if out_layout is None else out_layout
+    in_layout = in_layout_for(x, C, use_packing) if in_layout is None else in_layout
+    if out_layout is None:
+        # unpacked mode: every blob is elempack 1 (Tensor/Net.cpp:388-405 with use_packing_layout = false)
+        out_layout = conv.default_out_layout() if use_packing else \
+            {capi.OUT_I32: capi.I32, capi.OUT_F32: capi.F32, capi.OUT_I8: capi.I8}[out_kind]
     xd = hip.to_device(capi.pack_np(x, capi.layout_pack(in_layout)))
     out = conv.forward(xd, in_layout, n, H, W, out_layout)
     hip.torch.cuda.synchronize()

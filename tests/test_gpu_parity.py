@@ -4,7 +4,7 @@ bit-exact; fp32 outputs within 1e-5 relative (they are in fact reproduced bitwis
 import numpy as np
 import pytest
 
-from cases import LAYER_CASES
+from cases import LAYER_CASES, UNPACKED_LAYER_CASES
 from gpu_util import ACT, host_scale_in, run_conv
 from oracle.binding import ROUND_EXACT, ROUND_SSE
 from tensor_amd import capi
@@ -46,6 +46,28 @@ def test_layer_against_reference_vectors(hip, oracle, golden, case):
     # the fast kernels must be the ones that ran, not the scalar fallback
     if C % 8 == 0 and (g == 1 or g == C == K):
         assert kind in (1, 2, 3)
+
+
+@pytest.mark.parametrize("case", UNPACKED_LAYER_CASES, ids=[c[0] for c in UNPACKED_LAYER_CASES])
+def test_unpacked_mode_layer_against_reference_vectors(hip, oracle, golden, case):
+    """use_packing_layout = false (the reference's unpacked sgemm_conv2d_int8_x86 route,
+    Tensor/ConvolutionMM2DInt8X86.cpp:1182-1262): every blob elempack 1, the scalar float2int8 in quantize and
+    requantize. Vectors written by the compiled reference's ConvolutionLayer::forward in that mode."""
+    name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params = case
+    x, wq = _g(golden, name, "x"), _g(golden, name, "wq")
+    common = dict(stride=s, pad=p, dil=d, groups=g, bias=_g(golden, name, "bias"),
+                  top_scale=float(_g(golden, name, "top_scale")), act=ACT[act],
+                  act_p0=float(act_params[0]) if act_params else 0.0, use_packing=False)
+    ws, ins = _g(golden, name, "w_scales"), float(_g(golden, name, "in_scale"))
+    acc, _ = run_conv(hip, oracle, x, wq, ws, ins, out_kind=capi.OUT_I32, **common)
+    np.testing.assert_array_equal(acc, _g(golden, name, "acc"))
+    want = _g(golden, name, "out")
+    out, _ = run_conv(hip, oracle, x, wq, ws, ins, out_kind=capi.OUT_I8 if i8_out else capi.OUT_F32, **common)
+    if i8_out:
+        np.testing.assert_array_equal(out, want)
+    else:
+        assert_f32_close(out, want)
+        np.testing.assert_array_equal(out.view(np.int32), want.view(np.int32))
 
 
 def test_layer_unpacked_input_layouts(hip, oracle, golden):
@@ -211,6 +233,21 @@ def test_halo3x3_every_fragment_count(hip, oracle, fn):
         acc, kind = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, out_kind=capi.OUT_I32, tile=(-1, fn))
         assert kind == 1
         np.testing.assert_array_equal(acc, acc_want)
+
+
+def test_halo3x3_ragged_last_tile_then_full_tile_in_one_workgroup(hip, oracle):
+    """Tiles of whole image rows (128 pixels = 8 rows of 16) on an image that is not a whole number of tiles (20 rows:
+    the third tile of an image has 4 rows), with so many output channels that the persistent grid is shorter than the
+    tile list: some workgroups start on a ragged tile and go on to a full one, whose lanes past the ragged tile's end
+    need their own LDS offsets."""
+    rng = np.random.default_rng(77)
+    C, K, N, H, W = 8, 1024, 32, 20, 16
+    x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
+    out, kind = run_conv(hip, oracle, x, wq, ws, 25.0, pad=1, bias=bias, top_scale=7.0, act=1, out_kind=capi.OUT_I8,
+                         tile=(-1, 4))
+    assert kind == 3
+    want = oracle.conv_layer_forward(x, wq, ws, 25.0, pad=(1, 1), bias=bias, top_scale=7.0, int8_out=True, act_type=1)
+    np.testing.assert_array_equal(out, want)
 
 
 @pytest.mark.parametrize("C,K,k,s,p,d,g,N,H,W", [

@@ -3,7 +3,7 @@
 import numpy as np
 import pytest
 
-from cases import LAYER_CASES
+from cases import LAYER_CASES, UNPACKED_LAYER_CASES
 from oracle.binding import ROUND_EXACT, ROUND_SSE
 
 ACT = {"": 0, "Relu": 1, "LRelu": 2, "Relu6": 3}
@@ -30,6 +30,27 @@ def test_layer_forward_matches_reference(oracle, golden, case):
         np.testing.assert_array_equal(out, want)
     else:
         # fp32 results are reproduced bitwise as well (fused multiply-add, same order)
+        np.testing.assert_array_equal(out.view(np.int32), want.view(np.int32))
+
+
+@pytest.mark.parametrize("case", UNPACKED_LAYER_CASES, ids=[c[0] for c in UNPACKED_LAYER_CASES])
+def test_unpacked_layer_forward_matches_reference(oracle, golden, case):
+    """use_packing_layout = false: the unpacked sgemm route with the scalar float2int8 in quantize / requantize
+    (Tensor/ConvolutionMM2DInt8X86.cpp:1182-1262, Tensor/QuantizeX86.cpp:617-641)."""
+    name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params = case
+    x, wq = _g(golden, name, "x"), _g(golden, name, "wq")
+    if not in_i8:
+        xq = oracle.quantize(x, [_g(golden, name, "in_scale")], oracle.quantize_round_mode(C, False))
+        np.testing.assert_array_equal(xq, _g(golden, name, "xq"))
+    out, acc = oracle.conv_layer_forward(
+        x, wq, _g(golden, name, "w_scales"), float(_g(golden, name, "in_scale")), stride=(s, s), pad=(p, p),
+        dil=(d, d), groups=g, bias=_g(golden, name, "bias"), top_scale=float(_g(golden, name, "top_scale")),
+        int8_out=i8_out, act_type=ACT[act], act_params=act_params, use_packing=False, want_acc=True)
+    np.testing.assert_array_equal(acc, _g(golden, name, "acc"))
+    want = _g(golden, name, "out")
+    if i8_out:
+        np.testing.assert_array_equal(out, want)
+    else:
         np.testing.assert_array_equal(out.view(np.int32), want.view(np.int32))
 
 
@@ -124,3 +145,50 @@ def test_pack_roundtrip_and_layout(oracle):
         pk = oracle.pack(a, p)
         np.testing.assert_array_equal(pk, a.reshape(2, 16 // p, p, 3, 5).transpose(0, 1, 3, 4, 2))
         np.testing.assert_array_equal(oracle.unpack(pk), a)
+
+
+def test_global_avgpool_against_closed_form(oracle):
+    """The mean over H*W per (image, channel), against a float64 mean and against cases with a known answer: a constant
+    plane returns the constant, a plane that is 1 at one pixel returns 1/(H*W) for that channel only (an index that
+    strides over channels instead of pixels, or a divisor of C instead of H*W, fails)."""
+    rng = np.random.default_rng(11)
+    x = rng.normal(0, 3, (3, 5, 7, 4)).astype(np.float32)
+    got = oracle.global_avgpool(x)
+    assert got.shape == (3, 5) and got.dtype == np.float32
+    np.testing.assert_allclose(got, x.astype(np.float64).mean(axis=(2, 3)), rtol=1e-6, atol=1e-7)
+    c = np.broadcast_to(np.arange(10, dtype=np.float32).reshape(2, 5, 1, 1), (2, 5, 3, 9))
+    np.testing.assert_array_equal(oracle.global_avgpool(c), np.arange(10, dtype=np.float32).reshape(2, 5))
+    one = np.zeros((2, 3, 4, 8), np.float32)
+    one[1, 2, 3, 5] = 1.0
+    want = np.zeros((2, 3), np.float32)
+    want[1, 2] = 1.0 / 32
+    np.testing.assert_array_equal(oracle.global_avgpool(one), want)
+
+
+def test_inner_product_against_closed_form(oracle):
+    """y[n][o] = sum_i x[n][i] * W[o][i] + b[o] (Tensor/InnerProductLayer.cpp:176-): a float64 matmul with a
+    NON-symmetric, non-square weight (a transposed weight index cannot even be evaluated consistently), unit vectors
+    that pick out single weight entries exactly, and the bias alone on a zero input."""
+    rng = np.random.default_rng(12)
+    n, in_f, out_f = 3, 37, 11
+    x = rng.normal(0, 1, (n, in_f)).astype(np.float32)
+    w = rng.normal(0, 1, (out_f, in_f)).astype(np.float32)
+    b = rng.normal(0, 1, out_f).astype(np.float32)
+    got = oracle.inner_product(x, w, b)
+    assert got.shape == (n, out_f) and got.dtype == np.float32
+    want = x.astype(np.float64) @ w.astype(np.float64).T + b.astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oracle.inner_product(x, w, None), want - b, rtol=1e-6, atol=1e-6)
+    # square but non-symmetric weight: e_i picks column i of W, i.e. y[o] = W[o][i] exactly
+    ws = rng.normal(0, 1, (6, 6)).astype(np.float32)
+    eye = np.eye(6, dtype=np.float32)
+    np.testing.assert_array_equal(oracle.inner_product(eye, ws, None), ws.T)
+    assert not np.array_equal(ws, ws.T)
+    np.testing.assert_array_equal(oracle.inner_product(np.zeros((2, in_f), np.float32), w, b), np.stack([b, b]))
+
+
+def test_eltwise_add_is_the_fp32_sum(oracle):
+    rng = np.random.default_rng(13)
+    a = rng.normal(0, 1e3, 1001).astype(np.float32)
+    b = rng.normal(0, 1e-3, 1001).astype(np.float32)
+    np.testing.assert_array_equal(oracle.eltwise_add(a, b), a + b)

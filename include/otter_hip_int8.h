@@ -139,6 +139,17 @@ size_t otter_hip_conv_workspace_bytes(const otter_hip_conv_t* handle, int in_lay
 int otter_hip_conv_forward(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h, int in_w,
                            void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference. For callers that cannot allocate device memory -- code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc: otter_hip_conv_forward with the workspace (the quantized copy
+ * of an fp32 input, or the channel-padded copy of a blob with C % 8 != 0) taken from a static device array of
+ * OTTER_HIP_STATIC_WORKSPACE_BYTES that the library holds on every GPU it runs on for the life of the process. Makes
+ * no hipMalloc / hipFree call. An input whose otter_hip_conv_workspace_bytes exceeds the array is refused with
+ * OTTER_HIP_ERR_UNSUPPORTED. Every call on one GPU shares that GPU's array: calls that overlap on one GPU (different
+ * streams or host threads) race; calls on one stream are ordered. Same results as otter_hip_conv_forward. */
+#define OTTER_HIP_STATIC_WORKSPACE_BYTES (32u << 20)
+int otter_hip_conv_forward_static(const otter_hip_conv_t* handle, const void* in, int in_layout, int n, int in_h,
+                                  int in_w, void* out, int out_layout, void* stream);
+
 /* The same forward for a layer with an fp32 result (out_kind F32, K % 8 == 0) whose top blob is read by int8
  * convolutions next: besides `out`, writes what each of those readers would compute first, its quantize_to_int8 of the
  * blob (Tensor/ConvolutionLayer.cpp:770-775), out_q = float2int8(out * q_scale) as Byte8 [N][K/8][OH*OW][8].

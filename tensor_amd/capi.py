@@ -71,7 +71,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
-           "otter_hip_concat_channels", "otter_hip_conv3x3_halo_plan"]
+           "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan"]
 
 
 def load_cdll():
@@ -282,6 +282,16 @@ class Conv:
         self.L._check(self.L.lib.otter_hip_conv_forward(
             self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout,
             self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))
+        return out
+
+    def forward_static(self, x, in_layout, n, h, w, out_layout=None, out=None):
+        """otter_hip_conv_forward_static: the workspace is the library's static device array (no allocation inside)."""
+        out_layout = self.default_out_layout() if out_layout is None else out_layout
+        oh, ow = self.out_hw(h, w)
+        if out is None:
+            out = self.L.empty(n * self.K * oh * ow, layout_dtype(out_layout))
+        self.L._check(self.L.lib.otter_hip_conv_forward_static(
+            self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout, self.L.stream()))
         return out
 
     def forward_twin(self, x, in_layout, n, h, w, q_scale, q_round_mode, out_layout=None):

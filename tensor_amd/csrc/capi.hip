@@ -2,6 +2,7 @@
 // weight re-layout at create time and kernel dispatch. No kernels live here.
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -45,6 +46,46 @@ int upload(T** dev, const T* host, size_t count, size_t padded_count, T pad_valu
     return OTTER_HIP_OK;
 }
 
+// ---- the workspace of otter_hip_conv_forward_static ---------------------------------------------------------
+// A file-scope device array: every GPU the library runs on holds its own copy, at its own address, until the process
+// ends. `scratch` below is only a host-side stand-in for the symbol: the device address comes from
+// hipGetSymbolAddress, once per device with that device current, and only that address is handed to kernels.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[OTTER_HIP_STATIC_WORKSPACE_BYTES];
+
+namespace {
+
+// device address of `scratch` on the current device (looked up on first use, then kept); null + error text on failure
+void* static_workspace(int* rc) {
+    *rc = OTTER_HIP_OK;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        *rc = hip_fail(e, "hipGetDevice");
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        *rc = fail(OTTER_HIP_ERR_UNSUPPORTED, "static workspace: device index out of range");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            *rc = hip_fail(e == hipSuccess ? hipErrorInvalidSymbol : e, "hipGetSymbolAddress(scratch)");
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
 }  // namespace
 
 struct otter_hip_conv {
@@ -78,7 +119,10 @@ int otter_hip_init(int device) {
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(OTTER_HIP_ERR_UNSUPPORTED,
                     std::string("otter_hip_init: this library is built for gfx950 only, found ") + prop.gcnArchName);
-    return OTTER_HIP_OK;
+    // this device's copy of the static workspace (otter_hip_conv_forward_static)
+    int rc = OTTER_HIP_OK;
+    (void)static_workspace(&rc);
+    return rc;
 }
 
 int otter_hip_shutdown(void) { return OTTER_HIP_OK; }
@@ -454,6 +498,21 @@ int otter_hip_conv_forward(const otter_hip_conv_t* h, const void* in, int in_lay
                            void* out, int out_layout, void* workspace, size_t workspace_bytes, void* stream) {
     return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, nullptr, 0.f,
                         0);
+}
+
+int otter_hip_conv_forward_static(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
+                                  void* out, int out_layout, void* stream) {
+    if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_static: bad argument");
+    const size_t need = otter_hip_conv_workspace_bytes(h, in_layout, n < 0 ? 0 : n, in_h, in_w);
+    if (need > (size_t)OTTER_HIP_STATIC_WORKSPACE_BYTES)
+        return fail(OTTER_HIP_ERR_UNSUPPORTED,
+                    "otter_hip_conv_forward_static: this input needs a workspace of " + std::to_string(need) +
+                        " bytes, the static one holds " + std::to_string((size_t)OTTER_HIP_STATIC_WORKSPACE_BYTES) +
+                        "; split the batch or use otter_hip_conv_forward with a workspace of your own");
+    int rc = OTTER_HIP_OK;
+    void* ws = need ? static_workspace(&rc) : nullptr;
+    if (rc != OTTER_HIP_OK) return rc;
+    return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, ws, need, stream, nullptr, 0.f, 0);
 }
 
 int otter_hip_conv_forward_residual(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,

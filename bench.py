@@ -1,13 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 convolution path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c0|c4|det] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c2i8|c0|c0n64|c4|det] [--no-cpu] [--no-also]
 
 Prints ONE JSON line. The headline workload is the fourth benchmark configuration (the MFMA-bound case the metric's
 "int8 conv TOPS (% MFMA peak)" is quoted on): four chained int8-in/int8-out 3x3 convolutions 128->128 at
 56x56, batch 64, fused requantize+ReLU. One step = the four layers back to back on device-resident int8
 activations. The other single-GPU configurations (depthwise c1 at stride 1 and 2 with its HBM roofline, the
-1x1 GEMM c2, the single-image c0) are measured the same way and reported under "also".
+1x1 GEMM c2 and its int8-output variant, the single-image c0 and the same layer at batch 64) are measured the same
+way and reported under "also". A bandwidth-bound kernel's roofline figure comes from a loop that rotates over enough
+buffer sets to exceed the 256 MB last-level cache; the figure of the loop over one (cache-resident) set is reported
+beside it as "roofline_resident".
 
 Timing: HIP events recorded on the stream the kernels are launched on (torch's current stream is handed to the
 C ABI as the launch stream), inputs resident in HBM before the timed region. Every timed loop is preceded by an
@@ -47,13 +50,22 @@ class Timer:
     def __init__(self, torch):
         self.torch = torch
 
-    def run(self, fn, steps, warmup):
+    def run(self, fn, steps, warmup, settle=None):
+        """fn: a closure, or a list of closures taken in turn (the same launch over different buffer sets, so that the
+        loop's footprint exceeds the caches)."""
         t = self.torch
+        if isinstance(fn, (list, tuple)):
+            fns, state = list(fn), [0]
+
+            def fn():
+                fns[state[0] % len(fns)]()
+                state[0] += 1
+        settle = SETTLE_S if settle is None else settle
         # The shader clock ramps up over the first tens of milliseconds of load (measured: the same 4-layer step
         # takes 135 us in its first 100 iterations after an idle period and 120 us from then on), so the step runs
         # untimed for SETTLE_S first; the W warm-up steps and the K timed steps follow as the contract has them.
         t0 = time.perf_counter()
-        while time.perf_counter() - t0 < SETTLE_S:
+        while time.perf_counter() - t0 < settle:
             for _ in range(10):
                 fn()
             t.cuda.synchronize()
@@ -74,6 +86,13 @@ class Timer:
 # ------------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------------
+
+COLD_BYTES = 320 << 20  # footprint of a rotating loop: above the 256 MB of the last-level (Infinity) cache
+
+
+def cold_sets(bytes_per_set):
+    return max(2, -(-COLD_BYTES // bytes_per_set))
+
 
 def build_c3(hip, capi, rng):
     """configs[3]: 4 x (128->128 3x3 s1 p1) at 56x56, batch 64, int8 in / int8 out, requantize+ReLU. The output
@@ -143,51 +162,75 @@ def build_c1(hip, capi, rng, stride):
         return out
 
     in_b, out_b = N * C * H * W, N * C * oh * ow
-    return dict(name="c1s%d" % stride, step=step, ops=2.0 * N * C * 9 * oh * ow, launches=2,
+    # the same launches over enough buffer sets that nothing a launch reads is still in a cache from the last time
+    step()
+    n_dom = cold_sets(in_b + out_b)
+    xqs, outs = [xq.clone() for _ in range(n_dom)], [hip.empty(out_b, np.int8) for _ in range(n_dom)]
+    dom_cold = [lambda i=i: conv.forward(xqs[i], capi.I8_P8, N, H, W, capi.I8_P8, out=outs[i]) for i in range(n_dom)]
+    n_aux = cold_sets(5 * in_b)
+    xds, xq2 = [xd.clone() for _ in range(n_aux)], [hip.empty(in_b, np.int8) for _ in range(n_aux)]
+    aux_cold = [lambda i=i: hip.quantize(xds[i], capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq2[i])
+                for i in range(n_aux)]
+    return dict(name="c1s%d" % stride, step=step, dom_fn_cold=dom_cold, ops=2.0 * N * C * 9 * oh * ow, launches=2,
                 bytes=5 * in_b + in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=in_b + out_b, bound="hbm",
                 workload="depthwise int8 3x3 s%d p1, 8x256x112x112 fp32 in -> quantize -> conv+bias+ReLU6+requantize "
                          "-> int8" % stride,
                 dom_kernel="depthwise 3x3 s%d + requantize (int8 in -> int8 out)" % stride,
                 dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out),
-                aux=dict(kernel="quantize fp32 Float8 -> Byte8", bytes=5 * in_b,
+                aux=dict(kernel="quantize fp32 Float8 -> Byte8", bytes=5 * in_b, fn_cold=aux_cold,
                          fn=lambda: hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8,
                                                  dst=xq)),
                 x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
                 shape=(N, C, H, W), stride=stride)
 
 
-def build_c2(hip, capi, rng):
-    """configs[2]: 1x1 conv 256->512 on 32x256x28x28 (GEMM M=512, N=25088, K=256), bias, dequantize+ReLU, fp32."""
+def build_c2(hip, capi, rng, int8_out=False):
+    """configs[2]: 1x1 conv 256->512 on 32x256x28x28 (GEMM M=512, N=25088, K=256), bias, dequantize+ReLU, fp32.
+    int8_out: the same layer requantizing to int8 (a fixed output scale), which takes the fp32 result off the bus."""
     N, C, K, H, W = 32, 256, 512, 28, 28
     x = rng.uniform(0, 1, (N, C, H, W)).astype(np.float32)
     wq, ws = quantize_weights(rng.normal(0, 0.03, (K, C, 1, 1)).astype(np.float32))
     bias = rng.normal(0, 0.01, K).astype(np.float32)
     in_scale = np.float32(127) / np.abs(x).max()
-    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale), act=1,
-                    out_kind=capi.OUT_F32)
+    out_scale = np.float32(20.0)
+    if int8_out:
+        conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale), act=1,
+                        out_scale=[out_scale], out_kind=capi.OUT_I8, out_round=capi.ROUND_SSE)
+    else:
+        conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale), act=1,
+                        out_kind=capi.OUT_F32)
+    out_layout, out_dt, out_esz = (capi.I8_P8, np.int8, 1) if int8_out else (capi.F32_P4, np.float32, 4)
     xd = hip.to_device(capi.pack_np(x, 8))
     xq = hip.empty(N * C * H * W, np.int8)
-    out = hip.empty(N * K * H * W, np.float32)
+    out = hip.empty(N * K * H * W, out_dt)
     scale_dev = hip.to_device(np.array([in_scale], np.float32))
 
     def step():
         hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
-        conv.forward(xq, capi.I8_P8, N, H, W, capi.F32_P4, out=out)
+        conv.forward(xq, capi.I8_P8, N, H, W, out_layout, out=out)
         return out
 
+    step()
+    dom_bytes = N * C * H * W + K * C + out_esz * N * K * H * W
+    n_dom = cold_sets(dom_bytes)
+    xqs, outs = [xq.clone() for _ in range(n_dom)], [hip.empty(N * K * H * W, out_dt) for _ in range(n_dom)]
+    dom_cold = [lambda i=i: conv.forward(xqs[i], capi.I8_P8, N, H, W, out_layout, out=outs[i]) for i in range(n_dom)]
     ops = 2.0 * N * K * C * H * W
-    return dict(name="c2", step=step, ops=ops, launches=2, dom_ops=ops,
-                dom_bytes=N * C * H * W + K * C + 4 * N * K * H * W, bound="hbm",
+    tail = "requantize + ReLU -> int8" if int8_out else "dequantize + ReLU -> fp32"
+    return dict(name="c2i8" if int8_out else "c2", step=step, ops=ops, launches=2, dom_ops=ops, dom_fn_cold=dom_cold,
+                dom_bytes=dom_bytes, bound="hbm",
                 workload="int8 1x1 conv 256->512 @28x28 batch 32 (GEMM 512x25088x256), fp32 in -> quantize -> conv + "
-                         "bias + dequantize + ReLU -> fp32",
-                dom_kernel="conv 1x1 256->512 (MFMA implicit GEMM, fp32 out)",
-                dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.F32_P4, out=out),
-                x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale))], shape=(N, C, H, W))
+                         "bias + " + tail,
+                dom_kernel="conv 1x1 256->512 (MFMA implicit GEMM, %s out)" % ("int8" if int8_out else "fp32"),
+                dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, out_layout, out=out),
+                x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
+                shape=(N, C, H, W), int8_out=int8_out)
 
 
-def build_c0(hip, capi, rng):
-    """configs[0]: one 3x3 s1 p1 conv 64->64 on 1x64x56x56 fp32, no bias, dequantize to fp32."""
-    N, C, K, H, W = 1, 64, 64, 56, 56
+def build_c0(hip, capi, rng, batch=1):
+    """configs[0]: one 3x3 s1 p1 conv 64->64 on 1x64x56x56 fp32, no bias, dequantize to fp32 (batch 64: the same layer
+    with enough work to fill the chip)."""
+    N, C, K, H, W = batch, 64, 64, 56, 56
     x = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
     wq, ws = quantize_weights(rng.normal(0, 0.05, (K, C, 3, 3)).astype(np.float32))
     in_scale = np.float32(127) / np.abs(x).max()
@@ -202,6 +245,22 @@ def build_c0(hip, capi, rng):
         return out
 
     ops = 2.0 * N * K * C * 9 * H * W
+    if batch > 1:
+        # the convolution alone on the quantized blob; 64 fp32 bytes out per int8 pixel in: bound by the writes
+        step()
+        xq = hip.empty(N * C * H * W, np.int8)
+        scale_dev = hip.to_device(np.array([in_scale], np.float32))
+        hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
+        dom_bytes = N * C * H * W + K * C * 9 + 4 * N * K * H * W
+        n_dom = cold_sets(dom_bytes)
+        xqs, outs = [xq.clone() for _ in range(n_dom)], [hip.empty(N * K * H * W, np.float32) for _ in range(n_dom)]
+        return dict(name="c0n%d" % batch, step=step, ops=ops, launches=2, dom_ops=ops, dom_bytes=dom_bytes, bound="hbm",
+                    workload="int8 3x3 conv 64->64 s1 p1, %dx64x56x56 fp32 in -> quantize -> conv -> fp32 out" % batch,
+                    dom_kernel="conv 3x3 64->64 (MFMA, LDS halo, fp32 out)",
+                    dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.F32_P4, out=out),
+                    dom_fn_cold=[lambda i=i: conv.forward(xqs[i], capi.I8_P8, N, H, W, capi.F32_P4, out=outs[i])
+                                 for i in range(n_dom)],
+                    x=x, params=[dict(wq=wq, ws=ws, bias=None, in_scale=float(in_scale))], shape=(N, C, H, W))
     return dict(name="c0", step=step, ops=ops, launches=2, dom_ops=ops,
                 dom_bytes=N * C * H * W + K * C * 9 + 4 * N * K * H * W, bound="mfma",
                 workload="single int8 3x3 conv 64->64 s1 p1, 1x64x56x56 fp32 in -> fp32 out (latency-bound)",
@@ -269,7 +328,25 @@ def build_copy(hip, capi, rng):
 # CPU baseline: the reference itself (oracle/_ref, kind "reference") or the C restatement (kind "port")
 # ------------------------------------------------------------------------------------------------------
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(wl, budget_s=15.0):
+    r = _cpu_baseline(wl, budget_s)
+    if isinstance(r, dict) and "cpu" not in r:
+        r["cpu"] = cpu_model()
+    return r
+
+
+def _cpu_baseline(wl, budget_s=15.0):
     from oracle import binding
     name = wl["name"]
     p = wl["params"]
@@ -344,17 +421,20 @@ def cpu_baseline(wl, budget_s=15.0):
         if r.returncode != 0:
             raise RuntimeError("c4 CPU child failed (%d): %s" % (r.returncode, r.stderr[-200:]))
         return json.loads(r.stdout.strip().splitlines()[-1])
-    if name in ("c2", "c0"):
+    if name in ("c2", "c0", "c2i8") or name.startswith("c0n"):
         n_img = min(4, N)
         K = p[0]["wq"].shape[0]
         k = p[0]["wq"].shape[2]
         ops = 2.0 * n_img * K * C * k * k * H * W
         if R is not None:
+            int8_out = bool(wl.get("int8_out"))
             opts = {"type": "Convolution", "in_channels": C, "out_channels": K, "kernel": k, "stride": 1,
-                    "padding": k // 2, "int8_scale_term": 2, "bias_term": "true" if p[0]["bias"] is not None else "false"}
-            if name == "c2":
+                    "padding": k // 2, "int8_scale_term": 102 if int8_out else 2,
+                    "bias_term": "true" if p[0]["bias"] is not None else "false"}
+            if name.startswith("c2"):
                 opts["activation"] = "Relu"
-            L = R.conv_layer(opts, (1, C, H, W), p[0]["wq"], p[0]["bias"], p[0]["ws"], p[0]["in_scale"], 1.0, True)
+            L = R.conv_layer(opts, (1, C, H, W), p[0]["wq"], p[0]["bias"], p[0]["ws"], p[0]["in_scale"],
+                             p[0].get("out_scale", 1.0), True)
             _, t = L.forward(x[:n_img], repeat=5, want_out=False)
             L.close()
             return dict(value=ops / t / 1e12, unit="TOPS", cores=R.num_threads(), kind="reference",
@@ -445,6 +525,12 @@ def measure(wl, timer, steps, warmup, unit_main):
         kms, _ = timer.run(wl["dom_fn"], max(steps * 4, 50), 5)
     else:
         kms = ms
+    # a bandwidth-bound kernel is priced on a loop that rotates over buffer sets larger than the last-level cache;
+    # the figure of the loop over ONE set (operands still cached from the previous launch) is reported beside it
+    kms_resident = None
+    if wl.get("dom_fn_cold"):
+        kms_resident = kms
+        kms, _ = timer.run(wl["dom_fn_cold"], max(steps * 4, 50), 2 * len(wl["dom_fn_cold"]))
     if wl["bound"] == "mfma":
         ach = wl["dom_ops"] / (kms * 1e-3) / 1e12
         res["roofline"] = dict(bound="mfma", achieved=ach, peak=PEAK_INT8_TOPS, unit="TOP/s", frac=ach / PEAK_INT8_TOPS,
@@ -454,10 +540,22 @@ def measure(wl, timer, steps, warmup, unit_main):
         res["roofline"] = dict(bound="hbm", achieved=ach, peak=PEAK_HBM_GBS, unit="GB/s", frac=ach / PEAK_HBM_GBS,
                                traffic=measured_traffic(wl["name"]), kernel=wl["dom_kernel"], kernel_ms=kms)
         res["roofline"]["tops"] = wl["dom_ops"] / (kms * 1e-3) / 1e12
+        if kms_resident is not None:
+            res["roofline"]["working_set"] = "%d buffer sets in turn, %d MB per loop" % (
+                len(wl["dom_fn_cold"]), len(wl["dom_fn_cold"]) * wl["dom_bytes"] >> 20)
+            res["roofline_resident"] = dict(kernel_ms=kms_resident, achieved=wl["dom_bytes"] / (kms_resident * 1e-3) / 1e9,
+                                            frac=wl["dom_bytes"] / (kms_resident * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                            working_set="one buffer set, %d MB (cache-resident)" % (wl["dom_bytes"] >> 20))
     if "aux" in wl:
-        ams, _ = timer.run(wl["aux"]["fn"], max(steps * 4, 50), 5)
-        res["aux_kernel"] = dict(kernel=wl["aux"]["kernel"], kernel_ms=ams, gbs=wl["aux"]["bytes"] / (ams * 1e-3) / 1e9,
-                                 frac_hbm=wl["aux"]["bytes"] / (ams * 1e-3) / 1e9 / PEAK_HBM_GBS)
+        aux = wl["aux"]
+        ams_res, _ = timer.run(aux["fn"], max(steps * 4, 50), 5)
+        ams = ams_res
+        if aux.get("fn_cold"):
+            ams, _ = timer.run(aux["fn_cold"], max(steps * 4, 50), 2 * len(aux["fn_cold"]))
+        res["aux_kernel"] = dict(kernel=aux["kernel"], kernel_ms=ams, gbs=aux["bytes"] / (ams * 1e-3) / 1e9,
+                                 frac_hbm=aux["bytes"] / (ams * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                 resident_kernel_ms=ams_res,
+                                 resident_frac_hbm=aux["bytes"] / (ams_res * 1e-3) / 1e9 / PEAK_HBM_GBS)
     return res
 
 
@@ -490,7 +588,8 @@ def main():
     timer = Timer(hip.torch)
     builders = {"c3": lambda r: build_c3(hip, capi, r), "c1s1": lambda r: build_c1(hip, capi, r, 1),
                 "c1s2": lambda r: build_c1(hip, capi, r, 2), "c2": lambda r: build_c2(hip, capi, r),
-                "c0": lambda r: build_c0(hip, capi, r), "copy": lambda r: build_copy(hip, capi, r)}
+                "c0": lambda r: build_c0(hip, capi, r), "copy": lambda r: build_copy(hip, capi, r),
+                "c2i8": lambda r: build_c2(hip, capi, r, int8_out=True), "c0n64": lambda r: build_c0(hip, capi, r, batch=64)}
     try:
         from tensor_amd import mobilenet  # noqa: F401
         builders["c4"] = lambda r: mobilenet.build_bench(hip, capi, r)
@@ -503,6 +602,17 @@ def main():
 
     wl = builders[a.workload](np.random.default_rng(0))
     unit = "images/s" if wl["name"] in ("c4", "det") else ("GB/s" if "bytes" in wl else "TOPS")
+    no_settle = None
+    if wl["name"] == "c3":
+        # the same measurement without the run-in, after an idle second (the clock at rest): reported beside the line
+        hip.torch.cuda.synchronize()
+        time.sleep(1.0)
+        ms0, _ = timer.run(wl["step"], a.steps, a.warmup, settle=0.0)
+        time.sleep(1.0)
+        k0, _ = timer.run(wl["dom_fn"], max(a.steps * 4, 50), 5, settle=0.0)
+        no_settle = dict(ms_per_step=ms0, tops=wl["ops"] / (ms0 * 1e-3) / 1e12, kernel_ms=k0,
+                         frac=wl["dom_ops"] / (k0 * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+                         note="same loops with settle_s = 0, each after one idle second")
     res = measure(wl, timer, a.steps, a.warmup, unit)
     if wl["name"] == "c4":
         value = wl["images"] / (res["ms_per_step"] * 1e-3)
@@ -526,6 +636,10 @@ def main():
             "roofline": res["roofline"], "wall_ms_per_step": res["wall_ms_per_step"]}
     if "aux_kernel" in res:
         line["aux_kernel"] = res["aux_kernel"]
+    if "roofline_resident" in res:
+        line["roofline_resident"] = res["roofline_resident"]
+    if no_settle is not None:
+        line["no_settle"] = no_settle
     if not a.no_cpu:
         try:
             line["cpu_baseline"] = cpu_baseline(wl)
@@ -533,7 +647,7 @@ def main():
             line["cpu_baseline"] = {"error": str(e)[:200]}
     if not a.no_also:
         also = []
-        for name in ("c1s1", "c1s2", "c2", "c0", "c4", "det"):
+        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det"):
             if name == a.workload or name not in builders:
                 continue
             w2 = builders[name](np.random.default_rng(0))
@@ -541,7 +655,7 @@ def main():
             entry = dict(name=name, **r2)
             if name in ("c4", "det"):
                 entry["images_per_s"] = w2["images"] / (r2["ms_per_step"] * 1e-3)
-            if not a.no_cpu and name != "c4":
+            if not a.no_cpu:
                 try:
                     entry["cpu_baseline"] = cpu_baseline(w2)
                 except Exception as e:

@@ -16,6 +16,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(HERE, "libotter_int8_oracle.so")
 REF_SO = os.path.join(HERE, "_ref", "libotter_ref.so")
+# the same reference plus the reference-side binding of the GPU library (oracle/ref_hip_layer.cpp)
+REF_HIP_SO = os.path.join(HERE, "_ref", "libotter_ref_hip.so")
 
 ROUND_SSE, ROUND_EXACT = 0, 1
 
@@ -197,11 +199,18 @@ def ref_available():
     return os.path.exists(REF_SO)
 
 
-class Ref:
-    """The compiled reference. Raises OSError if oracle/_ref/libotter_ref.so is absent or cannot load."""
+def ref_hip_available():
+    return os.path.exists(REF_HIP_SO)
 
-    def __init__(self):
-        L = self.lib = C.CDLL(REF_SO)
+
+class Ref:
+    """The compiled reference. Raises OSError if oracle/_ref/libotter_ref.so is absent or cannot load.
+    hip=True: the build that also holds the GPU convolution layer written against the reference's headers
+    (use_hip_convolution switches the reference's layer registry to it and back)."""
+
+    def __init__(self, hip=False):
+        L = self.lib = C.CDLL(REF_HIP_SO if hip else REF_SO)
+        self.hip = hip
         L.otter_ref_last_error.restype = C.c_char_p
         L.otter_ref_conv_layer_create.restype = C.c_void_p
         L.otter_ref_conv_layer_forward.restype = C.c_double
@@ -213,6 +222,19 @@ class Ref:
 
     def num_threads(self):
         return self.lib.otter_ref_num_threads()
+
+    def use_hip_convolution(self, on):
+        """Registers the GPU layer under "Convolution" in the reference's LayerRegistry (nets opened afterwards get
+        it), or restores the stock creator."""
+        assert self.hip
+        rc = self.lib.otter_ref_use_hip_convolution(C.c_int(int(on)))
+        if rc != 0:
+            self.lib.otter_ref_hip_last_error.restype = C.c_char_p
+            raise RuntimeError("GPU layer: " + self.lib.otter_ref_hip_last_error().decode(errors="replace"))
+
+    def hip_forward_count(self):
+        self.lib.otter_ref_hip_forward_count.restype = C.c_long
+        return self.lib.otter_ref_hip_forward_count()
 
     def set_num_threads(self, n):
         self.lib.otter_ref_set_num_threads(C.c_int(n))

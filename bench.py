@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 convolution path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c2i8|c0|c0n64|c4|det] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c2i8|c0|c0n64|c4|det|dil2|grp8|s2|odd55] [--no-cpu] [--no-also]
 
 Prints ONE JSON line. The headline workload is the fourth benchmark configuration (the MFMA-bound case the metric's
 "int8 conv TOPS (% MFMA peak)" is quoted on): four chained int8-in/int8-out 3x3 convolutions 128->128 at
@@ -269,6 +269,44 @@ def build_c0(hip, capi, rng, batch=1):
                 shape=(N, C, H, W))
 
 
+LAYER_SHAPES = {
+    # name: (C, K, kernel, stride, pad, dilation, groups, N, H, W, what)
+    "dil2": (128, 128, 3, 1, 2, 2, 1, 64, 56, 56, "dilated (2) 3x3 128->128"),
+    "grp8": (256, 256, 3, 1, 1, 1, 8, 64, 28, 28, "grouped (8 groups of 32->32) 3x3 256->256"),
+    "s2": (128, 128, 3, 2, 1, 1, 1, 64, 56, 56, "3x3 stride 2 128->128"),
+    "odd55": (128, 128, 3, 1, 1, 1, 1, 64, 55, 55, "3x3 128->128 on an odd image width"),
+}
+
+
+def build_layer(hip, capi, rng, name):
+    """One int8-in / int8-out convolution layer (bias, ReLU, requantize) of a shape outside the tuned benchmark
+    configurations: the variants of the path (dilation, groups, stride 2, odd widths)."""
+    C, K, k, s, p, d, g, N, H, W, what = LAYER_SHAPES[name]
+    x = rng.integers(-127, 128, size=(N, C, H, W), dtype=np.int8)
+    wq, ws = quantize_weights(rng.normal(0, 0.04, (K, C // g, k, k)).astype(np.float32))
+    bias = rng.normal(0, 0.01, K).astype(np.float32)
+    conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, np.float32(127.0)), bias=bias, out_scale=[np.float32(40.0)],
+                    stride=(s, s), pad=(p, p), dil=(d, d), groups=g, act=1, out_kind=capi.OUT_I8, out_round=capi.ROUND_SSE)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    oh, ow = conv.out_hw(H, W)
+    out = hip.empty(N * K * oh * ow, np.int8)
+
+    def step():
+        conv.forward(xd, capi.I8_P8, N, H, W, capi.I8_P8, out=out)
+        return out
+
+    ops = 2.0 * N * K * (C // g) * k * k * oh * ow
+    nbytes = N * C * H * W + N * K * oh * ow + K * (C // g) * k * k
+    kind = conv.kernel_kind(capi.I8_P8, N, H, W, capi.I8_P8)
+    bound = "mfma" if ops / nbytes > PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9) else "hbm"
+    return dict(name=name, step=step, ops=ops, launches=1, dom_ops=ops, dom_bytes=nbytes, bound=bound,
+                workload="int8 %s s%d p%d @%dx%d, batch %d, int8 in/out, requantize+ReLU (kernel family %d)"
+                         % (what, s, p, H, W, N, kind),
+                dom_kernel="the layer's one launch", dom_fn=None, x=x,
+                params=[dict(wq=wq, ws=ws, bias=bias, in_scale=127.0, out_scale=40.0)], shape=(N, C, H, W),
+                layer=(C, K, k, s, p, d, g))
+
+
 def build_det(hip, capi, rng, batch=16):
     """The reference's own int8 detection model description (benchmark/nanodet-plus-m-1.5x_416_int8_fused.otter, a data
     file kept under tests/golden) read by Net::load_otter, with synthetic int8 weights written as an ncnn .bin and read by
@@ -421,6 +459,27 @@ def _cpu_baseline(wl, budget_s=15.0):
         if r.returncode != 0:
             raise RuntimeError("c4 CPU child failed (%d): %s" % (r.returncode, r.stderr[-200:]))
         return json.loads(r.stdout.strip().splitlines()[-1])
+    if name in LAYER_SHAPES:
+        Cc, K, k, st, pd, dl, gr = wl["layer"]
+        if R is None or gr > 1:
+            # (the compiled reference's packed int8 path stops on an assertion for a grouped, non-depthwise layer:
+            # Tensor/ExpandUtils.cpp:75 under Tensor/Convolution.cpp:396-408; the C restatement stands in)
+            O = binding.Oracle()
+            t0 = time.perf_counter()
+            O.conv_layer_forward(x[:1], p[0]["wq"], p[0]["ws"], p[0]["in_scale"], stride=(st, st), pad=(pd, pd),
+                                 dil=(dl, dl), groups=gr, bias=p[0]["bias"], top_scale=p[0]["out_scale"], int8_out=True,
+                                 act_type=1)
+            t = time.perf_counter() - t0
+            return dict(value=wl["ops"] / N / t / 1e12, unit="TOPS", cores=O.num_threads(), kind="port",
+                        sample="1 image, C restatement of the layer")
+        n_img = 4
+        opts = {"type": "Convolution", "in_channels": Cc, "out_channels": K, "kernel": k, "stride": st, "padding": pd,
+                "dilation": dl, "groups": gr, "int8_scale_term": 102, "activation": "Relu"}
+        L = R.conv_layer(opts, (1, Cc, H, W), p[0]["wq"], p[0]["bias"], p[0]["ws"], p[0]["in_scale"], p[0]["out_scale"], True)
+        _, t = L.forward(x[:n_img], repeat=5, want_out=False)
+        L.close()
+        return dict(value=wl["ops"] * n_img / N / t / 1e12, unit="TOPS", cores=R.num_threads(), kind="reference",
+                    sample="%d images, reference layer forward, min of 5" % n_img)
     if name in ("c2", "c0", "c2i8") or name.startswith("c0n"):
         n_img = min(4, N)
         K = p[0]["wq"].shape[0]
@@ -596,6 +655,8 @@ def main():
     except ImportError:
         pass
     builders["det"] = lambda r: build_det(hip, capi, r)
+    for lname in LAYER_SHAPES:
+        builders[lname] = lambda r, lname=lname: build_layer(hip, capi, r, lname)
     if a.workload not in builders:
         print("unknown workload %s (have %s)" % (a.workload, sorted(builders)), file=sys.stderr)
         sys.exit(2)
@@ -647,7 +708,7 @@ def main():
             line["cpu_baseline"] = {"error": str(e)[:200]}
     if not a.no_also:
         also = []
-        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det"):
+        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det") + tuple(LAYER_SHAPES):
             if name == a.workload or name not in builders:
                 continue
             w2 = builders[name](np.random.default_rng(0))

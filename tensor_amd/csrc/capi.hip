@@ -218,7 +218,8 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
     h->d = d;
     const int K = d.out_channels, C = d.in_channels, g = d.groups, maxk = d.kernel_h * d.kernel_w;
     h->depthwise = (C == g && g == K);
-    const int kpad = igemm_padded_rows(K);  // the kernels read the per-channel arrays up to the padded row count
+    // the kernels read the per-channel arrays up to the padded row count (of the last group, for a grouped layer)
+    const int kpad = g > 1 ? K + 128 : igemm_padded_rows(K);
     int rc = OTTER_HIP_OK;
     do {
         const size_t wcount = (size_t)K * (C / g) * maxk;
@@ -235,7 +236,17 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             if ((rc = upload<float>(&h->scale_out, so.data(), K, kpad, 1.f))) break;
         }
         if ((rc = upload<float>(&h->in_scale, &in_scale, 1, 1, 0.f))) break;
-        if (h->depthwise && C % 8 == 0) {
+        if (h->depthwise && C % 8) {
+            // depthwise on a channel count that is not whole octets: the channels are zero-padded to the next octet on the
+            // way in (weights of the padding channels are zero, their results are never stored)
+            const int cp = (C + 7) / 8 * 8;
+            std::vector<int8_t> wpad((size_t)cp * maxk, 0);
+            std::memcpy(wpad.data(), weight, (size_t)C * maxk);
+            std::vector<int32_t> wm(dw_packed_weight_bytes(cp, d.kernel_h, d.kernel_w) / sizeof(int32_t));
+            dw_pack_weights(wpad.data(), cp, d.kernel_h, d.kernel_w, wm.data());
+            if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
+            h->c_pad = cp;
+        } else if (h->depthwise) {
             std::vector<int32_t> wm(dw_packed_weight_bytes(C, d.kernel_h, d.kernel_w) / sizeof(int32_t));
             dw_pack_weights(weight, C, d.kernel_h, d.kernel_w, wm.data());
             if ((rc = upload<int32_t>(&h->w_dw, wm.data(), wm.size(), wm.size(), 0))) break;
@@ -248,6 +259,11 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
         } else if (g == 1 && C % 8 == 0) {
             std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
             igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
+            if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
+        } else if (g > 1 && !h->depthwise && (C / g) % 8 == 0) {
+            // grouped: every group's weights packed by itself (one launch, a group per grid.z slice)
+            std::vector<int8_t> wp(igemm_grouped_weight_bytes(K, C, g, d.kernel_h, d.kernel_w));
+            igemm_pack_weights_grouped(weight, K, C, g, d.kernel_h, d.kernel_w, wp.data());
             if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
         } else if (g == 1) {
             // C % 8 != 0 (e.g. an RGB stem): zero-pad the input channels to the next octet, weights included
@@ -347,6 +363,7 @@ static bool use_stem(const otter_hip_conv* h, int in_layout, const ConvGeom& g_i
 static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g, const Epilogue& ep) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
+        if (h->w_igemm && g.groups > 1) return igemm_grouped_applicable(g, ep) ? 1 : 0;  // else the scalar catch-all
         if (h->w_igemm) {
             if (h->force_tm > 0 || h->force_tm == -4) return 1;  // forced generic kernel (-4: with automatic tiles)
             if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g, ep)) return 3;
@@ -453,7 +470,7 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
 
     Epilogue ep = make_epilogue(h, out_layout);
     const int kind = pick_kernel(h, q_layout, g, ep);
-    if ((twin || residual) && kind == 1 && (!twin || g.K % 8 == 0) && pick_epilogue(ep, g.K) == EPI_F32_P4) {
+    if ((twin || residual) && kind == 1 && g.groups == 1 && (!twin || g.K % 8 == 0) && pick_epilogue(ep, g.K) == EPI_F32_P4) {
         ep.twin = twin, ep.twin_scale = twin_scale;
         ep.twin_half = twin_round == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
         ep.residual = residual;

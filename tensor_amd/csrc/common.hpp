@@ -154,6 +154,9 @@ struct ConvGeom {
     int K, OH, OW;         // output
     int kh, kw, sh, sw, ph, pw, dh, dw;
     int groups;
+    // channels per image of the tensors in memory, when the kernel works on a channel slice of them (one group of a
+    // grouped convolution: C, K are the group's, Cs, Ks the tensors'); 0 = the same as C / K
+    int Cs = 0, Ks = 0;
 };
 
 // ---------------------------------------------------------------------------------------------------

@@ -16,7 +16,9 @@
 //   * the MFMA "A" operand (weights) is read straight from global memory, already in MFMA lane order
 //     (igemm_pack_weights), one coalesced 1 KB read per 16x64 fragment, prefetched two k-chunks ahead. Every
 //     workgroup reads the same <= 147 KB of weights, so they stay in L2.
-// The image width must be even (a lane moves an aligned pixel pair) and the input below 2 GiB (32-bit offsets).
+// An odd image width ends on half a pixel pair: the transfer then brings the first pixel of the next row along, and the
+// wave that issued it overwrites that pixel with zeros once its transfers have landed, before the barrier.
+// The input must stay below 2 GiB (32-bit offsets).
 #include "common.hpp"
 #include "conv_igemm.hpp"
 
@@ -78,7 +80,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
             // 512-byte lines: one instruction moves a row of BOTH octets of a pair (adjacent lines in LDS): lanes 0-31
             // the first octet, lanes 32-63 the second, 16 bytes = pixels 2*pp-2 and 2*pp-1 each
             const int hl = lane >> 5, pp = lane & 31;
-            const bool col_ok = pp >= 1 && 2 * pp - 1 < g.W;
+            const bool col_ok = pp >= 1 && 2 * pp - 2 < g.W;  // (an odd width: the last pair is half padding, see fix_odd)
             const unsigned v_px = (unsigned)(2 * pp - 2) * 8u;
             const unsigned v_both = col_ok ? v_px + (unsigned)hl * (unsigned)(g.H * g.W * 8) : HALO_OOB;
             const unsigned v_first = (col_ok && hl == 0) ? v_px : HALO_OOB;  // an odd octet count ends on half a pair
@@ -98,7 +100,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                 }
             }
         } else {
-            const bool col_ok = lane >= 1 && 2 * lane - 1 < g.W;  // lane: pixels 2*lane-2 and 2*lane-1
+            const bool col_ok = lane >= 1 && 2 * lane - 2 < g.W;  // lane: pixels 2*lane-2 and 2*lane-1
             const unsigned v_col = col_ok ? (unsigned)(2 * lane - 2) * 8u : HALO_OOB;
             if (2 * lane < EW) {
                 for (int oc = wave; oc < cb / 8; oc += 4) {
@@ -113,6 +115,25 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                     }
                 }
             }
+        }
+    };
+
+    // Odd width: pixel W (the right zero column, LDS pixel index W + 2) of every line this wave staged holds the next
+    // row's first pixel; zero it. Runs after the wave's own transfers have landed and before the barrier, over exactly
+    // the (octet, row) lines the loops of stage() give this wave.
+    auto fix_odd = [&](int p0) {
+        if (!(g.W & 1)) return;
+        const int p_last = min(p0 + PT, OHW) - 1;
+        const int R = p_last / g.OW - p0 / g.OW + 3;
+        const int lines = (cb / 8) * R;  // (octet, row) lines of the stage
+        for (int i = lane; i < lines; i += 64) {
+            const int oc = i / R, r = i - oc * R;
+            // the wave that staged octet oc: pairs go round the four waves (512-byte lines, both octets of a pair in
+            // one transfer), or single octets do
+            const int owner = LOGP == 9 ? (oc >> 1) & 3 : oc & 3;
+            if (owner != wave) continue;
+            int8_t* line = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((2 * r + (oc & 1)) << LOGP);
+            *reinterpret_cast<v2i*>(line + (g.W + 2) * 8) = v2i{0, 0};
         }
     };
 
@@ -177,6 +198,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
             };
             // the halo transfers of this stage were issued one stage ago: wait for this wave's, then for everyone's
             __builtin_amdgcn_s_waitcnt(0);
+            fix_odd(p0);
             __syncthreads();
             load_a(0, 0, ring[0]);
             if constexpr (RD == 3) load_a(0, 1, ring[1]);
@@ -422,7 +444,7 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep) {
     if (!(g.kh == 3 && g.kw == 3 && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.groups == 1)) return false;
     if (g.ph > 1 || g.pw > 1 || g.C % 8) return false;
-    if ((g.W & 1) || (size_t)g.N * g.C * g.H * g.W >= ((size_t)1 << 31)) return false;  // pixel pairs, 32-bit offsets
+    if ((size_t)g.N * g.C * g.H * g.W >= ((size_t)1 << 31)) return false;  // 32-bit offsets
     if (pick_epilogue(ep, g.K) == EPI_GENERIC) return false;
     HaloPlan p;
     return plan_halo(g, 0, &p);

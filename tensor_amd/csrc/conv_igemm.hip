@@ -55,6 +55,20 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     }
     const int mt0 = blockIdx.y * (TM / 16);  // first 16-row tile of this workgroup
     const int OHW = g.OH * g.OW;
+    // Grouped convolution: blockIdx.z is the group, g.C / g.K are ONE group's channels and g.Cs / g.Ks the tensors'.
+    // A group is a channel slice of both tensors (whole octets in, whole output elements out), with its own block of
+    // packed weights and its own run of the per-channel constants.
+    const int Cs8 = (g.Cs ? g.Cs : g.C) / 8;
+    const int Ks = g.Ks ? g.Ks : g.K;
+    if (blockIdx.z) {
+        const int grp = blockIdx.z;
+        x += (size_t)grp * (g.C / 8) * g.H * g.W * 8;
+        wpk += (size_t)grp * (g.kh * g.kw * c_groups) * m_tiles16 * 1024;
+        out = (char*)out + (size_t)grp * g.K * OHW * (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG ? 1 : 4);
+        ep.scale_in += grp * g.K;
+        ep.bias += grp * g.K;
+        if (ep.scale_out) ep.scale_out += grp * g.K;
+    }
     // 32-bit pixel indices: the C ABI refuses tensors of 2^31 elements or more, and a 64-bit division costs ~4x
     const unsigned total_pix = (unsigned)g.N * (unsigned)OHW;
     const unsigned tile_base = (unsigned)pt * TN;
@@ -75,7 +89,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         const int oy = (int)((unsigned)pix / (unsigned)g.OW), ox = pix - oy * g.OW;
         iy0 = oy * g.sh - g.ph;
         ix0 = ox * g.sw - g.pw;
-        xn = x + (size_t)n * C8 * HW * 8;
+        xn = x + (size_t)n * Cs8 * HW * 8;
     }
 
     v2i breg[Cfg::B_V][2];
@@ -184,19 +198,19 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                 const int n = (int)nn, pix = (int)pp;
                 if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
                     epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
-                                                             elem_offset(8, n, ch0, pix, g.K, OHW), a8);
+                                                             elem_offset(8, n, ch0, pix, Ks, OHW), a8);
                 } else if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P4_FUSED) {
                     constexpr bool FUSED = EPI == EPI_F32_P4_FUSED;
                     ohip_v2i tw = {0, 0};
                     tw[0] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si, prm.bi,
-                                                         elem_offset(4, n, ch0, pix, g.K, OHW), a8[0], a8[1], a8[2], a8[3]);
+                                                         elem_offset(4, n, ch0, pix, Ks, OHW), a8[0], a8[1], a8[2], a8[3]);
                     if (ch0 + 4 < g.K)
                         tw[1] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si + 4, prm.bi + 4,
-                                                             elem_offset(4, n, ch0 + 4, pix, g.K, OHW), a8[4], a8[5], a8[6],
+                                                             elem_offset(4, n, ch0 + 4, pix, Ks, OHW), a8[4], a8[5], a8[6],
                                                              a8[7]);
                     if constexpr (FUSED)
                         if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
-                            *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, g.K, OHW)) = tw;
+                            *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, Ks, OHW)) = tw;
                 } else {
                     epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
                                             a8[6], a8[7]);
@@ -248,8 +262,9 @@ static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, 
     const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
     const int mpad = igemm_padded_rows(g.K);
     const int m_tiles = (mpad + TM - 1) / TM;
-    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI>), dim3(n_pix_tiles, m_tiles), dim3(256), 0, stream, x,
-                       wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
+    const int grid_z = g.Cs ? g.Cs / g.C : 1;  // groups of a grouped convolution
+    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI>), dim3(n_pix_tiles, m_tiles, grid_z), dim3(256), 0, stream,
+                       x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
     return hipGetLastError();
 }
 
@@ -300,8 +315,39 @@ void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
     *tn = TN;
 }
 
-hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+// A grouped (non-depthwise) convolution runs as one launch, a group per grid.z slice, when a group is whole octets of the
+// input and whole elements of the output and the fast epilogues apply to a group's channel count.
+bool igemm_grouped_applicable(const ConvGeom& g, const Epilogue& ep) {
+    if (g.groups <= 1 || g.C % g.groups || g.K % g.groups || g.groups > 65535) return false;
+    const int cg = g.C / g.groups, kg = g.K / g.groups;
+    if (cg % 8) return false;
+    const int epi = pick_epilogue(ep, kg);
+    if (epi == EPI_GENERIC) return false;
+    if (ep.twin != nullptr || ep.residual != nullptr) return false;
+    return (epi == EPI_F32_P4) ? kg % 4 == 0 : kg % 8 == 0;
+}
+
+size_t igemm_grouped_weight_bytes(int K, int C, int groups, int kh, int kw) {
+    return (size_t)groups * igemm_packed_weight_bytes(K / groups, C / groups, kh, kw);
+}
+
+// weight [K, C/groups, kh, kw]: every group's [K/groups, C/groups, kh, kw] block packed by itself, one after the other
+void igemm_pack_weights_grouped(const int8_t* w, int K, int C, int groups, int kh, int kw, int8_t* dst) {
+    const int kg = K / groups, cg = C / groups;
+    const size_t per = igemm_packed_weight_bytes(kg, cg, kh, kw);
+    for (int grp = 0; grp < groups; ++grp)
+        igemm_pack_weights(w + (size_t)grp * kg * cg * kh * kw, kg, cg, kh, kw, dst + grp * per);
+}
+
+hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g_in, const Epilogue& ep,
                           int tm, int tn, hipStream_t stream) {
+    ConvGeom g = g_in;
+    if (g.groups > 1) {  // one group's problem, the tensors' channel counts as strides
+        if (!igemm_grouped_applicable(g_in, ep)) return hipErrorInvalidValue;
+        g.Cs = g_in.C, g.Ks = g_in.K;
+        g.C = g_in.C / g_in.groups, g.K = g_in.K / g_in.groups;
+        g.groups = 1;
+    }
     if (tm == 0 || tn == 0) igemm_choose_tiles(g, &tm, &tn);
     // a row tile must not reach past the padded weight rows
     if (igemm_padded_rows(g.K) % tm != 0) return hipErrorInvalidValue;

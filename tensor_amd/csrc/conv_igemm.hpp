@@ -11,6 +11,9 @@ int igemm_row_channel(int row);
 size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw);
 void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst);
 void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn);
+bool igemm_grouped_applicable(const ConvGeom& g, const Epilogue& ep);
+size_t igemm_grouped_weight_bytes(int K, int C, int groups, int kh, int kw);
+void igemm_pack_weights_grouped(const int8_t* w, int K, int C, int groups, int kh, int kw, int8_t* dst);
 hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep, int tm,
                           int tn, hipStream_t stream);
 

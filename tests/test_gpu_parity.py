@@ -210,13 +210,15 @@ def test_igemm_every_tile_shape(hip, oracle, tile):
 
 @pytest.mark.parametrize("fn", [4, 5, 6, 7])
 def test_halo3x3_every_fragment_count(hip, oracle, fn):
-    """The 3x3 stride-1 LDS-halo MFMA kernel (even image widths): wide (K > 64) and narrow wave layouts, padded
-    channel counts, pad 0 and 1, ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at
-    once), both LDS line pitches (up to 60 columns and up to 124), several tiles per workgroup."""
+    """The 3x3 stride-1 LDS-halo MFMA kernel: wide (K > 64) and narrow wave layouts, padded channel counts, pad 0 and 1,
+    ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at once), both LDS line pitches
+    (up to 60 columns and up to 124), several tiles per workgroup, odd image widths (the last pixel pair of a row is
+    half padding: both pitches, the widest rows of either, the last row of the tensor, an odd octet count)."""
     rng = np.random.default_rng(fn)
     for (C, K, p, N, H, W) in [(128, 128, 1, 2, 19, 22), (64, 64, 1, 1, 56, 56), (72, 24, 0, 2, 11, 10),
                                (16, 160, 1, 1, 7, 8), (320, 96, 1, 1, 14, 30), (8, 16, 1, 1, 9, 66),
-                               (16, 136, 1, 3, 5, 124)]:
+                               (16, 136, 1, 3, 5, 124), (128, 128, 1, 2, 13, 55), (24, 64, 1, 3, 9, 59),
+                               (64, 40, 0, 1, 7, 123), (8, 32, 1, 2, 5, 7), (32, 96, 0, 1, 6, 61)]:
         x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
         in_scale = 25.0
         for int8_out in (True, False):
@@ -229,7 +231,7 @@ def test_halo3x3_every_fragment_count(hip, oracle, fn):
                 np.testing.assert_array_equal(out, want)
             else:
                 assert_f32_close(out, want)
-        # odd widths and raw accumulators take the generic implicit-GEMM kernel
+        # raw accumulators take the generic implicit-GEMM kernel
         acc, kind = run_conv(hip, oracle, x, wq, ws, in_scale, pad=p, out_kind=capi.OUT_I32, tile=(-1, fn))
         assert kind == 1
         np.testing.assert_array_equal(acc, acc_want)
@@ -258,8 +260,8 @@ def test_halo3x3_ragged_last_tile_then_full_tile_in_one_workgroup(hip, oracle):
     (8, 20, 3, 1, 1, 1, 1, 1, 9, 9),        # K % 8 != 0, K % 4 == 0 -> Int4 / Byte
     (8, 10, 3, 2, 1, 1, 1, 2, 9, 7),        # K % 4 != 0 -> unpacked outputs
     (32, 32, 3, 1, 2, 2, 1, 1, 11, 11),     # dilation
-    (16, 16, 3, 1, 1, 1, 2, 1, 8, 8),       # grouped, non-depthwise: scalar kernel
-    (6, 6, 3, 1, 1, 1, 6, 1, 8, 8),         # depthwise with C % 8 != 0: scalar kernel
+    (16, 16, 3, 1, 1, 1, 2, 1, 8, 8),       # grouped, non-depthwise: a group per grid slice of the implicit GEMM
+    (6, 6, 3, 1, 1, 1, 6, 1, 8, 8),         # depthwise with C % 8 != 0: channels zero-padded to an octet
     (12, 8, 3, 1, 1, 1, 1, 1, 8, 8),        # C % 8 != 0
     (64, 64, 3, 1, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s1, ragged strips
     (64, 64, 3, 2, 1, 1, 64, 2, 17, 13),    # depthwise 3x3 s2
@@ -356,6 +358,41 @@ def test_leaky_relu_fast_epilogues(hip, oracle, C, K, k, s, p, g, N, H, W, kind)
                                          int8_out=int8_out, act_type=2, act_params=[0.1])
         out, got_kind = run_conv(hip, oracle, x, wq, ws, 18.0, stride=s, pad=p, groups=g, bias=bias, top_scale=13.0,
                                  act=2, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        assert got_kind == kind
+        if int8_out:
+            np.testing.assert_array_equal(out, want)
+        else:
+            assert_f32_close(out, want)
+
+
+@pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,kind_i8,kind_f32", [
+    (16, 16, 3, 1, 1, 2, 2, 9, 11, 1, 1),       # two groups of 8 -> 8
+    (64, 128, 3, 1, 1, 4, 3, 14, 14, 1, 1),     # four groups of 16 -> 32
+    (32, 48, 1, 1, 0, 2, 2, 13, 7, 1, 1),       # pointwise, groups of 16 -> 24
+    (48, 24, 3, 2, 1, 3, 2, 15, 17, 1, 1),      # stride 2, three groups of 16 -> 8
+    (16, 8, 3, 1, 1, 2, 2, 8, 8, 0, 1),         # groups of 8 -> 4: whole Float4 elements, but half a Byte8 element
+    (24, 24, 3, 1, 1, 2, 1, 8, 8, 0, 0),        # groups of 12 channels: not whole octets -> the scalar catch-all
+    (6, 6, 3, 1, 1, 6, 2, 9, 10, 2, 2),         # depthwise, C % 8 != 0
+    (20, 20, 3, 2, 1, 20, 3, 13, 15, 2, 2),     # depthwise stride 2, C % 4 == 0
+    (12, 12, 5, 1, 2, 12, 2, 11, 11, 2, 2),     # depthwise 5x5
+])
+def test_grouped_and_odd_depthwise_routes(hip, oracle, C, K, k, s, p, g, N, H, W, kind_i8, kind_f32):
+    """Grouped non-depthwise convolutions (Tensor/Convolution.cpp:396-408: the reference slices the channels and runs
+    a convolution per group) run as one launch of the implicit-GEMM kernel with the group on grid.z when a group is
+    whole octets in and whole elements out; depthwise layers whose channel count is not a multiple of 8 run on the
+    depthwise kernels over a zero-padded octet. Accumulators, int8 and fp32 results against the oracle."""
+    rng = np.random.default_rng(C * 5 + K + k + s + g)
+    x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W)
+    in_scale = 23.0
+    want_acc = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), groups=g, bias=bias,
+                                         top_scale=12.0, int8_out=True, act_type=1, want_acc=True)[1]
+    acc, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, groups=g, out_kind=capi.OUT_I32)
+    np.testing.assert_array_equal(acc, want_acc)
+    for int8_out, act, kind in ((True, 1, kind_i8), (True, 0, kind_i8), (False, 3, kind_f32)):
+        want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), groups=g, bias=bias,
+                                         top_scale=12.0, int8_out=int8_out, act_type=act)
+        out, got_kind = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, groups=g, bias=bias, top_scale=12.0,
+                                 act=act, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
         assert got_kind == kind
         if int8_out:
             np.testing.assert_array_equal(out, want)

@@ -122,7 +122,7 @@ def build_c3(hip, capi, rng):
         in_scale = out_scale
     bufs = [hip.empty(N * C * H * W, np.int8) for _ in range(2)]
 
-    def step():
+    def step_layers():
         src = xd
         for l, conv in enumerate(layers):
             dst = bufs[l & 1]
@@ -130,12 +130,26 @@ def build_c3(hip, capi, rng):
             src = dst
         return src
 
+    # the chain through the entry point that takes consecutive layers at once (one persistent launch for this chain)
+    chain_ws = hip.empty(3 * N * C * H * W + 1024, np.int8)
+    chain_out = hip.empty(N * C * H * W, np.int8)
+
+    def step():
+        return hip.conv_chain(layers, xd, N, H, W, out=chain_out, workspace=chain_ws)
+
     ops_layer = 2.0 * N * C * C * 9 * H * W
-    return dict(name="c3", step=step, ops=L * ops_layer, launches=L, dom_ops=ops_layer,
+    launches = hip.conv_chain_launches(layers, N, H, W)
+    layer_fn = lambda: layers[1].forward(bufs[0], capi.I8_P8, N, H, W, capi.I8_P8, out=bufs[1])  # noqa: E731
+    # the dominant kernel is the chain's one launch (all four layers' operations); when the library runs the chain
+    # layer by layer it is one layer's launch
+    one = launches == 1
+    return dict(name="c3", step=step, step_layers=step_layers, layer_fn=layer_fn, ops=L * ops_layer, launches=launches,
+                dom_ops=L * ops_layer if one else ops_layer,
                 dom_bytes=2 * N * C * H * W + C * C * 9, bound="mfma",
                 workload="4 x int8 3x3 conv 128->128 s1 p1 @56x56, batch 64, int8 in/out, requantize+ReLU",
-                dom_kernel="conv 3x3 128->128 (MFMA implicit GEMM)",
-                dom_fn=lambda: layers[1].forward(bufs[0], capi.I8_P8, N, H, W, capi.I8_P8, out=bufs[1]),
+                dom_kernel="conv3x3_chain_kernel (the 4 layers in one persistent launch)" if one
+                else "conv 3x3 128->128 (MFMA implicit GEMM)",
+                dom_fn=step if one else layer_fn, layer_ops=ops_layer,
                 x=x, params=params, shape=(N, C, H, W))
 
 
@@ -674,6 +688,12 @@ def main():
         no_settle = dict(ms_per_step=ms0, tops=wl["ops"] / (ms0 * 1e-3) / 1e12, kernel_ms=k0,
                          frac=wl["dom_ops"] / (k0 * 1e-3) / 1e12 / PEAK_INT8_TOPS,
                          note="same loops with settle_s = 0, each after one idle second")
+        # the same four layers as four launches of the per-layer entry point, and one of those launches alone
+        msl, _ = timer.run(wl["step_layers"], a.steps, a.warmup)
+        kl, _ = timer.run(wl["layer_fn"], max(a.steps * 4, 50), 5)
+        layer_by_layer = dict(ms_per_step=msl, tops=wl["ops"] / (msl * 1e-3) / 1e12, launches_per_step=4,
+                              kernel="conv3x3_halo_kernel (one layer per launch)", kernel_ms=kl,
+                              frac=wl["layer_ops"] / (kl * 1e-3) / 1e12 / PEAK_INT8_TOPS)
     res = measure(wl, timer, a.steps, a.warmup, unit)
     if wl["name"] == "c4":
         value = wl["images"] / (res["ms_per_step"] * 1e-3)
@@ -701,6 +721,7 @@ def main():
         line["roofline_resident"] = res["roofline_resident"]
     if no_settle is not None:
         line["no_settle"] = no_settle
+        line["layer_by_layer"] = layer_by_layer
     if not a.no_cpu:
         try:
             line["cpu_baseline"] = cpu_baseline(wl)

@@ -172,6 +172,23 @@ int otter_hip_conv_forward_residual(const otter_hip_conv_t* handle, const void* 
                                     float q_scale, int q_round_mode, void* workspace, size_t workspace_bytes,
                                     void* stream);
 
+/* A chain of layers that each map an int8 Byte8 blob to an int8 Byte8 blob (consecutive Convolution layers of a
+ * Net, Tensor/Net.cpp:413-505 runs them one after the other): out = layer[n-1](... layer[0](in)). The result is what
+ * n calls of otter_hip_conv_forward give. The intermediate blobs live in `workspace`
+ * (otter_hip_conv_chain_workspace_bytes, one buffer per intermediate blob). Where all layers are the same 3x3
+ * stride-1 pad-1 geometry with 65..128 channels, the chain runs as ONE persistent launch in which a tile of a layer
+ * starts as soon as the tiles of the previous layer it reads are done; otherwise as n launches. The single launch
+ * waits on flags between workgroups; every wait is bounded, and otter_hip_conv_chain_status reports (after
+ * synchronizing the device) whether one ever gave up, in which case the outputs of the chain calls since the last
+ * status call are not valid. */
+size_t otter_hip_conv_chain_workspace_bytes(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);
+int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_layers, const void* in, int n, int in_h,
+                                 int in_w, void* out, void* workspace, size_t workspace_bytes, void* stream);
+int otter_hip_conv_chain_status(int* gave_up);
+/* For tests and profiling: the number of convolution launches otter_hip_conv_chain_forward makes for this chain and
+ * input (1: the single persistent launch; n_layers: layer by layer), or a negative status. */
+int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);
+
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
  * blob). For tests and profiling. */

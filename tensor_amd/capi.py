@@ -71,7 +71,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_channel_shuffle", "otter_hip_maxpool2d", "otter_hip_upsample2d", "otter_hip_shuffle2_split",
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
-           "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan"]
+           "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
+           "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches"]
 
 
 def load_cdll():
@@ -92,6 +93,7 @@ class Library:
         L = self.lib = load_cdll()
         L.otter_hip_last_error.restype = C.c_char_p
         L.otter_hip_conv_workspace_bytes.restype = C.c_size_t
+        L.otter_hip_conv_chain_workspace_bytes.restype = C.c_size_t
         self.device = torch.device("cuda", device)
         self._check(L.otter_hip_init(C.c_int(device)))
 
@@ -231,6 +233,34 @@ class Library:
 
     def conv(self, **kw):
         return Conv(self, **kw)
+
+    def conv_chain(self, convs, x, n, h, w, out=None, workspace=None):
+        """otter_hip_conv_chain_forward: x (int8 Byte8) through the layers `convs`, intermediate blobs in `workspace`."""
+        hs = (C.c_void_p * len(convs))(*[c.h for c in convs])
+        ws_bytes = self.lib.otter_hip_conv_chain_workspace_bytes(hs, len(convs), n, h, w)
+        if ws_bytes and workspace is None:
+            workspace = self.empty(ws_bytes, np.int8)
+        oh, ow = h, w
+        for c in convs:
+            oh, ow = c.out_hw(oh, ow)
+        if out is None:
+            out = self.empty(n * convs[-1].K * oh * ow, np.int8)
+        self._check(self.lib.otter_hip_conv_chain_forward(hs, len(convs), self.ptr(x), n, h, w, self.ptr(out),
+                                                          self.ptr(workspace) if workspace is not None else None,
+                                                          C.c_size_t(ws_bytes), self.stream()))
+        return out
+
+    def conv_chain_launches(self, convs, n, h, w):
+        hs = (C.c_void_p * len(convs))(*[c.h for c in convs])
+        r = self.lib.otter_hip_conv_chain_launches(hs, len(convs), n, h, w)
+        self._check(min(r, 0))
+        return r
+
+    def conv_chain_gave_up(self):
+        """otter_hip_conv_chain_status: synchronizes; True if a chain launch since the last call gave up a wait."""
+        v = C.c_int(0)
+        self._check(self.lib.otter_hip_conv_chain_status(C.byref(v)))
+        return bool(v.value)
 
 
 class Conv:

@@ -532,6 +532,129 @@ int otter_hip_conv_forward_static(const otter_hip_conv_t* h, const void* in, int
     return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, ws, need, stream, nullptr, 0.f, 0);
 }
 
+// ---- a chain of layers -------------------------------------------------------------------------------------------
+
+static int chain_check(const otter_hip_conv_t* const* hs, int layers, int n, int in_h, int in_w, const char* who) {
+    if (!hs || layers < 1) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": no layers");
+    for (int l = 0; l < layers; ++l) {
+        if (!hs[l]) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": null layer");
+        const otter_hip_conv_desc& d = hs[l]->d;
+        if (d.out_kind != OTTER_HIP_OUT_I8 || d.in_channels % 8 || d.out_channels % 8)
+            return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": every layer must map Byte8 to Byte8 (int8 output, channels in octets)");
+        if (l && d.in_channels != hs[l - 1]->d.out_channels)
+            return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": channel counts of consecutive layers do not match");
+    }
+    if (n < 0 || in_h < 1 || in_w < 1) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": bad shape");
+    return OTTER_HIP_OK;
+}
+
+// the blob sizes along the chain: bytes of the output of layer l (Byte8) into out_bytes[l]; returns false on an empty blob
+static bool chain_shapes(const otter_hip_conv_t* const* hs, int layers, int n, int h, int w, size_t* out_bytes, int* hh,
+                         int* ww) {
+    for (int l = 0; l < layers; ++l) {
+        hh[l] = h, ww[l] = w;
+        const otter_hip_conv_desc& d = hs[l]->d;
+        h = conv_out_size(h, d.kernel_h, d.stride_h, d.pad_h, d.dilation_h);
+        w = conv_out_size(w, d.kernel_w, d.stride_w, d.pad_w, d.dilation_w);
+        if (h < 1 || w < 1) return false;
+        out_bytes[l] = (size_t)n * d.out_channels * h * w;
+    }
+    return true;
+}
+
+// true when the chain runs as one persistent launch (conv3x3_chain.hip): every layer the same 3x3 stride-1 pad-1
+// geometry, same rounding and epilogue family
+static bool chain_single_launch(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {
+    if (n_layers < 2 || n_layers > 8 || n < 1) return false;
+    const otter_hip_conv_desc& d0 = handles[0]->d;
+    for (int l = 0; l < n_layers; ++l) {
+        const otter_hip_conv_desc& d = handles[l]->d;
+        const bool same = handles[l]->w_igemm && !handles[l]->c_pad && handles[l]->force_tm == 0 && d.in_channels == d0.in_channels &&
+                          d.out_channels == d0.out_channels && d.kernel_h == 3 && d.kernel_w == 3 && d.stride_h == 1 &&
+                          d.stride_w == 1 && d.pad_h == 1 && d.pad_w == 1 && d.dilation_h == 1 && d.dilation_w == 1 &&
+                          d.groups == 1 && d.out_round_mode == d0.out_round_mode && d.out_kind == OTTER_HIP_OUT_I8;
+        if (!same) return false;
+    }
+    const ConvGeom g = make_geom(d0, n, in_h, in_w);
+    const Epilogue ep0 = make_epilogue(handles[0], OTTER_HIP_I8_P8);
+    for (int l = 1; l < n_layers; ++l)
+        if (pick_epilogue(make_epilogue(handles[l], OTTER_HIP_I8_P8), g.K) != pick_epilogue(ep0, g.K)) return false;
+    int plan[4];
+    return g.OH > 0 && g.OW > 0 && conv3x3_chain_applicable(g, ep0, n_layers, plan);
+}
+
+int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {
+    int rc = chain_check(handles, n_layers, n, in_h, in_w, "otter_hip_conv_chain_launches");
+    if (rc) return rc;
+    return chain_single_launch(handles, n_layers, n, in_h, in_w) ? 1 : n_layers;
+}
+
+size_t otter_hip_conv_chain_workspace_bytes(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {
+    if (!handles || n_layers < 1 || n_layers > 64) return 0;
+    for (int l = 0; l < n_layers; ++l)
+        if (!handles[l]) return 0;
+    std::vector<size_t> ob(n_layers);
+    std::vector<int> hh(n_layers), ww(n_layers);
+    if (!chain_shapes(handles, n_layers, n, in_h, in_w, ob.data(), hh.data(), ww.data())) return 0;
+    size_t total = 0;
+    for (int l = 0; l + 1 < n_layers; ++l) total += (ob[l] + 255) / 256 * 256;  // one buffer per intermediate blob
+    return total;
+}
+
+int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_layers, const void* in, int n, int in_h,
+                                 int in_w, void* out, void* workspace, size_t workspace_bytes, void* stream_) {
+    if (!in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_forward: null");
+    if (n_layers > 64) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_forward: too many layers");
+    int rc = chain_check(handles, n_layers, n, in_h, in_w, "otter_hip_conv_chain_forward");
+    if (rc) return rc;
+    std::vector<size_t> ob(n_layers);
+    std::vector<int> hh(n_layers), ww(n_layers);
+    if (!chain_shapes(handles, n_layers, n, in_h, in_w, ob.data(), hh.data(), ww.data()))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_forward: empty output");
+    const size_t need = otter_hip_conv_chain_workspace_bytes(handles, n_layers, n, in_h, in_w);
+    if (need && (!workspace || workspace_bytes < need))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_forward: needs the workspace reported by "
+                                           "otter_hip_conv_chain_workspace_bytes");
+    if (n == 0) return OTTER_HIP_OK;
+    // the blobs: in, one workspace buffer per intermediate blob (each written once per call), out
+    std::vector<const int8_t*> act(n_layers + 1);
+    act[0] = (const int8_t*)in;
+    size_t ofs = 0;
+    for (int l = 0; l + 1 < n_layers; ++l) {
+        act[l + 1] = (const int8_t*)workspace + ofs;
+        ofs += (ob[l] + 255) / 256 * 256;
+    }
+    act[n_layers] = (const int8_t*)out;
+    hipStream_t stream = (hipStream_t)stream_;
+
+    // one launch for the whole chain where every layer is the same 3x3 "same" convolution geometry
+    if (chain_single_launch(handles, n_layers, n, in_h, in_w)) {
+        const ConvGeom g = make_geom(handles[0]->d, n, in_h, in_w);
+        std::vector<Epilogue> eps(n_layers);
+        std::vector<const int8_t*> wpk(n_layers);
+        for (int l = 0; l < n_layers; ++l) {
+            eps[l] = make_epilogue(handles[l], OTTER_HIP_I8_P8);
+            wpk[l] = handles[l]->w_igemm;
+        }
+        OHIP_CHECK(run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream));
+        return OTTER_HIP_OK;
+    }
+    // anything else: the layers one after the other, the same blobs
+    for (int l = 0; l < n_layers; ++l) {
+        rc = conv_forward(handles[l], act[l], OTTER_HIP_I8_P8, n, hh[l], ww[l], (void*)act[l + 1], OTTER_HIP_I8_P8, nullptr, 0,
+                          stream_, nullptr, 0.f, 0);
+        if (rc) return rc;
+    }
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_conv_chain_status(int* gave_up) {
+    if (!gave_up) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_status: null");
+    OHIP_CHECK(hipDeviceSynchronize());
+    OHIP_CHECK(conv3x3_chain_error(gave_up));
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_conv_forward_residual(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w,
                                     const float* residual, void* out, int out_layout, void* out_q, float q_scale,
                                     int q_round_mode, void* workspace, size_t workspace_bytes, void* stream) {

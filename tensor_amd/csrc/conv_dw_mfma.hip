@@ -132,10 +132,21 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
     constexpr int PH = 4 / S;              // output pixels per lane column
     constexpr int T = S == 1 ? 2 : 1;      // A sets
     const int C8 = g.C / 8;
-    const int o = blockIdx.y % C8;
-    const int n0 = (blockIdx.y / C8) * ipw;
-    const int chunk = blockIdx.x % col_chunks;
-    const int strip = __builtin_amdgcn_readfirstlane((blockIdx.x / col_chunks) * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    // Workgroups go to the 8 XCDs round-robin in launch order. Work items that share input cache lines - the column
+    // chunks of a row (a 128-byte line straddles the chunk border), the strip groups of a plane (halo rows), the
+    // octets of an image - get consecutive indices on ONE XCD, so that a shared line comes from memory once.
+    unsigned bx = blockIdx.x, by = blockIdx.y;
+    {
+        const unsigned id = by * gridDim.x + bx, total = gridDim.x * gridDim.y, per = total / 8;
+        if (id < per * 8) {
+            const unsigned w = (id % 8) * per + id / 8;
+            bx = w % gridDim.x, by = w / gridDim.x;
+        }
+    }
+    const int o = by % C8;
+    const int n0 = (by / C8) * ipw;
+    const int chunk = bx % col_chunks;
+    const int strip = __builtin_amdgcn_readfirstlane((bx / col_chunks) * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (strip >= n_strips) return;  // whole wave
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
     int di = 0, nl = chunk * 16 + n;  // image within the wave, lane column within the image

@@ -23,6 +23,12 @@ bool conv3x3_halo_plan(const ConvGeom& g, int force_fn, int plan[8]);
 hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                             int force_fn, hipStream_t stream);
 
+// conv3x3_chain.hip: a chain of same-shape 3x3 int8 -> int8 layers as one persistent launch
+bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers, int plan[4]);
+hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_t* const* wpk, const int8_t* const* act,
+                             int layers, int* error_word_out, hipStream_t stream);
+hipError_t conv3x3_chain_error(int* error_word);
+
 // conv_direct.hip
 hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void* out, const ConvGeom& g,
                            const Epilogue& ep, hipStream_t stream);

@@ -1,0 +1,111 @@
+"""otter_hip_conv_chain_forward: a chain of int8 -> int8 convolution layers. Where the layers are the same 3x3 "same"
+geometry the chain is one persistent launch whose workgroups hand tiles from layer to layer through flags; the result
+must be, bit for bit, what the layers give one by one (and what the oracle gives on sampled images), call after call,
+with no workgroup ever giving up a wait. Other chains run layer by layer behind the same entry point."""
+import numpy as np
+import pytest
+
+from tensor_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def quantize_weights(wf):
+    K = wf.shape[0]
+    ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
+    wq = np.clip(np.round(wf * ws[:, None, None, None]), -127, 127).astype(np.int8)
+    return wq, ws
+
+
+def _layers(hip, rng, chans, k=3, pad=1, act=1, stride=1):
+    convs, params = [], []
+    in_scale = np.float32(127.0)
+    for cin, cout in zip(chans[:-1], chans[1:]):
+        wq, ws = quantize_weights(rng.normal(0, 0.05, (cout, cin, k, k)).astype(np.float32))
+        bias = rng.normal(0, 0.02, cout).astype(np.float32)
+        out_scale = np.float32(rng.uniform(20, 60))
+        si = (np.float32(1.0) / (in_scale * ws)).astype(np.float32)
+        convs.append(hip.conv(wq=wq, scale_in=si, bias=bias, out_scale=[out_scale], stride=(stride, stride), pad=(pad, pad),
+                              act=act, out_kind=capi.OUT_I8, out_round=capi.ROUND_SSE))
+        params.append(dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale)))
+        in_scale = out_scale
+    return convs, params
+
+
+def _one_by_one(hip, convs, xd, n, h, w):
+    cur = xd
+    for c in convs:
+        cur = c.forward(cur, capi.I8_P8, n, h, w, capi.I8_P8)
+        h, w = c.out_hw(h, w)
+    return cur
+
+
+@pytest.mark.parametrize("C,N,H,W,L,act", [
+    (128, 16, 28, 28, 4, 1),     # whole tiles, two images per XCD, ReLU
+    (72, 19, 13, 26, 3, 3),      # padded channels, ragged tiles, images not a multiple of the XCDs, clip
+    (128, 64, 56, 56, 4, 1),     # the benchmark's chain
+    (96, 9, 15, 55, 2, 0),       # odd width, no activation (signed results)
+    (128, 3, 56, 56, 8, 1),      # fewer images than XCDs, the longest chain one launch takes
+])
+def test_same_shape_chain_is_one_launch_and_equals_the_layers_one_by_one(hip, oracle, C, N, H, W, L, act):
+    rng = np.random.default_rng(C + N + H + L)
+    convs, params = _layers(hip, rng, [C] * (L + 1), act=act)
+    x = rng.integers(-127, 128, size=(N, C, H, W), dtype=np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    want = _one_by_one(hip, convs, xd, N, H, W).cpu().numpy()
+    assert not hip.conv_chain_gave_up()
+    assert hip.conv_chain_launches(convs, N, H, W) == 1
+    for rep in range(3):  # the flags and queue counters carry over from launch to launch
+        got = hip.conv_chain(convs, xd, N, H, W)
+        assert not hip.conv_chain_gave_up()
+        np.testing.assert_array_equal(got.cpu().numpy(), want, err_msg="call %d" % rep)
+    # and the oracle through all layers on two images
+    for n in (0, N - 1):
+        cur = x[n:n + 1]
+        for p in params:
+            cur = oracle.conv_layer_forward(cur, p["wq"], p["ws"], p["in_scale"], pad=(1, 1), bias=p["bias"],
+                                            top_scale=p["out_scale"], int8_out=True, act_type=act)
+        got_n = capi.unpack_np(got.cpu().numpy(), 8, (N, C, H, W))[n:n + 1]
+        np.testing.assert_array_equal(got_n, cur)
+
+
+def test_other_chains_run_layer_by_layer(hip, oracle):
+    rng = np.random.default_rng(5)
+    # channel counts change along the chain, and a 1x1 in the middle
+    convs, _ = _layers(hip, rng, [32, 64], k=3)
+    c2, _ = _layers(hip, rng, [64, 64], k=1, pad=0)
+    c3, _ = _layers(hip, rng, [64, 24], k=3, stride=2)
+    chain = convs + c2 + c3
+    N, H, W = 3, 17, 20
+    x = rng.integers(-127, 128, size=(N, 32, H, W), dtype=np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    want = _one_by_one(hip, chain, xd, N, H, W).cpu().numpy()
+    assert hip.conv_chain_launches(chain, N, H, W) == 3
+    got = hip.conv_chain(chain, xd, N, H, W).cpu().numpy()
+    np.testing.assert_array_equal(got, want)
+    assert not hip.conv_chain_gave_up()
+
+
+def test_same_shape_chain_that_needs_two_lds_stages_runs_layer_by_layer(hip):
+    """72 channels at 13x22: a tile's rows of all 128 padded channels do not fit LDS at once, which the one-launch
+    kernel requires; the entry point runs the layers one after the other and the result is the same."""
+    rng = np.random.default_rng(8)
+    convs, _ = _layers(hip, rng, [72] * 4, act=3)
+    N, H, W = 5, 13, 22
+    x = rng.integers(-127, 128, size=(N, 72, H, W), dtype=np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    want = _one_by_one(hip, convs, xd, N, H, W).cpu().numpy()
+    assert hip.conv_chain_launches(convs, N, H, W) == 3
+    np.testing.assert_array_equal(hip.conv_chain(convs, xd, N, H, W).cpu().numpy(), want)
+
+
+def test_chain_argument_checks(hip):
+    rng = np.random.default_rng(6)
+    convs, _ = _layers(hip, rng, [16, 32])
+    other, _ = _layers(hip, rng, [16, 16])
+    x = hip.to_device(np.zeros(2 * 16 * 8 * 8, np.int8))
+    with pytest.raises(capi.HipError):
+        hip.conv_chain(convs + other, x, 2, 8, 8)  # 32 channels out, 16 in
+    f32 = hip.conv(wq=np.zeros((16, 16, 3, 3), np.int8), scale_in=np.ones(16, np.float32), pad=(1, 1), out_kind=capi.OUT_F32)
+    with pytest.raises(capi.HipError):
+        hip.conv_chain(other + [f32], x, 2, 8, 8)  # an fp32 result inside a chain

@@ -287,14 +287,16 @@ __device__ __forceinline__ void epi8_clamp_init(const Epilogue& ep, Epi8& p) {
     }
 }
 
-template <bool NONNEG>
-__device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const Epilogue& ep, const Epi8& p, size_t elem,
-                                                const int (&a8)[8]) {
+// LRELU: 0 = no LeakyReLU, 1 = LeakyReLU, -1 = decided by ep.lrelu at run time (a select per value)
+template <bool NONNEG, int LRELU = -1>
+__device__ __forceinline__ ohip_v2i epi8_quant_i8p8(const Epilogue& ep, const Epi8& p, const int (&a8)[8]) {
     int q[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float v = __fmaf_rn((float)a8[e], p.si[e], p.bi[e]);
-        if (!NONNEG && ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch
+        if constexpr (!NONNEG && LRELU != 0) {
+            if (LRELU == 1 || ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform
+        }
         v = __fmul_rn(v, p.so[e]);
         float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
         q[e] = (int)adj;  // toward zero, saturating
@@ -316,7 +318,29 @@ __device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const 
         }
         pk[h] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
     }
-    *reinterpret_cast<ohip_v2i*>(out + elem) = pk;
+    return pk;
+}
+
+template <bool NONNEG>
+__device__ __forceinline__ void epi8_store_i8p8(int8_t* __restrict__ out, const Epilogue& ep, const Epi8& p, size_t elem,
+                                                const int (&a8)[8]) {
+    *reinterpret_cast<ohip_v2i*>(out + elem) = epi8_quant_i8p8<NONNEG>(ep, p, a8);
+}
+
+// dequantize 4 channels with the clamp activation (LRELU false) or LeakyReLU (true): the bits of one Float4 element
+template <bool LRELU>
+__device__ __forceinline__ ohip_v4i epi4_dequant_f32p4(const Epilogue& ep, const float* si, const float* bi, int a0, int a1,
+                                                       int a2, int a3) {
+    const int a[4] = {a0, a1, a2, a3};
+    ohip_v4i r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float v = __fmaf_rn((float)a[e], si[e], bi[e]);
+        if constexpr (LRELU) v = fmaxf(v, __fmul_rn(v, ep.act_p0));
+        else v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
+        r[e] = __float_as_int(v);
+    }
+    return r;
 }
 
 // dequantize (+clamp activation) 4 channels and store one Float4 element. FUSED: first add the residual blob's element

@@ -13,6 +13,9 @@
 #include "common.hpp"
 #include "conv_igemm.hpp"
 
+#include <algorithm>
+#include <type_traits>
+
 namespace ohip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -32,14 +35,19 @@ struct IgemmCfg {
     static_assert(TN % 64 == 0, "pixel tile");
 };
 
-template <int TM, int TN, int WM, int WN, int EPI>
+// KC = k-chunks per stage. KC == 1: LDS double buffer, the next chunk in registers while one is multiplied (one
+// global-memory latency per chunk: right for long reductions, where several workgroups per CU cover it). KC > 1: a
+// stage of KC chunks in a single LDS buffer, the whole next stage in registers meanwhile; a reduction of at most KC
+// chunks (pointwise layers) then pays the latency once per workgroup instead of once per chunk.
+template <int TM, int TN, int WM, int WN, int EPI, int KC>
 __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                          void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
                                                          int c_groups, int n_pix_tiles) {
     using Cfg = IgemmCfg<TM, TN, WM, WN>;
     constexpr int FM = Cfg::FM, FN = Cfg::FN;
-    __shared__ __attribute__((aligned(16))) int8_t lds_a[2][Cfg::A_BYTES];
-    __shared__ __attribute__((aligned(16))) int8_t lds_b[2][Cfg::B_BYTES];
+    constexpr int NBUF = KC == 1 ? 2 : KC;
+    __shared__ __attribute__((aligned(16))) int8_t lds_a[NBUF][Cfg::A_BYTES];
+    __shared__ __attribute__((aligned(16))) int8_t lds_b[NBUF][Cfg::B_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -92,11 +100,11 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         xn = x + (size_t)n * Cs8 * HW * 8;
     }
 
-    v2i breg[Cfg::B_V][2];
-    v4i areg[Cfg::A_V];
+    v2i breg[KC][Cfg::B_V][2];
+    v4i areg[KC][Cfg::A_V];
     const int n_chunks = g.kh * g.kw * c_groups;
 
-    auto load_global = [&](int kc) {
+    auto load_global = [&](int kc, int q) {
         const int tap = kc / c_groups, cgp = kc % c_groups;
         const int u = tap / g.kw, v = tap % g.kw;
         const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
@@ -108,27 +116,27 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             v2i lo = {0, 0}, hi = {0, 0};
             if (inb && o0 < C8) lo = *reinterpret_cast<const v2i*>(px + (size_t)o0 * HW * 8);
             if (inb && o0 + 1 < C8) hi = *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * HW * 8);
-            breg[r][0] = lo;
-            breg[r][1] = hi;
+            breg[q][r][0] = lo;
+            breg[q][r][1] = hi;
         }
         const int8_t* wa = wpk + ((size_t)kc * m_tiles16 + mt0) * 1024;
 #pragma unroll
         for (int r = 0; r < Cfg::A_V; ++r) {
             const int vi = tid + r * 256;
-            if (vi * 16 < Cfg::A_BYTES) areg[r] = *reinterpret_cast<const v4i*>(wa + (size_t)vi * 16);
+            if (vi * 16 < Cfg::A_BYTES) areg[q][r] = *reinterpret_cast<const v4i*>(wa + (size_t)vi * 16);
         }
     };
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](int buf, int q) {
 #pragma unroll
         for (int r = 0; r < Cfg::B_V; ++r) {
             const int j = j0 + r * J_STEP;
-            v4i t = {breg[r][0][0], breg[r][0][1], breg[r][1][0], breg[r][1][1]};
+            v4i t = {breg[q][r][0][0], breg[q][r][0][1], breg[q][r][1][0], breg[q][r][1][1]};
             *reinterpret_cast<v4i*>(&lds_b[buf][(j * TN + p_l) * 16]) = t;
         }
 #pragma unroll
         for (int r = 0; r < Cfg::A_V; ++r) {
             const int vi = tid + r * 256;
-            if (vi * 16 < Cfg::A_BYTES) *reinterpret_cast<v4i*>(&lds_a[buf][vi * 16]) = areg[r];
+            if (vi * 16 < Cfg::A_BYTES) *reinterpret_cast<v4i*>(&lds_a[buf][vi * 16]) = areg[q][r];
         }
     };
 
@@ -138,13 +146,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-
-    for (int kc = 0; kc < n_chunks; ++kc) {
-        const int buf = kc & 1;
-        if (kc + 1 < n_chunks) load_global(kc + 1);
+    auto multiply = [&](int buf) {
         v4i a[FM], b[FN];
 #pragma unroll
         for (int i = 0; i < FM; ++i)
@@ -158,10 +160,44 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
 #pragma unroll
             for (int j = 0; j < FN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
-        if (kc + 1 < n_chunks) store_lds(buf ^ 1);
+    };
+    if constexpr (KC == 1) {
+        load_global(0, 0);
+        store_lds(0, 0);
         __syncthreads();
+        for (int kc = 0; kc < n_chunks; ++kc) {
+            const int buf = kc & 1;
+            if (kc + 1 < n_chunks) load_global(kc + 1, 0);
+            multiply(buf);
+            if (kc + 1 < n_chunks) store_lds(buf ^ 1, 0);
+            __syncthreads();
+        }
+    } else {
+        // (the chunk tests are uniform over the workgroup)
+#pragma unroll
+        for (int q = 0; q < KC; ++q)
+            if (q < n_chunks) load_global(q, q);
+#pragma unroll
+        for (int q = 0; q < KC; ++q)
+            if (q < n_chunks) store_lds(q, q);
+        __syncthreads();
+        for (int k0 = 0; k0 < n_chunks; k0 += KC) {
+            const int k1 = k0 + KC;  // first chunk of the next stage
+#pragma unroll
+            for (int q = 0; q < KC; ++q)
+                if (k1 + q < n_chunks) load_global(k1 + q, q);
+#pragma unroll
+            for (int q = 0; q < KC; ++q)
+                if (k0 + q < n_chunks) multiply(q);
+            if (k1 < n_chunks) {
+                __syncthreads();  // everyone has read this stage
+#pragma unroll
+                for (int q = 0; q < KC; ++q)
+                    if (k1 + q < n_chunks) store_lds(q, q);
+                __syncthreads();
+            }
+        }
     }
-
     // ---- epilogue -----------------------------------------------------------------------------------
     // (no `continue` / early exits inside the unrolled loops: the accumulator array must stay in registers)
     const int gq = lane >> 4;
@@ -171,49 +207,106 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     const unsigned n0 = gp0 / (unsigned)OHW;
     const unsigned pix0 = gp0 - n0 * (unsigned)OHW;
     const bool wide = (unsigned)OHW >= 16u * FN;  // then a column is at most one image further than the first
-#pragma unroll
-    for (int ip = 0; ip < FM / 2; ++ip) {
-        const int tpair = (mt0 + wm * FM) / 2 + ip;
-        const int ch0 = 32 * tpair + 8 * gq;  // this lane's 8 consecutive output channels
-        const bool ch_ok = ch0 < g.K;
-        Epi8 prm;
-        if constexpr (EPI != EPI_GENERIC) epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
+    if constexpr (EPI == EPI_F32_P4 || EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
+        // Packed outputs without the fused extras. A lane's stores differ by a column offset (image, pixel) and a row
+        // offset (channel group): each computed once, one 64-bit addition per store. LeakyReLU is decided once, in
+        // front of the unrolled loops, not per value.
+        constexpr bool F32 = EPI == EPI_F32_P4;
+        constexpr int EB = F32 ? 16 : 8;       // bytes of one (pixel, channel group) element
+        constexpr int CG = F32 ? 4 : 8;        // channels per group
+        const size_t plane = (size_t)OHW * EB;  // one channel group of one image
+        const size_t image = plane * (size_t)(Ks / CG);
+        size_t col_ofs[FN];
+        bool col_ok[FN];
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             const unsigned gpo = gp0 + j * 16;
-            int a8[8];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                a8[e] = acc[2 * ip][j][e];
-                a8[4 + e] = acc[2 * ip + 1][j][e];
+            unsigned nn = n0, pp = pix0 + j * 16;
+            if (wide) {
+                if (pp >= (unsigned)OHW) pp -= (unsigned)OHW, ++nn;
+            } else {
+                nn = gpo / (unsigned)OHW;
+                pp = gpo - nn * (unsigned)OHW;
             }
-            if (ch_ok && gpo < total_pix) {
-                unsigned nn = n0, pp = pix0 + j * 16;
-                if (wide) {
-                    if (pp >= (unsigned)OHW) pp -= (unsigned)OHW, ++nn;
-                } else {
-                    nn = gpo / (unsigned)OHW;
-                    pp = gpo - nn * (unsigned)OHW;
+            col_ok[j] = gpo < total_pix;
+            col_ofs[j] = (size_t)nn * image + (size_t)pp * EB;
+        }
+        auto rows = [&](auto lrelu_c) {
+            constexpr bool LRELU = decltype(lrelu_c)::value;
+#pragma unroll
+            for (int ip = 0; ip < FM / 2; ++ip) {
+                const int tpair = (mt0 + wm * FM) / 2 + ip;
+                const int ch0 = 32 * tpair + 8 * gq;  // this lane's 8 consecutive output channels
+                const bool ch_ok = ch0 < g.K;
+                Epi8 prm;
+                epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
+                char* row = (char*)out + (size_t)(ch0 / CG) * plane;
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    int a8[8];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        a8[e] = acc[2 * ip][j][e];
+                        a8[4 + e] = acc[2 * ip + 1][j][e];
+                    }
+                    if (ch_ok && col_ok[j]) {
+                        char* o = row + col_ofs[j];
+                        if constexpr (F32) {
+                            *reinterpret_cast<ohip_v4i*>(o) =
+                                epi4_dequant_f32p4<LRELU>(ep, prm.si, prm.bi, a8[0], a8[1], a8[2], a8[3]);
+                            if (ch0 + 4 < g.K)
+                                *reinterpret_cast<ohip_v4i*>(o + plane) =
+                                    epi4_dequant_f32p4<LRELU>(ep, prm.si + 4, prm.bi + 4, a8[4], a8[5], a8[6], a8[7]);
+                        } else {
+                            *reinterpret_cast<ohip_v2i*>(o) =
+                                epi8_quant_i8p8<EPI == EPI_I8_P8_NONNEG, LRELU ? 1 : 0>(ep, prm, a8);
+                        }
+                    }
                 }
-                const int n = (int)nn, pix = (int)pp;
-                if constexpr (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
-                    epi8_store_i8p8<EPI == EPI_I8_P8_NONNEG>((int8_t*)out, ep, prm,
-                                                             elem_offset(8, n, ch0, pix, Ks, OHW), a8);
-                } else if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P4_FUSED) {
-                    constexpr bool FUSED = EPI == EPI_F32_P4_FUSED;
-                    ohip_v2i tw = {0, 0};
-                    tw[0] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si, prm.bi,
-                                                         elem_offset(4, n, ch0, pix, Ks, OHW), a8[0], a8[1], a8[2], a8[3]);
-                    if (ch0 + 4 < g.K)
-                        tw[1] = (int)epi4_store_f32p4<FUSED>((float*)out, ep, prm.si + 4, prm.bi + 4,
-                                                             elem_offset(4, n, ch0 + 4, pix, Ks, OHW), a8[4], a8[5], a8[6],
-                                                             a8[7]);
-                    if constexpr (FUSED)
+            }
+        };
+        if (EPI != EPI_I8_P8_NONNEG && ep.lrelu) rows(std::true_type{});
+        else rows(std::false_type{});
+    } else {
+#pragma unroll
+        for (int ip = 0; ip < FM / 2; ++ip) {
+            const int tpair = (mt0 + wm * FM) / 2 + ip;
+            const int ch0 = 32 * tpair + 8 * gq;  // this lane's 8 consecutive output channels
+            const bool ch_ok = ch0 < g.K;
+            Epi8 prm;
+            if constexpr (EPI != EPI_GENERIC) epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const unsigned gpo = gp0 + j * 16;
+                int a8[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a8[e] = acc[2 * ip][j][e];
+                    a8[4 + e] = acc[2 * ip + 1][j][e];
+                }
+                if (ch_ok && gpo < total_pix) {
+                    unsigned nn = n0, pp = pix0 + j * 16;
+                    if (wide) {
+                        if (pp >= (unsigned)OHW) pp -= (unsigned)OHW, ++nn;
+                    } else {
+                        nn = gpo / (unsigned)OHW;
+                        pp = gpo - nn * (unsigned)OHW;
+                    }
+                    const int n = (int)nn, pix = (int)pp;
+                    if constexpr (EPI == EPI_F32_P4_FUSED) {
+                        ohip_v2i tw = {0, 0};
+                        tw[0] = (int)epi4_store_f32p4<true>((float*)out, ep, prm.si, prm.bi,
+                                                            elem_offset(4, n, ch0, pix, Ks, OHW), a8[0], a8[1], a8[2], a8[3]);
+                        if (ch0 + 4 < g.K)
+                            tw[1] = (int)epi4_store_f32p4<true>((float*)out, ep, prm.si + 4, prm.bi + 4,
+                                                                elem_offset(4, n, ch0 + 4, pix, Ks, OHW), a8[4], a8[5], a8[6],
+                                                                a8[7]);
                         if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
                             *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, Ks, OHW)) = tw;
-                } else {
-                    epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
-                                            a8[6], a8[7]);
+                    } else {
+                        epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
+                                                a8[6], a8[7]);
+                    }
                 }
             }
         }
@@ -255,38 +348,63 @@ void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* d
                 }
 }
 
-template <int TM, int TN, int WM, int WN, int EPI>
-static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+// k-chunks per stage of the staged variant: as many as keep a workgroup's LDS at 64 KB or less
+template <int TM, int TN>
+struct IgemmStage {
+    static constexpr int KC = (TM + TN) * 64 * 4 <= 64 * 1024 ? 4 : 2;
+};
+
+template <int TM, int TN, int WM, int WN, int EPI, int KC>
+static hipError_t launch_igemm_k(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                                  hipStream_t stream) {
     const long total_pix = (long)g.N * g.OH * g.OW;
     const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
     const int mpad = igemm_padded_rows(g.K);
     const int m_tiles = (mpad + TM - 1) / TM;
     const int grid_z = g.Cs ? g.Cs / g.C : 1;  // groups of a grouped convolution
-    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI>), dim3(n_pix_tiles, m_tiles, grid_z), dim3(256), 0, stream,
-                       x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
+    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI, KC>), dim3(n_pix_tiles, m_tiles, grid_z), dim3(256), 0,
+                       stream, x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
     return hipGetLastError();
+}
+
+template <int TM, int TN, int WM, int WN, int EPI>
+static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                                 int stage, hipStream_t stream) {
+    // The staged variant shortens a workgroup's life (one global-memory latency per KC chunks) but needs KC times the
+    // LDS. It pays when the whole grid is resident at once even so - the launch is then one workgroup life long -
+    // and costs where the grid runs in rounds, which the smaller footprint packs tighter. (256 compute units.)
+    const int n_chunks = g.kh * g.kw * igemm_channel_groups(g.C);
+    bool staged = false;
+    if (n_chunks >= 2) {
+        constexpr int KCS = IgemmStage<TM, TN>::KC;
+        const long per_cu = std::min<long>(4, (160 * 1024) / ((TM + TN) * 64 * KCS));
+        const long wgs = ((long)g.N * g.OH * g.OW + TN - 1) / TN * (igemm_padded_rows(g.K) / TM) * (g.Cs ? g.Cs / g.C : 1);
+        staged = wgs <= per_cu * 256;
+        if (stage) staged = stage == 2;  // forced by a test
+    }
+    if (staged) return launch_igemm_k<TM, TN, WM, WN, EPI, IgemmStage<TM, TN>::KC>(x, wpk, out, g, ep, stream);
+    return launch_igemm_k<TM, TN, WM, WN, EPI, 1>(x, wpk, out, g, ep, stream);
 }
 
 template <int TM, int TN, int WM, int WN>
 static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
-                               hipStream_t stream) {
+                               int stage, hipStream_t stream) {
     switch (pick_epilogue(ep, g.K)) {
     case EPI_I8_P8:
-        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8>(x, wpk, out, g, ep, stream);
+        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8>(x, wpk, out, g, ep, stage, stream);
     case EPI_I8_P8_NONNEG:
-        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8_NONNEG>(x, wpk, out, g, ep, stream);
+        return launch_igemm_e<TM, TN, WM, WN, EPI_I8_P8_NONNEG>(x, wpk, out, g, ep, stage, stream);
     case EPI_F32_P4:
         if (ep.twin != nullptr || ep.residual != nullptr)
-            return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4_FUSED>(x, wpk, out, g, ep, stream);
-        return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, stream);
+            return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4_FUSED>(x, wpk, out, g, ep, stage, stream);
+        return launch_igemm_e<TM, TN, WM, WN, EPI_F32_P4>(x, wpk, out, g, ep, stage, stream);
     default:
-        return launch_igemm_e<TM, TN, WM, WN, EPI_GENERIC>(x, wpk, out, g, ep, stream);
+        return launch_igemm_e<TM, TN, WM, WN, EPI_GENERIC>(x, wpk, out, g, ep, stage, stream);
     }
 }
 
-// tile choice. Long reductions (3x3 and larger over many channels) are MFMA-bound: the widest row tile that does not
-// pad M further, then the widest pixel tile that still leaves two workgroups per compute unit. Short reductions
+// tile choice. Long reductions (3x3 and larger over many channels): the widest row tile that does not pad M further,
+// then a pixel tile of 128 where that still gives every compute unit work, else 64. Short reductions
 // (pointwise layers, at most 16 k-chunks) are bound by latency and HBM: there the 128x256 tile's register count costs
 // more occupancy than its reuse saves, and the tiles below were the fastest ones measured on MI355X over the pointwise
 // shapes of a MobileNetV2 at batch 64 and 256->512 at 28x28.
@@ -299,8 +417,9 @@ void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
     if (n_chunks > 16) {
         if (mpad % 128 == 0) TM = 128;
         else if (mpad % 64 == 0) TM = 64;
-        if (wgs(TM, 256) >= 512) TN = 256;
-        else if (wgs(TM, 128) >= 512) TN = 128;
+        // measured over 3x3 / 5x5 layers of 64..512 channels at 14x14..112x112: 128 pixels beat 256 everywhere (the
+        // wider tile halves the resident workgroups and its rounds quantise worse), 64 win below ~1.5 workgroups per CU
+        if (wgs(TM, 128) >= 384) TN = 128;
     } else if (mpad >= 512 && mpad % 128 == 0) {
         TM = 128;
     } else if (mpad >= 64) {
@@ -348,11 +467,14 @@ hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const C
         g.C = g_in.C / g_in.groups, g.K = g_in.K / g_in.groups;
         g.groups = 1;
     }
+    // a forced pixel tile may carry the stage choice in its low bits (1: one chunk per stage, 2: the staged variant)
+    const int stage = tn & 3;
+    tn &= ~3;
     if (tm == 0 || tn == 0) igemm_choose_tiles(g, &tm, &tn);
     // a row tile must not reach past the padded weight rows
     if (igemm_padded_rows(g.K) % tm != 0) return hipErrorInvalidValue;
 #define OHIP_IG(TM_, TN_, WM_, WN_) \
-    if (tm == TM_ && tn == TN_) return launch_igemm<TM_, TN_, WM_, WN_>(x, wpk, out, g, ep, stream);
+    if (tm == TM_ && tn == TN_) return launch_igemm<TM_, TN_, WM_, WN_>(x, wpk, out, g, ep, stage, stream);
     OHIP_IG(128, 256, 2, 2)
     OHIP_IG(128, 128, 2, 2)
     OHIP_IG(128, 64, 4, 1)

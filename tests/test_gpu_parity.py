@@ -191,9 +191,14 @@ def _rand_problem(rng, C, K, k, g, N, H, W, in_i8=True):
 TILES = [(128, 256), (128, 128), (128, 64), (64, 256), (64, 128), (64, 64), (32, 256), (32, 128), (32, 64)]
 
 
+@pytest.mark.parametrize("stage", [1, 2], ids=["chunkwise", "staged"])
 @pytest.mark.parametrize("tile", TILES, ids=["%dx%d" % t for t in TILES])
-def test_igemm_every_tile_shape(hip, oracle, tile):
+def test_igemm_every_tile_shape(hip, oracle, tile, stage):
+    """Every tile shape in both variants of the kernel (one 64-deep slice of the reduction per stage, or several):
+    accumulators, the int8 epilogue with ReLU, without activation and with LeakyReLU, the fp32 epilogue with ReLU and
+    LeakyReLU. The reductions are 9, 1 and 18 slices long: shorter than, equal to and not a multiple of a stage."""
     rng = np.random.default_rng(tile[0] * 1000 + tile[1])
+    tile = (tile[0], tile[1] + stage)
     # K = 128 divides every row tile; 2 x 19 x 23 pixels leaves a ragged last pixel tile
     for (C, K, k, s, p) in [(64, 128, 3, 1, 1), (24, 128, 1, 1, 0), (72, 128, 3, 2, 1)]:
         x, wq, ws, bias = _rand_problem(rng, C, K, k, 1, 2, 19, 23)
@@ -206,6 +211,15 @@ def test_igemm_every_tile_shape(hip, oracle, tile):
         out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, bias=bias, top_scale=9.0, act=1,
                           out_kind=capi.OUT_I8, tile=tile)
         np.testing.assert_array_equal(out, want)
+        for act, int8_out in [(0, True), (2, True), (1, False), (2, False)]:
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), bias=bias, top_scale=9.0,
+                                             int8_out=int8_out, act_type=act, act_params=[0.1])
+            out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, bias=bias, top_scale=9.0, act=act,
+                              act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32, tile=tile)
+            if int8_out:
+                np.testing.assert_array_equal(out, want)
+            else:
+                np.testing.assert_allclose(out, want, rtol=FP32_RTOL, atol=0)
 
 
 @pytest.mark.parametrize("fn", [4, 5, 6, 7])

@@ -647,6 +647,8 @@ def main():
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-also", action="store_true")
+    ap.add_argument("--per-layer", action="store_true",
+                    help="print one JSON line with every convolution layer of the c4 network timed by itself, and exit")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path shards by batch: images are independent); "
@@ -659,6 +661,16 @@ def main():
     from tensor_amd import capi
     hip = capi.Library(0)
     timer = Timer(hip.torch)
+    if a.per_layer:
+        from tensor_amd import mobilenet
+        rows = mobilenet.per_layer(hip, capi, np.random.default_rng(0),
+                                   lambda fn: timer.run(fn, max(a.steps * 2, 100), a.warmup, settle=0.05)[0])
+        for r in rows:
+            r["frac_hbm"] = r["gbs"] / PEAK_HBM_GBS
+            r["frac_mfma"] = r["tops"] / PEAK_INT8_TOPS
+        print(json.dumps({"workload": "c4 layers one by one, batch 64", "sum_us": sum(r["us"] for r in rows),
+                          "layers": rows}))
+        return
     builders = {"c3": lambda r: build_c3(hip, capi, r), "c1s1": lambda r: build_c1(hip, capi, r, 1),
                 "c1s2": lambda r: build_c1(hip, capi, r, 2), "c2": lambda r: build_c2(hip, capi, r),
                 "c0": lambda r: build_c0(hip, capi, r), "copy": lambda r: build_copy(hip, capi, r),

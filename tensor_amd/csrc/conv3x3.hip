@@ -29,7 +29,9 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 
 constexpr unsigned HALO_OOB = 0x80000000u;  // beyond the buffer descriptor: reads as zero
 
-template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
+// S = stride (1 or 2), D = dilation (1 or 2; not both 2): the staged rows are (output rows - 1) * S + 2 * D + 1, a
+// lane's pixel sits at column ox * S, and the taps are D pixels / D rows apart. Everything else is the same kernel.
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S = 1, int D = 1>
 __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                            void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
                                                            int c_groups, int r_max, int cb, int tiles_per_img, int prm_ofs,
@@ -75,7 +77,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
     auto stage = [&](int n, int p0, int cb0) {
         const int p_last = min(p0 + PT, OHW) - 1;
         const int r_lo = p0 / g.OW;
-        const int R = p_last / g.OW - r_lo + 3;
+        const int R = (p_last / g.OW - r_lo) * S + 2 * D + 1;
         if constexpr (LOGP == 9) {
             // 512-byte lines: one instruction moves a row of BOTH octets of a pair (adjacent lines in LDS): lanes 0-31
             // the first octet, lanes 32-63 the second, 16 bytes = pixels 2*pp-2 and 2*pp-1 each
@@ -89,7 +91,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                     const int o = cb0 / 8 + 2 * pj;
                     const bool both = o + 1 < C8;
                     for (int r = 0; r < R; ++r) {
-                        const int iy = r_lo - g.ph + r;
+                        const int iy = r_lo * S - g.ph + r;
                         const bool ok = o < C8 && iy >= 0 && iy < g.H;  // wave-uniform
                         const unsigned s_off = ok ? (unsigned)((n * C8 + o) * g.H + iy) * (unsigned)(g.W * 8) : 0u;
                         int8_t* dst = lds + (size_t)pj * pair_bytes + (size_t)((2 * r) << LOGP);
@@ -106,7 +108,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                 for (int oc = wave; oc < cb / 8; oc += 4) {
                     const int o = cb0 / 8 + oc;
                     for (int r = 0; r < R; ++r) {
-                        const int iy = r_lo - g.ph + r;
+                        const int iy = r_lo * S - g.ph + r;
                         const bool ok = o < C8 && iy >= 0 && iy < g.H;  // wave-uniform
                         const unsigned s_off = ok ? (unsigned)((n * C8 + o) * g.H + iy) * (unsigned)(g.W * 8) : 0u;
                         int8_t* dst = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((2 * r + (oc & 1)) << LOGP);
@@ -124,7 +126,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
     auto fix_odd = [&](int p0) {
         if (!(g.W & 1)) return;
         const int p_last = min(p0 + PT, OHW) - 1;
-        const int R = p_last / g.OW - p0 / g.OW + 3;
+        const int R = (p_last / g.OW - p0 / g.OW) * S + 2 * D + 1;
         const int lines = (cb / 8) * R;  // (octet, row) lines of the stage
         for (int i = lane; i < lines; i += 64) {
             const int oc = i / R, r = i - oc * R;
@@ -160,7 +162,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
             for (int f = 0; f < FN; ++f) {
                 const int pix = min(p0 + (wn * FN + f) * 16 + (lane & 15), OHW - 1);
                 const int oy = pix / g.OW, ox = pix % g.OW;
-                bcc[f] = (oy - r_lo) * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
+                bcc[f] = (oy - r_lo) * S * 2 * PITCH + (ox * S - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
             }
         }
 
@@ -217,7 +219,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                     constexpr int AH = RD - 1;  // taps ahead
                     const int8_t* pa = tap + AH < 9 ? a_ptr(cc, tap + AH) : a_ptr(cc_next, tap + AH - 9);
                     constexpr int kRowB = 2 * PITCH;
-                    const int nofs = tap < 8 ? ((tap + 1) / 3) * kRowB + ((tap + 1) % 3) * 8 : 0;  // compile-time
+                    const int nofs = tap < 8 ? ((tap + 1) / 3) * D * kRowB + ((tap + 1) % 3) * D * 8 : 0;  // compile-time
 #pragma unroll
                     for (int f = 0; f < FN; ++f) {
 #pragma unroll
@@ -330,12 +332,12 @@ struct HaloPlan {
     double cost;
 };
 
-// rows of output a run of pt pixels starting at a multiple of pt can touch, +2 halo rows
-int halo_rows(int pt, int OW, int OHW) {
+// input rows a run of pt output pixels starting at a multiple of pt can touch (stride s, dilation d), halo included
+int halo_rows(int pt, int OW, int OHW, int s, int d) {
     int worst = 0;
     for (int p0 = 0; p0 < OHW; p0 += pt) {
         const int last = (p0 + pt < OHW ? p0 + pt : OHW) - 1;
-        const int rows = last / OW - p0 / OW + 3;
+        const int rows = (last / OW - p0 / OW) * s + 2 * d + 1;
         if (rows > worst) worst = rows;
     }
     return worst;
@@ -354,10 +356,10 @@ void halo_grid(int mpad, int tiles16_per_wg, int total_tiles, int* m_blocks, int
     *grid_x = gx;
 }
 
-template <int FM, int FN, int WM, int WN, int EPI, int LOGP>
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S, int D>
 hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                          const HaloPlan& pl, hipStream_t stream) {
-    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI, LOGP>;
+    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI, LOGP, S, D>;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -380,8 +382,20 @@ hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const Co
 template <int FM, int FN, int WM, int WN, int EPI>
 hipError_t launch_halo_e(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                          const HaloPlan& pl, hipStream_t stream) {
-    if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9>(x, wpk, out, g, ep, pl, stream);
-    return launch_halo_p<FM, FN, WM, WN, EPI, 10>(x, wpk, out, g, ep, pl, stream);
+    // the strided and the dilated variant exist for row blocks of 64 channels and more (FM == 4)
+    if constexpr (FM == 4) {
+        if (g.sh == 2) {
+            if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9, 2, 1>(x, wpk, out, g, ep, pl, stream);
+            return launch_halo_p<FM, FN, WM, WN, EPI, 10, 2, 1>(x, wpk, out, g, ep, pl, stream);
+        }
+        if (g.dh == 2) {
+            if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9, 1, 2>(x, wpk, out, g, ep, pl, stream);
+            return launch_halo_p<FM, FN, WM, WN, EPI, 10, 1, 2>(x, wpk, out, g, ep, pl, stream);
+        }
+    }
+    if (g.sh != 1 || g.dh != 1) return hipErrorInvalidValue;
+    if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9, 1, 1>(x, wpk, out, g, ep, pl, stream);
+    return launch_halo_p<FM, FN, WM, WN, EPI, 10, 1, 1>(x, wpk, out, g, ep, pl, stream);
 }
 
 template <int FM, int FN, int WM, int WN>
@@ -417,7 +431,7 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
         HaloPlan p;
         p.fn = fn;
         p.logp = logp;
-        p.r_max = halo_rows(pt, g.OW, OHW);
+        p.r_max = halo_rows(pt, g.OW, OHW, g.sh, g.dh);
         const size_t per64 = (size_t)8 * p.r_max << logp;  // 64 channels = 8 octets
         if (per64 > (size_t)kMaxLdsBytes) continue;
         int cb = (int)(kMaxLdsBytes / per64) * 64;
@@ -442,8 +456,13 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
 }  // namespace
 
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep) {
-    if (!(g.kh == 3 && g.kw == 3 && g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.groups == 1)) return false;
-    if (g.ph > 1 || g.pw > 1 || g.C % 8) return false;
+    if (!(g.kh == 3 && g.kw == 3 && g.groups == 1 && g.sh == g.sw && g.dh == g.dw)) return false;
+    // stride 1 dilation 1 (any row block), or stride 2 / dilation 2 (not both) for 33 output channels and more
+    const bool plain = g.sh == 1 && g.dh == 1;
+    const bool variant = (g.sh == 2 && g.dh == 1) || (g.sh == 1 && g.dh == 2);
+    if (!plain && !(variant && igemm_padded_rows(g.K) >= 64)) return false;
+    // the LDS lines carry two zero columns on either side: padding up to the dilation (a tap never reaches further)
+    if (g.ph > g.dh || g.pw > g.dw || g.C % 8) return false;
     if ((size_t)g.N * g.C * g.H * g.W >= ((size_t)1 << 31)) return false;  // 32-bit offsets
     if (pick_epilogue(ep, g.K) == EPI_GENERIC) return false;
     HaloPlan p;

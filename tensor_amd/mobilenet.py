@@ -212,3 +212,55 @@ def build_bench(hip, capi, rng, batch=64, hw=224, calib=32):
                          "layer): %d convolutions + 10 adds + avgpool + inner product" % sum(l["kind"] == "conv" for l in layers),
                 dom_kernel="whole network (all kernels of one forward pass)", dom_fn=None, x=x, params=[],
                 shape=(batch, 3, hw, hw), _keep=(net, sess))
+
+
+KERNEL_NAMES = {0: "direct", 1: "implicit GEMM (MFMA)", 2: "depthwise", 3: "3x3 LDS-halo (MFMA)", 4: "few-channel 3x3"}
+
+
+def per_layer(hip, capi, rng, time_fn, batch=64, hw=224, calib=32):
+    """Every convolution layer of the network by itself, through the C ABI, on a device-resident input of the layer's
+    own shape (the image for the stem, Byte8 elsewhere: inside the network the producers write their readers' int8
+    input). time_fn(closure) -> milliseconds per call. Returns one dict per layer: shape, kernel family, time,
+    algorithmic bytes (input + output + weights) and operations with the rates they amount to."""
+    layers = describe()
+    params = init_weights(layers, rng)
+    calibrate(hip, capi, layers, params, rng.uniform(0, 1, (calib, 3, hw, hw)).astype(np.float32))
+    size = {"data": hw}
+    rows = []
+    for l in layers:
+        if l["kind"] != "conv":
+            if l["kind"] == "add":
+                size[l["name"]] = size[l["a"]]
+            continue
+        p = params[l["name"]]
+        hin = size[l["input"]]
+        cin, cout, k, s = l["cin"], l["cout"], l["k"], l["stride"]
+        si = (np.float32(1.0) / (np.float32(p["in_scale"]) * p["ws"])).astype(np.float32)
+        conv = hip.conv(wq=p["wq"], scale_in=si, bias=p["bias"], in_scale=p["in_scale"], stride=(s, s), pad=(k // 2,) * 2,
+                        groups=l["groups"], act=_act_id(l["act"]),
+                        in_round=capi.ROUND_SSE if cin % 8 == 0 else capi.ROUND_EXACT,
+                        out_kind=capi.OUT_I8 if l["int8_out"] else capi.OUT_F32,
+                        out_scale=[p["top_scale"]] if l["int8_out"] else None)
+        hout = conv.out_hw(hin, hin)[0]
+        size[l["name"]] = hout
+        if l["name"] == "stem":
+            x = hip.to_device(rng.uniform(0, 1, (batch, 3, hin, hin)).astype(np.float32))
+            in_layout, in_bytes = capi.F32, 4 * batch * 3 * hin * hin
+        else:
+            x = hip.to_device(rng.integers(-127, 128, size=batch * cin * hin * hin, dtype=np.int8))
+            in_layout, in_bytes = capi.I8_P8, batch * cin * hin * hin
+        out_layout = conv.default_out_layout()
+        out = hip.empty(batch * cout * hout * hout, capi.layout_dtype(out_layout))
+        ms = time_fn(lambda: conv.forward(x, in_layout, batch, hin, hin, out_layout, out=out))
+        out_bytes = batch * cout * hout * hout * (1 if l["int8_out"] else 4)
+        nbytes = in_bytes + out_bytes + p["wq"].size
+        ops = 2.0 * batch * cout * hout * hout * (cin // l["groups"]) * k * k
+        rows.append(dict(layer=l["name"], cin=cin, cout=cout, k=k, stride=s, groups=l["groups"], h_in=hin, h_out=hout,
+                         out="int8" if l["int8_out"] else "fp32",
+                         kernel=KERNEL_NAMES.get(conv.kernel_kind(in_layout, batch, hin, hin, out_layout), "?"),
+                         us=ms * 1e3, mbytes=nbytes / 1e6, gbs=nbytes / (ms * 1e-3) / 1e9, gops=ops / 1e9,
+                         tops=ops / (ms * 1e-3) / 1e12))
+        conv.close()
+        del x, out
+    return rows
+

@@ -251,6 +251,42 @@ def test_halo3x3_every_fragment_count(hip, oracle, fn):
         np.testing.assert_array_equal(acc, acc_want)
 
 
+@pytest.mark.parametrize("fn", [4, 5, 6, 7])
+def test_halo3x3_stride2_and_dilation2(hip, oracle, fn):
+    """The strided and the dilated variant of the LDS-halo kernel (row blocks of 64 channels and more): paddings 0 up
+    to the dilation, both wave layouts, both line pitches, odd and even widths and heights, ragged last tiles, several
+    channel blocks per tile, several tiles per workgroup. K <= 32 stays on the implicit-GEMM kernel."""
+    rng = np.random.default_rng(100 + fn)
+    cases = [  # C, K, stride, dilation, pad, N, H, W
+        (128, 128, 2, 1, 1, 2, 56, 56), (64, 128, 2, 1, 1, 2, 33, 51), (72, 40, 2, 1, 0, 2, 11, 13),
+        (16, 160, 2, 1, 1, 1, 9, 124), (128, 72, 2, 1, 1, 2, 40, 60), (192, 256, 2, 1, 0, 1, 30, 53),
+        (128, 128, 1, 2, 2, 2, 19, 22), (64, 64, 1, 2, 2, 1, 56, 56), (72, 40, 1, 2, 0, 2, 11, 13),
+        (16, 160, 1, 2, 1, 1, 9, 123), (320, 96, 1, 2, 2, 1, 14, 30), (24, 136, 1, 2, 2, 3, 7, 59),
+    ]
+    for (C, K, s, d, p, N, H, W) in cases:
+        x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
+        in_scale = 25.0
+        for int8_out in (True, False):
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), dil=(d, d), pad=(p, p), bias=bias,
+                                             top_scale=7.0, int8_out=int8_out, act_type=1)
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, dil=d, pad=p, bias=bias, top_scale=7.0,
+                                 act=1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32, tile=(-1, fn))
+            assert kind == 3, (C, K, s, d, p)
+            if int8_out:
+                np.testing.assert_array_equal(out, want)
+            else:
+                assert_f32_close(out, want)
+    # 32 output channels, or a stride-2 tile whose input rows do not fit LDS: the implicit-GEMM kernel
+    for (C, K, s, d, p, H, W) in [(64, 32, 2, 1, 1, 12, 12), (64, 32, 1, 2, 2, 12, 12), (128, 128, 2, 1, 1, 19, 22)]:
+        x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, 1, H, W)
+        want = oracle.conv_layer_forward(x, wq, ws, 25.0, stride=(s, s), dil=(d, d), pad=(p, p), bias=bias, top_scale=7.0,
+                                         int8_out=True, act_type=1)
+        out, kind = run_conv(hip, oracle, x, wq, ws, 25.0, stride=s, dil=d, pad=p, bias=bias, top_scale=7.0, act=1,
+                             out_kind=capi.OUT_I8)
+        assert kind == 1
+        np.testing.assert_array_equal(out, want)
+
+
 def test_halo3x3_ragged_last_tile_then_full_tile_in_one_workgroup(hip, oracle):
     """Tiles of whole image rows (128 pixels = 8 rows of 16) on an image that is not a whole number of tiles (20 rows:
     the third tile of an image has 4 rows), with so many output channels that the persistent grid is shorter than the

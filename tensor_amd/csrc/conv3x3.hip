@@ -31,7 +31,10 @@ constexpr unsigned HALO_OOB = 0x80000000u;  // beyond the buffer descriptor: rea
 
 // S = stride (1 or 2), D = dilation (1 or 2; not both 2): the staged rows are (output rows - 1) * S + 2 * D + 1, a
 // lane's pixel sits at column ox * S, and the taps are D pixels / D rows apart. Everything else is the same kernel.
-template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S = 1, int D = 1>
+// ODDW: the image width is odd (the pixel slot behind a row's last pixel is cleared after every transfer). A template
+// parameter because the 7-fragment tile has no register to spare: with the clearing code compiled in, its int8 and
+// fp32 instances spill (measured: 64->64 @56x56 batch 64, 17.5 -> 22.5 us); odd widths use at most 6 fragments.
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S = 1, int D = 1, bool ODDW = false>
 __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                            void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
                                                            int c_groups, int r_max, int cb, int tiles_per_img, int prm_ofs,
@@ -124,18 +127,16 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
     // row's first pixel; zero it. Runs after the wave's own transfers have landed and before the barrier, over exactly
     // the (octet, row) lines the loops of stage() give this wave.
     auto fix_odd = [&](int p0) {
-        if (!(g.W & 1)) return;
+        if constexpr (!ODDW) return;
         const int p_last = min(p0 + PT, OHW) - 1;
         const int R = (p_last / g.OW - p0 / g.OW) * S + 2 * D + 1;
-        const int lines = (cb / 8) * R;  // (octet, row) lines of the stage
-        for (int i = lane; i < lines; i += 64) {
-            const int oc = i / R, r = i - oc * R;
-            // the wave that staged octet oc: pairs go round the four waves (512-byte lines, both octets of a pair in
-            // one transfer), or single octets do
-            const int owner = LOGP == 9 ? (oc >> 1) & 3 : oc & 3;
-            if (owner != wave) continue;
-            int8_t* line = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((2 * r + (oc & 1)) << LOGP);
-            *reinterpret_cast<v2i*>(line + (g.W + 2) * 8) = v2i{0, 0};
+        // lane = octet of the stage (at most 64 octets = 512 channels per stage); the wave that staged octet oc: pairs go
+        // round the four waves (512-byte lines, both octets of a pair in one transfer), or single octets do
+        const int oc = lane;
+        const int owner = LOGP == 9 ? (oc >> 1) & 3 : oc & 3;
+        if (oc < cb / 8 && owner == wave) {
+            int8_t* line = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((oc & 1) << LOGP) + (g.W + 2) * 8;
+            for (int r = 0; r < R; ++r) *reinterpret_cast<v2i*>(line + (size_t)((2 * r) << LOGP)) = v2i{0, 0};
         }
     };
 
@@ -356,10 +357,10 @@ void halo_grid(int mpad, int tiles16_per_wg, int total_tiles, int* m_blocks, int
     *grid_x = gx;
 }
 
-template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S, int D>
-hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S, int D, bool ODDW>
+hipError_t launch_halo_w(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                          const HaloPlan& pl, hipStream_t stream) {
-    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI, LOGP, S, D>;
+    auto kern = conv3x3_halo_kernel<FM, FN, WM, WN, EPI, LOGP, S, D, ODDW>;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -377,6 +378,16 @@ hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const Co
                        out, g, ep, mpad / 16, igemm_channel_groups(g.C), pl.r_max, pl.cb, pl.tiles_per_img, prm_ofs,
                        total_tiles, in_bytes, halo_tile_invariant(WN * FN * 16, g.OW, g.OH * g.OW) ? 1 : 0);
     return hipGetLastError();
+}
+
+template <int FM, int FN, int WM, int WN, int EPI, int LOGP, int S, int D>
+hipError_t launch_halo_p(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                         const HaloPlan& pl, hipStream_t stream) {
+    if (g.W & 1) {
+        if constexpr (FN <= 6) return launch_halo_w<FM, FN, WM, WN, EPI, LOGP, S, D, true>(x, wpk, out, g, ep, pl, stream);
+        return hipErrorInvalidValue;  // (the planner gives odd widths at most 6 fragments)
+    }
+    return launch_halo_w<FM, FN, WM, WN, EPI, LOGP, S, D, false>(x, wpk, out, g, ep, pl, stream);
 }
 
 template <int FM, int FN, int WM, int WN, int EPI>
@@ -427,6 +438,7 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
     bool found = false;
     for (int fn = 4; fn <= 7; ++fn) {  // 8 fragments would spill at two waves per SIMD
         if (force_fn && fn != force_fn) continue;
+        if (fn == 7 && (g.W & 1)) continue;  // odd widths: at most 6 fragments (see the kernel's ODDW parameter)
         const int pt = (wide ? 32 : 64) * fn;
         HaloPlan p;
         p.fn = fn;

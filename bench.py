@@ -664,7 +664,7 @@ def main():
     if a.per_layer:
         from tensor_amd import mobilenet
         rows = mobilenet.per_layer(hip, capi, np.random.default_rng(0),
-                                   lambda fn: timer.run(fn, max(a.steps * 2, 100), a.warmup, settle=0.05)[0])
+                                   lambda fn: timer.run(fn, max(a.steps * 2, 100), a.warmup, settle=0.02)[0])
         for r in rows:
             r["frac_hbm"] = r["gbs"] / PEAK_HBM_GBS
             r["frac_mfma"] = r["tops"] / PEAK_INT8_TOPS

@@ -360,7 +360,7 @@ static hipError_t launch_igemm_k(const int8_t* x, const int8_t* wpk, void* out, 
     const long total_pix = (long)g.N * g.OH * g.OW;
     const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
     const int mpad = igemm_padded_rows(g.K);
-    const int m_tiles = (mpad + TM - 1) / TM;
+    const int m_tiles = (g.K + TM - 1) / TM;  // row blocks that hold at least one real channel (the rows are padded further)
     const int grid_z = g.Cs ? g.Cs / g.C : 1;  // groups of a grouped convolution
     hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI, KC>), dim3(n_pix_tiles, m_tiles, grid_z), dim3(256), 0,
                        stream, x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
@@ -378,7 +378,7 @@ static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, 
     if (n_chunks >= 2) {
         constexpr int KCS = IgemmStage<TM, TN>::KC;
         const long per_cu = std::min<long>(4, (160 * 1024) / ((TM + TN) * 64 * KCS));
-        const long wgs = ((long)g.N * g.OH * g.OW + TN - 1) / TN * (igemm_padded_rows(g.K) / TM) * (g.Cs ? g.Cs / g.C : 1);
+        const long wgs = ((long)g.N * g.OH * g.OW + TN - 1) / TN * ((g.K + TM - 1) / TM) * (g.Cs ? g.Cs / g.C : 1);
         staged = wgs <= per_cu * 256;
         if (stage) staged = stage == 2;  // forced by a test
     }
@@ -412,7 +412,7 @@ void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
     const int mpad = igemm_padded_rows(g.K);
     const long total_pix = (long)g.N * g.OH * g.OW;
     const int n_chunks = g.kh * g.kw * igemm_channel_groups(g.C);
-    auto wgs = [&](int TM, int TN) { return ((total_pix + TN - 1) / TN) * (mpad / TM); };
+    auto wgs = [&](int TM, int TN) { return ((total_pix + TN - 1) / TN) * ((g.K + TM - 1) / TM); };
     int TM = 32, TN = 64;
     if (n_chunks > 16) {
         if (mpad % 128 == 0) TM = 128;

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <random>
 #include <sstream>
@@ -661,6 +662,44 @@ int ConvolutionLayer::forward_int8(const Tensor& bottom_in, const Tensor* shortc
             if (rc) return rc;
         }
         top.mark_device_written();
+    } catch (const Error&) {
+        return -100;
+    }
+    return 0;
+}
+
+static std::atomic<long> g_chain_forwards{0};
+long ConvolutionLayer::chain_forward_count() { return g_chain_forwards.load(); }
+
+int ConvolutionLayer::forward_chain(const std::vector<const ConvolutionLayer*>& run, const Tensor& bottom, Tensor& top,
+                                    const NetOption& opt) {
+    if (run.size() < 2 || !opt.use_packing_layout || !bottom.defined() || bottom.dim() != 4 ||
+        bottom.scalar_type() != ScalarType::Byte8)
+        return 1;
+    std::vector<const otter_hip_conv*> handles;
+    for (const ConvolutionLayer* c : run) {
+        if (!c->handle_ || c->int8_scale_term <= 100 || c->force_out_layout >= 0) return 1;
+        handles.push_back(c->handle_);
+    }
+    const int N = (int)bottom.size(0), H = (int)bottom.size(2), W = (int)bottom.size(3);
+    if (bottom.channels() != run.front()->in_channels) return 1;
+    if (otter_hip_conv_chain_launches(handles.data(), (int)handles.size(), N, H, W) != 1) return 1;
+    int h = H, w = W;
+    for (const otter_hip_conv* hd : handles) {
+        int oh = 0, ow = 0;
+        if (otter_hip_conv_output_shape(hd, h, w, &oh, &ow)) return 1;
+        h = oh, w = ow;
+    }
+    try {
+        top = Tensor::empty_device({N, run.back()->out_channels / 8, h, w}, ScalarType::Byte8);
+        const size_t ws_bytes = otter_hip_conv_chain_workspace_bytes(handles.data(), (int)handles.size(), N, H, W);
+        Tensor ws;
+        if (ws_bytes) ws = Tensor::empty_device({(int64_t)ws_bytes}, ScalarType::Byte);
+        const int rc = otter_hip_conv_chain_forward(handles.data(), (int)handles.size(), bottom.device_ptr(), N, H, W,
+                                                    top.device_ptr(), ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
+        if (rc) return rc;
+        top.mark_device_written();
+        ++g_chain_forwards;
     } catch (const Error&) {
         return -100;
     }
@@ -1549,6 +1588,19 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
             if (rc <= 0) return rc;
         }
     }
+    {
+        const auto unit = chain_units_.find(li);
+        if (unit != chain_units_.end()) {
+            // only when nothing inside the run has been computed (or set by the caller) yet
+            bool fresh = true;
+            for (size_t k = 0; k + 1 < unit->second.size(); ++k)
+                fresh = fresh && !blobs[layers_[unit->second[k]]->tops[0]].defined();
+            if (fresh) {
+                const int rc = forward_chain_unit(unit->second, blobs, opt);
+                if (rc <= 0) return rc;
+            }
+        }
+    }
     for (int b : layer->bottoms)
         if (!blobs[b].defined()) {
             int rc = forward_layer(blobs_[b].producer, blobs, opt);
@@ -1671,7 +1723,55 @@ void Net::plan_fused_quantize() const {
         shuffle_units_[lo] = u;
         shuffle_units_[hi] = u;
     }
+    // Runs of int8 -> int8 convolutions, each blob read by the next convolution only (no Split: one reader), at most 8 long
+    chain_units_.clear();
+    auto chainable = [&](int li) {
+        const auto* c = dynamic_cast<const ConvolutionLayer*>(layers_[li]);
+        // (what the chain entry point runs as one launch, as far as the layer alone tells: the same 3x3 "same"
+        // convolution over one channel count; the rest is decided per input by otter_hip_conv_chain_launches)
+        return c && c->int8_scale_term > 100 && c->force_out_layout < 0 && c->bottoms.size() == 1 && c->tops.size() == 1 &&
+               c->in_channels % 8 == 0 && c->in_channels == c->out_channels && c->groups == 1 && c->kernel_height == 3 &&
+               c->kernel_width == 3 && c->stride_height == 1 && c->stride_width == 1 && c->padding_height == 1 &&
+               c->padding_width == 1 && c->dilation_height == 1 && c->dilation_width == 1;
+    };
+    for (size_t li = 0; li < layers_.size(); ++li) {
+        if (!chainable((int)li)) continue;
+        const int pi = blobs_[layers_[li]->bottoms[0]].producer;
+        if (pi >= 0 && chainable(pi) && sole_reader(layers_[pi]->tops[0]) == (int)li) continue;  // not the head of a run
+        std::vector<int> run = {(int)li};
+        for (;;) {
+            const int next = sole_reader(layers_[run.back()]->tops[0]);
+            if (next < 0 || !chainable(next)) break;
+            if (static_cast<const ConvolutionLayer*>(layers_[next])->in_channels !=
+                static_cast<const ConvolutionLayer*>(layers_[run.back()])->out_channels)
+                break;
+            run.push_back(next);
+        }
+        for (size_t k = 0; k + 1 < run.size(); k += 8) {  // pieces of at most 8 layers, at least 2
+            const size_t end = std::min(run.size(), k + 8);
+            if (end - k >= 2) chain_units_[run[end - 1]] = std::vector<int>(run.begin() + k, run.begin() + end);
+        }
+    }
     planned_ = true;
+}
+
+// A run of convolutions in one launch (ConvolutionLayer::forward_chain). Returns 1 when the run or the blob at hand does
+// not allow it; the caller then runs the layers one by one.
+int Net::forward_chain_unit(const std::vector<int>& run, std::vector<Tensor>& blobs, const NetOption& opt) const {
+    const Layer* head = layers_[run.front()];
+    const int in_blob = head->bottoms[0];
+    if (!blobs[in_blob].defined()) {
+        const int rc = forward_layer(blobs_[in_blob].producer, blobs, opt);
+        if (rc) return rc;
+    }
+    std::vector<const ConvolutionLayer*> convs;
+    for (int li : run) convs.push_back(static_cast<const ConvolutionLayer*>(layers_[li]));
+    Tensor top;
+    const int rc = ConvolutionLayer::forward_chain(convs, blobs[in_blob], top, opt);
+    if (rc) return rc;
+    blobs[layers_[run.back()]->tops[0]] = top;
+    if (opt.lightmode && blobs_[in_blob].consumers.size() == 1) blobs[in_blob] = Tensor();
+    return 0;
 }
 
 // Convolution and Eltwise sum in one launch (otter_hip_conv_forward_residual). Returns 1 when the blobs at hand do not

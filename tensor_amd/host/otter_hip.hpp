@@ -214,6 +214,12 @@ public:
     // have the layouts that takes (the caller then runs the two layers one after the other).
     int forward_residual(const Tensor& bottom_blob, const Tensor& shortcut, float q_scale, int q_round, Tensor& sum,
                          const NetOption& opt) const;
+    // A run of int8 -> int8 convolution layers, each reading the one before, as one call of the C ABI's chain entry point
+    // when that takes the run as a single launch (otter_hip_conv_chain_launches == 1); `top` is the last layer's blob,
+    // the blobs in between are not made. Returns 1, and does nothing, for any other run or input.
+    static int forward_chain(const std::vector<const ConvolutionLayer*>& run, const Tensor& bottom_blob, Tensor& top,
+                             const NetOption& opt);
+    static long chain_forward_count();  // runs executed that way so far in this process (for tests)
 
 private:
     int create_pipeline_int8(const NetOption& opt);
@@ -311,6 +317,10 @@ private:
     };
     mutable std::map<int, ResidualUnit> residual_units_;
     int forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
+    // Runs of 2..8 int8 -> int8 convolution layers, each read only by the next, found by the plan: last layer's index ->
+    // the run; forward_layer hands the run to ConvolutionLayer::forward_chain when none of its blobs exists yet.
+    mutable std::map<int, std::vector<int>> chain_units_;
+    int forward_chain_unit(const std::vector<int>& run, std::vector<Tensor>& blobs, const NetOption& opt) const;
 };
 
 class Extractor {

@@ -53,6 +53,51 @@ def test_net_chain_int8_activations_flow_between_layers(oracle):
 
 
 @pytest.mark.gpu
+def test_net_runs_a_stack_of_same_shape_3x3_layers_as_one_launch(oracle):
+    """Input -> 3x3 conv to 72 channels (int8 out) -> three more 3x3 convs 72 -> 72 (int8 out) -> 1x1 conv (fp32 out).
+    The three 72 -> 72 layers are one run for the chain entry point (the first layer
+    changes the channel count and stays by itself); the Net must give the oracle's blobs whether the run goes
+    through in one launch (only its last blob asked for) or layer by layer (a blob inside the run asked for first)."""
+    rng = np.random.default_rng(15)
+    N, C0, C, H, W = 3, 16, 72, 13, 26
+    x = rng.uniform(-1, 1, (N, C0, H, W)).astype(np.float32)
+    names = ["c0", "c1", "c2", "c3"]
+    chans = [C0, C, C, C, C]
+    net = hostnet.Net()
+    net.add_layer(type="Input", name="data", batchsize=N, channel=C0, height=H, width=W)
+    for i, nm in enumerate(names):
+        net.add_layer(type="Convolution", name=nm, out_channels=chans[i + 1], kernel=3, padding=1, int8_scale_term=102,
+                      activation="Relu")
+    net.add_layer(type="Convolution", name="head", out_channels=8, kernel=1, int8_scale_term=2)
+    net.compile()
+    scale = np.float32(127) / np.abs(x).max()
+    want, cur = {}, x
+    for i, nm in enumerate(names):
+        w, s = _qweights(rng, chans[i + 1], chans[i], 3)
+        b = rng.normal(0, 0.05, chans[i + 1]).astype(np.float32)
+        top = np.float32(rng.uniform(15, 30))
+        net.set_conv(nm, w, b, s, scale, top)
+        cur = oracle.conv_layer_forward(cur, w, s, scale, pad=(1, 1), bias=b, top_scale=top, int8_out=True, act_type=1)
+        want[nm] = cur
+        scale = top
+    wh, sh = _qweights(rng, 8, C, 1)
+    bh = rng.normal(0, 0.05, 8).astype(np.float32)
+    net.set_conv("head", wh, bh, sh, scale)
+    want["head"] = oracle.conv_layer_forward(cur, wh, sh, scale, bias=bh)
+
+    # (Net.run makes two passes: one for the shape, one for the data)
+    before = hostnet.chain_forward_count()
+    np.testing.assert_allclose(net.run("data", x, "head"), want["head"], rtol=1e-5, atol=1e-30)
+    assert hostnet.chain_forward_count() == before + 2   # c1..c3 in one launch per pass
+    np.testing.assert_array_equal(net.run("data", x, "c3"), want["c3"])
+    assert hostnet.chain_forward_count() == before + 4
+    # a blob inside the run: every pass computes from scratch, the layers up to that blob one by one
+    np.testing.assert_array_equal(net.run("data", x, "c2"), want["c2"])
+    np.testing.assert_array_equal(net.run("data", x, "c1"), want["c1"])
+    assert hostnet.chain_forward_count() == before + 4
+
+
+@pytest.mark.gpu
 def test_net_residual_block_with_auto_split(oracle):
     """A MobileNetV2-style inverted residual: the block input feeds the expand conv AND the element-wise add, so the
     graph builder must insert a Split; the project conv feeds the add, so it stays fp32."""

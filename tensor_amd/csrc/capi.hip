@@ -636,8 +636,10 @@ int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_l
             eps[l] = make_epilogue(handles[l], OTTER_HIP_I8_P8);
             wpk[l] = handles[l]->w_igemm;
         }
-        OHIP_CHECK(run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream));
-        return OTTER_HIP_OK;
+        const hipError_t ce = run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream);
+        if (ce == hipSuccess) return OTTER_HIP_OK;
+        if (ce != hipErrorNotReady) OHIP_CHECK(ce);
+        // (every flag set of this GPU belongs to another stream: this stream takes the layers one by one)
     }
     // anything else: the layers one after the other, the same blobs
     for (int l = 0; l < n_layers; ++l) {

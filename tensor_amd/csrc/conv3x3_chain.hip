@@ -24,6 +24,8 @@
 //     passed s_waitcnt vmcnt(0) by then, so all of the tile's stores have been acknowledged by L2.
 //   * Each layer writes a buffer nobody has read before in this launch (the caller provides layers - 1 intermediate
 //     buffers), so a compute unit's vector L1 cannot hold a stale line of what it is about to read.
+#include <mutex>
+
 #include "common.hpp"
 #include "conv_igemm.hpp"
 
@@ -43,8 +45,11 @@ constexpr int CHAIN_MAX_FLAGS = 1 << 16;   // tiles of all layers
 constexpr int CHAIN_SPIN_LIMIT = 1 << 17;  // polls of a producer flag before giving up (~0.1 s)
 
 // per-device state of the chain launches: tile flags (epoch numbers), one queue counter per XCD, exit counter, error word
-__device__ int g_chain_flags[CHAIN_MAX_FLAGS];
-__device__ int g_chain_ctl[16];  // [0..7] queue counters, [8] workgroups that have left, [9] error
+// One set of flags and counters per stream that uses the entry point, for up to CHAIN_SLOTS streams per GPU: launches on
+// different streams may overlap and must not share them.
+constexpr int CHAIN_SLOTS = 4;
+__device__ int g_chain_flags[CHAIN_SLOTS * CHAIN_MAX_FLAGS];
+__device__ int g_chain_ctl[CHAIN_SLOTS * 16];  // per slot: [0..7] queue counters, [8] workgroups that have left, [9] error
 
 struct ChainArgs {
     const int8_t* act[CHAIN_MAX_LAYERS + 1];  // act[l]: input of layer l; act[l + 1]: its output
@@ -403,10 +408,14 @@ constexpr int kChainPrmBytes = 3 * 128 * 4 + 64;
 struct ChainDevice {
     int* flags = nullptr;
     int* ctl = nullptr;
-    int epoch = 0;
     int xcds = 0;
+    // slot -> the stream that owns it (first come, for the life of the process) and that stream's launch count
+    hipStream_t stream[CHAIN_SLOTS] = {};
+    bool used[CHAIN_SLOTS] = {};
+    int epoch[CHAIN_SLOTS] = {};
 };
 ChainDevice g_chain_dev[16];
+std::mutex g_chain_mutex;
 
 }  // namespace
 
@@ -436,14 +445,25 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     ChainDevice& cd = g_chain_dev[dev];
-    if (!cd.flags) {
-        void *pf = nullptr, *pc = nullptr;
-        if ((e = hipGetSymbolAddress(&pf, HIP_SYMBOL(g_chain_flags))) != hipSuccess) return e;
-        if ((e = hipGetSymbolAddress(&pc, HIP_SYMBOL(g_chain_ctl))) != hipSuccess) return e;
-        hipDeviceProp_t prop;
-        if ((e = hipGetDeviceProperties(&prop, dev)) != hipSuccess) return e;
-        cd.flags = (int*)pf, cd.ctl = (int*)pc;
-        cd.xcds = std::max(1, std::min(8, prop.multiProcessorCount / 32));
+    int slot = -1, epoch = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_chain_mutex);
+        if (!cd.flags) {
+            void *pf = nullptr, *pc = nullptr;
+            if ((e = hipGetSymbolAddress(&pf, HIP_SYMBOL(g_chain_flags))) != hipSuccess) return e;
+            if ((e = hipGetSymbolAddress(&pc, HIP_SYMBOL(g_chain_ctl))) != hipSuccess) return e;
+            hipDeviceProp_t prop;
+            if ((e = hipGetDeviceProperties(&prop, dev)) != hipSuccess) return e;
+            cd.flags = (int*)pf, cd.ctl = (int*)pc;
+            cd.xcds = std::max(1, std::min(8, prop.multiProcessorCount / 32));
+        }
+        for (int i = 0; i < CHAIN_SLOTS && slot < 0; ++i)
+            if (cd.used[i] && cd.stream[i] == stream) slot = i;
+        for (int i = 0; i < CHAIN_SLOTS && slot < 0; ++i)
+            if (!cd.used[i]) cd.used[i] = true, cd.stream[i] = stream, slot = i;
+        if (slot < 0) return hipErrorNotReady;  // more streams than slots: the caller runs the layers one by one
+        epoch = ++cd.epoch[slot];
+        if (cd.epoch[slot] == 0x7fffffff) cd.epoch[slot] = 0;  // (flags of 2^31 launches ago could alias; unreachable)
     }
     ChainArgs ca;
     for (int l = 0; l < layers; ++l) {
@@ -453,9 +473,8 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
         ca.act_hi[l] = eps[l].act_hi, ca.act_p0[l] = eps[l].act_p0, ca.lrelu[l] = eps[l].lrelu ? 1 : 0;
     }
     ca.act[layers] = act[layers];
-    ca.layers = layers, ca.xcds = cd.xcds, ca.epoch = ++cd.epoch;
-    ca.flags = cd.flags, ca.ctl = cd.ctl;
-    if (cd.epoch == 0x7fffffff) cd.epoch = 0;  // (flags of 2^31 launches ago could alias; unreachable in practice)
+    ca.layers = layers, ca.xcds = cd.xcds, ca.epoch = epoch;
+    ca.flags = cd.flags + (size_t)slot * CHAIN_MAX_FLAGS, ca.ctl = cd.ctl + slot * 16;
     const int fn = plan[0], r_max = plan[1], tpi = plan[2], logp = plan[3];
     const int epi = pick_epilogue(eps[0], g.K);
     const unsigned act_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W);
@@ -506,11 +525,15 @@ hipError_t conv3x3_chain_error(int* error_word) {
     if (e != hipSuccess) return e;
     *error_word = 0;
     if (dev < 0 || dev >= 16 || !g_chain_dev[dev].ctl) return hipSuccess;
-    int ctl[16];
+    int ctl[CHAIN_SLOTS * 16];
     if ((e = hipMemcpy(ctl, g_chain_dev[dev].ctl, sizeof(ctl), hipMemcpyDeviceToHost)) != hipSuccess) return e;
-    *error_word = ctl[9];
-    if (ctl[9] || ctl[8] || ctl[0]) {  // a launch that gave up (or was cut short) leaves the counters dirty: rewind
-        int zeros[16] = {0};
+    bool dirty = false;
+    for (int s = 0; s < CHAIN_SLOTS; ++s) {
+        *error_word |= ctl[s * 16 + 9];
+        dirty = dirty || ctl[s * 16 + 9] || ctl[s * 16 + 8] || ctl[s * 16];
+    }
+    if (dirty) {  // a launch that gave up (or was cut short) leaves the counters dirty: rewind
+        int zeros[CHAIN_SLOTS * 16] = {0};
         if ((e = hipMemcpy(g_chain_dev[dev].ctl, zeros, sizeof(zeros), hipMemcpyHostToDevice)) != hipSuccess) return e;
     }
     return hipSuccess;

@@ -99,6 +99,33 @@ def test_same_shape_chain_that_needs_two_lds_stages_runs_layer_by_layer(hip):
     np.testing.assert_array_equal(hip.conv_chain(convs, xd, N, H, W).cpu().numpy(), want)
 
 
+def test_chains_on_several_streams_at_once(hip):
+    """Every stream that uses the entry point gets a flag set of its own (four per GPU); launches on different streams
+    may overlap. Six streams each run their own chain, enqueued back to back without a synchronisation in between: the
+    first four as one launch each, the last two layer by layer (no flag set left) - every result equals the layers one
+    by one."""
+    torch = hip.torch
+    rng = np.random.default_rng(21)
+    N, C, H, W, L = 8, 128, 28, 28, 4
+    jobs = []
+    for j in range(6):
+        convs, _ = _layers(hip, rng, [C] * (L + 1), act=1)
+        x = rng.integers(-127, 128, size=(N, C, H, W), dtype=np.int8)
+        xd = hip.to_device(capi.pack_np(x, 8))
+        want = _one_by_one(hip, convs, xd, N, H, W).cpu().numpy()
+        jobs.append((convs, xd, want, torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    outs = []
+    for rep in range(3):
+        outs = []
+        for convs, xd, want, st in jobs:
+            with torch.cuda.stream(st):
+                outs.append(hip.conv_chain(convs, xd, N, H, W))
+    assert not hip.conv_chain_gave_up()  # (synchronizes the device)
+    for (convs, xd, want, st), got in zip(jobs, outs):
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
 def test_chain_argument_checks(hip):
     rng = np.random.default_rng(6)
     convs, _ = _layers(hip, rng, [16, 32])

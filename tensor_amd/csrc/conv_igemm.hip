@@ -84,20 +84,39 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     const int HW = g.H * g.W;
 
     // ---- per-thread constants of the activation loader -------------------------------------------
+    // (image, pixel) of a global pixel index: the tile's first pixel is divided once for the whole workgroup (uniform
+    // operands), a lane then only steps over at most one image boundary; images smaller than a tile take the division
+    const unsigned n_tile = tile_base / (unsigned)OHW;
+    const unsigned rem_tile = tile_base - n_tile * (unsigned)OHW;
+    auto locate = [&](unsigned ofs, unsigned& n, unsigned& pix) {  // pixel tile_base + ofs, ofs < TN
+        n = n_tile, pix = rem_tile + ofs;
+        if ((unsigned)OHW >= (unsigned)TN) {
+            if (pix >= (unsigned)OHW) pix -= (unsigned)OHW, ++n;
+        } else {
+            const unsigned k = pix / (unsigned)OHW;
+            n += k, pix -= k * (unsigned)OHW;
+        }
+    };
+    // a pointwise layer (1x1, stride 1, no padding) reads input pixel = output pixel: no row / column split, no bounds
+    const bool pointwise = g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0;
     const int p_l = tid % TN;
     const int j0 = tid / TN;
     constexpr int J_STEP = 256 / TN > 0 ? 256 / TN : 1;
-    const unsigned gp = tile_base + p_l;
-    const bool pvalid = gp < total_pix;
+    const bool pvalid = tile_base + p_l < total_pix;
     int iy0 = 0, ix0 = 0;
-    const int8_t* xn = x;
+    const int8_t* px00 = x;  // this thread's pixel at tap (0, 0), octet 0 (only dereferenced where in bounds)
     if (pvalid) {
-        const int n = (int)(gp / (unsigned)OHW);
-        const int pix = (int)(gp - (unsigned)n * (unsigned)OHW);
-        const int oy = (int)((unsigned)pix / (unsigned)g.OW), ox = pix - oy * g.OW;
-        iy0 = oy * g.sh - g.ph;
-        ix0 = ox * g.sw - g.pw;
-        xn = x + (size_t)n * Cs8 * HW * 8;
+        unsigned n, pix;
+        locate((unsigned)p_l, n, pix);
+        const int8_t* xn = x + (size_t)n * Cs8 * HW * 8;
+        if (pointwise) {
+            px00 = xn + (size_t)pix * 8;
+        } else {
+            const int oy = (int)(pix / (unsigned)g.OW), ox = (int)pix - oy * g.OW;
+            iy0 = oy * g.sh - g.ph;
+            ix0 = ox * g.sw - g.pw;
+            px00 = xn + ((ptrdiff_t)iy0 * g.W + ix0) * 8;
+        }
     }
 
     v2i breg[KC][Cfg::B_V][2];
@@ -107,9 +126,12 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     auto load_global = [&](int kc, int q) {
         const int tap = kc / c_groups, cgp = kc % c_groups;
         const int u = tap / g.kw, v = tap % g.kw;
-        const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
-        const bool inb = pvalid && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-        const int8_t* px = xn + ((size_t)iy * g.W + ix) * 8;
+        bool inb = pvalid;
+        if (!pointwise) {
+            const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
+            inb = pvalid && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+        }
+        const int8_t* px = px00 + ((ptrdiff_t)(u * g.dh) * g.W + v * g.dw) * 8;  // (uniform offset)
 #pragma unroll
         for (int r = 0; r < Cfg::B_V; ++r) {
             const int o0 = cgp * 8 + 2 * (j0 + r * J_STEP);
@@ -141,12 +163,9 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     };
 
     v4i acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    auto multiply = [&](int buf) {
+    // first: the accumulators start from the constant zero instead of being cleared beforehand
+    auto multiply = [&](int buf, bool first) {
         v4i a[FM], b[FN];
 #pragma unroll
         for (int i = 0; i < FM; ++i)
@@ -155,11 +174,19 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         for (int j = 0; j < FN; ++j)
             b[j] = *reinterpret_cast<const v4i*>(
                 &lds_b[buf][((lane >> 4) * TN + wn * (TN / WN) + j * 16 + (lane & 15)) * 16]);
+        if (first) {
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], v4i{0, 0, 0, 0}, 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
     };
     if constexpr (KC == 1) {
         load_global(0, 0);
@@ -168,7 +195,8 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         for (int kc = 0; kc < n_chunks; ++kc) {
             const int buf = kc & 1;
             if (kc + 1 < n_chunks) load_global(kc + 1, 0);
-            multiply(buf);
+            if (kc == 0) multiply(buf, true);
+            else multiply(buf, false);
             if (kc + 1 < n_chunks) store_lds(buf ^ 1, 0);
             __syncthreads();
         }
@@ -188,7 +216,10 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                 if (k1 + q < n_chunks) load_global(k1 + q, q);
 #pragma unroll
             for (int q = 0; q < KC; ++q)
-                if (k0 + q < n_chunks) multiply(q);
+                if (k0 + q < n_chunks) {
+                    if (k0 + q == 0) multiply(q, true);
+                    else multiply(q, false);
+                }
             if (k1 < n_chunks) {
                 __syncthreads();  // everyone has read this stage
 #pragma unroll
@@ -204,8 +235,8 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     // image and pixel of this lane's first column; the other columns are 16, 32, ... pixels further: one division per
     // lane instead of one per column (a 32-bit division is ~20 vector instructions)
     const unsigned gp0 = tile_base + wn * (TN / WN) + (lane & 15);
-    const unsigned n0 = gp0 / (unsigned)OHW;
-    const unsigned pix0 = gp0 - n0 * (unsigned)OHW;
+    unsigned n0, pix0;
+    locate((unsigned)(wn * (TN / WN) + (lane & 15)), n0, pix0);
     const bool wide = (unsigned)OHW >= 16u * FN;  // then a column is at most one image further than the first
     if constexpr (EPI == EPI_F32_P4 || EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
         // Packed outputs without the fused extras. A lane's stores differ by a column offset (image, pixel) and a row

@@ -344,6 +344,45 @@ def test_random_shapes_against_oracle(hip, oracle, C, K, k, s, p, d, g, N, H, W)
             assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_drawn_geometries_against_oracle(hip, oracle, seed):
+    """Eight geometries per seed drawn from the whole domain of the layer (kernel 1..5, stride 1..2, dilation 1..2,
+    padding 0..dilation*(k/2), dense / grouped / depthwise, channel counts that are and are not multiples of 8 and 4,
+    int8 and fp32 inputs, odd sizes), whatever kernel each one routes to: int8 result bit for bit, fp32 within 1e-5."""
+    rng = np.random.default_rng(1000 + seed)
+    done = 0
+    while done < 8:
+        k = int(rng.choice([1, 3, 3, 3, 5]))
+        s = int(rng.integers(1, 3))
+        d = 1 if k == 1 else int(rng.integers(1, 3))
+        p = int(rng.integers(0, d * (k // 2) + 1))
+        kind = rng.choice(["dense", "dense", "grouped", "depthwise"])
+        if kind == "dense":
+            C, K, g = int(rng.choice([8, 16, 24, 40, 64, 72, 128, 12, 3])), int(rng.choice([8, 16, 20, 32, 64, 96, 136, 10])), 1
+        elif kind == "grouped":
+            g = int(rng.choice([2, 4]))
+            C, K = g * int(rng.choice([8, 16, 4])), g * int(rng.choice([8, 16, 12]))
+        else:
+            C = K = g = int(rng.choice([8, 16, 24, 64, 6]))
+        N, H, W = int(rng.integers(1, 4)), int(rng.integers(5, 30)), int(rng.integers(5, 70))
+        if (H + 2 * p - d * (k - 1) - 1) // s + 1 < 1 or (W + 2 * p - d * (k - 1) - 1) // s + 1 < 1:
+            continue
+        done += 1
+        x, wq, ws, bias = _rand_problem(rng, C, K, k, g, N, H, W, in_i8=bool(rng.integers(0, 2)))
+        in_scale = 20.0 if x.dtype == np.int8 else 100.0
+        act = int(rng.choice([0, 1, 2, 3]))
+        int8_out = bool(rng.integers(0, 2))
+        what = (C, K, k, s, p, d, g, N, H, W, str(x.dtype), act, int8_out)
+        want = oracle.conv_layer_forward(x, wq, ws, in_scale, stride=(s, s), pad=(p, p), dil=(d, d), groups=g, bias=bias,
+                                         top_scale=11.0, int8_out=int8_out, act_type=act, act_params=[0.25])
+        out, _ = run_conv(hip, oracle, x, wq, ws, in_scale, stride=s, pad=p, dil=d, groups=g, bias=bias, top_scale=11.0,
+                          act=act, act_p0=0.25, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        if int8_out:
+            np.testing.assert_array_equal(out, want, err_msg=str(what))
+        else:
+            np.testing.assert_allclose(out, want, rtol=FP32_RTOL, atol=1e-30, err_msg=str(what))
+
+
 @pytest.mark.parametrize("shift", [0, 1, 2])
 @pytest.mark.parametrize("s", [1, 2])
 @pytest.mark.parametrize("family", [-2, -3], ids=["mfma", "valu"])

@@ -289,6 +289,7 @@ LAYER_SHAPES = {
     "grp8": (256, 256, 3, 1, 1, 1, 8, 64, 28, 28, "grouped (8 groups of 32->32) 3x3 256->256"),
     "s2": (128, 128, 3, 2, 1, 1, 1, 64, 56, 56, "3x3 stride 2 128->128"),
     "odd55": (128, 128, 3, 1, 1, 1, 1, 64, 55, 55, "3x3 128->128 on an odd image width"),
+    "w224": (64, 64, 3, 1, 1, 1, 1, 8, 224, 224, "3x3 64->64 on 224-pixel rows"),
 }
 
 

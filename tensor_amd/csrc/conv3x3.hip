@@ -16,6 +16,7 @@
 //   * the MFMA "A" operand (weights) is read straight from global memory, already in MFMA lane order
 //     (igemm_pack_weights), one coalesced 1 KB read per 16x64 fragment, prefetched two k-chunks ahead. Every
 //     workgroup reads the same <= 147 KB of weights, so they stay in L2.
+// Rows of up to 252 pixels take 2048-byte lines (two transfers per line; stride 1 and dilation 1 only).
 // An odd image width ends on half a pixel pair: the transfer then brings the first pixel of the next row along, and the
 // wave that issued it overwrites that pixel with zeros once its transfers have landed, before the barrier.
 // The input must stay below 2 GiB (32-bit offsets).
@@ -104,7 +105,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                     }
                 }
             }
-        } else {
+        } else if constexpr (LOGP == 10) {
             const bool col_ok = lane >= 1 && 2 * lane - 2 < g.W;  // lane: pixels 2*lane-2 and 2*lane-1
             const unsigned v_col = col_ok ? (unsigned)(2 * lane - 2) * 8u : HALO_OOB;
             if (2 * lane < EW) {
@@ -118,6 +119,32 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                         __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, (__attribute__((address_space(3))) void*)dst, 16,
                                                                  (int)(ok ? v_col : HALO_OOB), (int)s_off, 0, 0);
                     }
+                }
+            }
+        } else {
+            // 2048-byte lines (rows of up to 252 pixels): two transfers per line, 1 KB = 128 pixels each
+            constexpr int SEGS = 1 << (LOGP - 10);
+            unsigned v_col[SEGS];
+            bool seg_on[SEGS];
+#pragma unroll
+            for (int sg = 0; sg < SEGS; ++sg) {
+                const int pl = lane + 64 * sg;  // pixel pair: pixels 2*pl-2 and 2*pl-1
+                const bool col_ok = pl >= 1 && 2 * pl - 2 < g.W;
+                v_col[sg] = col_ok ? (unsigned)(2 * pl - 2) * 8u : HALO_OOB;
+                seg_on[sg] = 2 * pl < EW;
+            }
+            for (int oc = wave; oc < cb / 8; oc += 4) {
+                const int o = cb0 / 8 + oc;
+                for (int r = 0; r < R; ++r) {
+                    const int iy = r_lo * S - g.ph + r;
+                    const bool ok = o < C8 && iy >= 0 && iy < g.H;  // wave-uniform
+                    const unsigned s_off = ok ? (unsigned)((n * C8 + o) * g.H + iy) * (unsigned)(g.W * 8) : 0u;
+                    int8_t* dst = lds + (size_t)(oc >> 1) * pair_bytes + (size_t)((2 * r + (oc & 1)) << LOGP);
+#pragma unroll
+                    for (int sg = 0; sg < SEGS; ++sg)
+                        if (seg_on[sg])
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(rin, (__attribute__((address_space(3))) void*)(dst + 1024 * sg),
+                                                                     16, (int)(ok ? v_col[sg] : HALO_OOB), (int)s_off, 0, 0);
                 }
             }
         }
@@ -406,6 +433,10 @@ hipError_t launch_halo_e(const int8_t* x, const int8_t* wpk, void* out, const Co
     }
     if (g.sh != 1 || g.dh != 1) return hipErrorInvalidValue;
     if (pl.logp == 9) return launch_halo_p<FM, FN, WM, WN, EPI, 9, 1, 1>(x, wpk, out, g, ep, pl, stream);
+    if (pl.logp == 11) {
+        if constexpr (FN <= 6) return launch_halo_p<FM, FN, WM, WN, EPI, 11, 1, 1>(x, wpk, out, g, ep, pl, stream);
+        return hipErrorInvalidValue;  // (the planner gives such rows at most 6 fragments)
+    }
     return launch_halo_p<FM, FN, WM, WN, EPI, 10, 1, 1>(x, wpk, out, g, ep, pl, stream);
 }
 
@@ -432,13 +463,16 @@ bool plan_halo(const ConvGeom& g, int force_fn, HaloPlan* best) {
     const int cpad = igemm_channel_groups(g.C) * 64;
     const bool wide = igemm_padded_rows(g.K) > 64;
     const int m_blocks = wide ? (igemm_padded_rows(g.K) / 16 + 7) / 8 : 1;
-    // LDS line pitch: 512 bytes hold rows of up to 60 pixels (+4 padding pixels), 1024 bytes up to 124
-    const int logp = (g.W + 4) * 8 <= 512 ? 9 : 10;
+    // LDS line pitch: 512 bytes hold rows of up to 60 pixels (+4 padding pixels), 1024 bytes up to 124, 2048 bytes up to
+    // 252 (stride 1, dilation 1 only)
+    const int logp = (g.W + 4) * 8 <= 512 ? 9 : ((g.W + 4) * 8 <= 1024 ? 10 : 11);
     if ((g.W + 4) * 8 > (1 << logp)) return false;
+    if (logp == 11 && (g.sh != 1 || g.dh != 1)) return false;
     bool found = false;
     for (int fn = 4; fn <= 7; ++fn) {  // 8 fragments would spill at two waves per SIMD
         if (force_fn && fn != force_fn) continue;
-        if (fn == 7 && (g.W & 1)) continue;  // odd widths: at most 6 fragments (see the kernel's ODDW parameter)
+        // odd widths and 2048-byte lines: at most 6 fragments (the 7-fragment tile has no register to spare for them)
+        if (fn == 7 && ((g.W & 1) || logp == 11)) continue;
         const int pt = (wide ? 32 : 64) * fn;
         HaloPlan p;
         p.fn = fn;

@@ -424,6 +424,7 @@ bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers,
     if (layers < 2 || layers > CHAIN_MAX_LAYERS) return false;
     if (g.C != g.K || g.ph != 1 || g.pw != 1 || g.OH != g.H || g.OW != g.W) return false;
     if (g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1) return false;
+    if ((g.W + 4) * 8 > 1024) return false;  // LDS lines of 512 and 1024 bytes only
     if (igemm_padded_rows(g.K) != 128) return false;  // 65..128 output channels: one row block of four wave tiles
     if (!conv3x3_halo_supported(g, ep)) return false;
     const int epi = pick_epilogue(ep, g.K);

@@ -225,14 +225,16 @@ def test_igemm_every_tile_shape(hip, oracle, tile, stage):
 @pytest.mark.parametrize("fn", [4, 5, 6, 7])
 def test_halo3x3_every_fragment_count(hip, oracle, fn):
     """The 3x3 stride-1 LDS-halo MFMA kernel: wide (K > 64) and narrow wave layouts, padded channel counts, pad 0 and 1,
-    ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at once), both LDS line pitches
-    (up to 60 columns and up to 124), several tiles per workgroup, odd image widths (the last pixel pair of a row is
+    ragged last tile, several channel blocks (C = 320 at 30 columns does not fit LDS at once), the three LDS line pitches
+    (up to 60, 124 and 252 columns), several tiles per workgroup, odd image widths (the last pixel pair of a row is
     half padding: both pitches, the widest rows of either, the last row of the tensor, an odd octet count)."""
     rng = np.random.default_rng(fn)
     for (C, K, p, N, H, W) in [(128, 128, 1, 2, 19, 22), (64, 64, 1, 1, 56, 56), (72, 24, 0, 2, 11, 10),
                                (16, 160, 1, 1, 7, 8), (320, 96, 1, 1, 14, 30), (8, 16, 1, 1, 9, 66),
                                (16, 136, 1, 3, 5, 124), (128, 128, 1, 2, 13, 55), (24, 64, 1, 3, 9, 59),
-                               (64, 40, 0, 1, 7, 123), (8, 32, 1, 2, 5, 7), (32, 96, 0, 1, 6, 61)]:
+                               (64, 40, 0, 1, 7, 123), (8, 32, 1, 2, 5, 7), (32, 96, 0, 1, 6, 61),
+                               (64, 128, 1, 1, 6, 125), (16, 72, 1, 2, 5, 252), (128, 64, 0, 1, 4, 201),
+                               (24, 32, 1, 1, 3, 130)]:
         x, wq, ws, bias = _rand_problem(rng, C, K, 3, 1, N, H, W)
         in_scale = 25.0
         for int8_out in (True, False):

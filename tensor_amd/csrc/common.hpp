@@ -346,7 +346,8 @@ __device__ __forceinline__ ohip_v4i epi4_dequant_f32p4(const Epilogue& ep, const
 // dequantize (+clamp activation) 4 channels and store one Float4 element. FUSED: first add the residual blob's element
 // if the epilogue carries one, and return the four bytes of the blob's int8 twin (float2int8(v * twin_scale)) if it
 // carries one
-template <bool FUSED = false>
+// LRELU: 0 = clamp activation only, 1 = LeakyReLU, -1 = decided by ep.lrelu at run time (a select per value)
+template <bool FUSED = false, int LRELU = -1>
 __device__ __forceinline__ unsigned epi4_store_f32p4(float* __restrict__ out, const Epilogue& ep, const float* si,
                                                      const float* bi, size_t elem, int a0, int a1, int a2, int a3) {
     const int a[4] = {a0, a1, a2, a3};
@@ -358,8 +359,10 @@ __device__ __forceinline__ unsigned epi4_store_f32p4(float* __restrict__ out, co
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float v = __fmaf_rn((float)a[e], si[e], bi[e]);
-        v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);
-        if (ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch; the clamp above is open then
+        if constexpr (LRELU != 1) v = fminf(fmaxf(v, ep.act_lo), ep.act_hi);  // (open for LeakyReLU)
+        if constexpr (LRELU != 0) {
+            if (LRELU == 1 || ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform
+        }
         if constexpr (FUSED) {
             if (ep.residual != nullptr) v = __fadd_rn(v, __int_as_float(res[e]));
             if (ep.twin != nullptr) {  // wave-uniform

@@ -238,16 +238,18 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     unsigned n0, pix0;
     locate((unsigned)(wn * (TN / WN) + (lane & 15)), n0, pix0);
     const bool wide = (unsigned)OHW >= 16u * FN;  // then a column is at most one image further than the first
-    if constexpr (EPI == EPI_F32_P4 || EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
-        // Packed outputs without the fused extras. A lane's stores differ by a column offset (image, pixel) and a row
+    if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P4_FUSED || EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG) {
+        // Packed outputs. A lane's stores differ by a column offset (image, pixel) and a row
         // offset (channel group): each computed once, one 64-bit addition per store. LeakyReLU is decided once, in
         // front of the unrolled loops, not per value.
-        constexpr bool F32 = EPI == EPI_F32_P4;
+        constexpr bool FUSED = EPI == EPI_F32_P4_FUSED;  // plus the residual addend and / or the int8 twin
+        constexpr bool F32 = EPI == EPI_F32_P4 || FUSED;
         constexpr int EB = F32 ? 16 : 8;       // bytes of one (pixel, channel group) element
         constexpr int CG = F32 ? 4 : 8;        // channels per group
         const size_t plane = (size_t)OHW * EB;  // one channel group of one image
         const size_t image = plane * (size_t)(Ks / CG);
         size_t col_ofs[FN];
+        unsigned col_twin[FUSED ? FN : 1];  // the same for the Byte8 twin (below 2 GiB)
         bool col_ok[FN];
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
@@ -261,6 +263,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             }
             col_ok[j] = gpo < total_pix;
             col_ofs[j] = (size_t)nn * image + (size_t)pp * EB;
+            if constexpr (FUSED) col_twin[j] = (nn * (unsigned)(Ks / 8) * (unsigned)OHW + pp) * 8u;
         }
         auto rows = [&](auto lrelu_c) {
             constexpr bool LRELU = decltype(lrelu_c)::value;
@@ -271,7 +274,8 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                 const bool ch_ok = ch0 < g.K;
                 Epi8 prm;
                 epi8_load<EPI>(prm, ep, ch0);  // arrays are padded to the padded rows
-                char* row = (char*)out + (size_t)(ch0 / CG) * plane;
+                const size_t row_ofs = (size_t)(ch0 / CG) * plane;
+                char* row = (char*)out + row_ofs;
 #pragma unroll
                 for (int j = 0; j < FN; ++j) {
                     int a8[8];
@@ -282,7 +286,17 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                     }
                     if (ch_ok && col_ok[j]) {
                         char* o = row + col_ofs[j];
-                        if constexpr (F32) {
+                        if constexpr (FUSED) {
+                            const size_t elem = (row_ofs + col_ofs[j]) >> 2;  // in floats, for the result and the addend
+                            ohip_v2i tw = {0, 0};
+                            tw[0] = (int)epi4_store_f32p4<true, LRELU ? 1 : 0>((float*)out, ep, prm.si, prm.bi, elem, a8[0], a8[1],
+                                                                              a8[2], a8[3]);
+                            if (ch0 + 4 < g.K)
+                                tw[1] = (int)epi4_store_f32p4<true, LRELU ? 1 : 0>((float*)out, ep, prm.si + 4, prm.bi + 4,
+                                                                                  elem + (plane >> 2), a8[4], a8[5], a8[6], a8[7]);
+                            if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
+                                *reinterpret_cast<ohip_v2i*>(ep.twin + (size_t)(ch0 / 8) * OHW * 8 + col_twin[j]) = tw;
+                        } else if constexpr (F32) {
                             *reinterpret_cast<ohip_v4i*>(o) =
                                 epi4_dequant_f32p4<LRELU>(ep, prm.si, prm.bi, a8[0], a8[1], a8[2], a8[3]);
                             if (ch0 + 4 < g.K)
@@ -324,17 +338,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
                         pp = gpo - nn * (unsigned)OHW;
                     }
                     const int n = (int)nn, pix = (int)pp;
-                    if constexpr (EPI == EPI_F32_P4_FUSED) {
-                        ohip_v2i tw = {0, 0};
-                        tw[0] = (int)epi4_store_f32p4<true>((float*)out, ep, prm.si, prm.bi,
-                                                            elem_offset(4, n, ch0, pix, Ks, OHW), a8[0], a8[1], a8[2], a8[3]);
-                        if (ch0 + 4 < g.K)
-                            tw[1] = (int)epi4_store_f32p4<true>((float*)out, ep, prm.si + 4, prm.bi + 4,
-                                                                elem_offset(4, n, ch0 + 4, pix, Ks, OHW), a8[4], a8[5], a8[6],
-                                                                a8[7]);
-                        if (ep.twin != nullptr)  // K % 8 == 0 then: the lane's 8 channels are one Byte8 element
-                            *reinterpret_cast<ohip_v2i*>(ep.twin + elem_offset(8, n, ch0, pix, Ks, OHW)) = tw;
-                    } else {
+                    {
                         epilogue_store8_generic(out, &ep, n, ch0, pix, g.K, OHW, a8[0], a8[1], a8[2], a8[3], a8[4], a8[5],
                                                 a8[6], a8[7]);
                     }

@@ -391,6 +391,13 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
         // the last workgroup to leave rewinds the queues for the next launch
         const int left = __hip_atomic_fetch_add(ca.ctl + 8, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (left == (int)gridDim.x - 1) {
+            // every list must have been walked to its end: a list whose XCD received no workgroup of this launch would
+            // otherwise go unnoticed (the host sizes the grid so that this does not happen; the status call reports it)
+            for (int xc = 0; xc < ca.xcds; ++xc) {
+                const int len = ((g.N - xc + ca.xcds - 1) / ca.xcds) * tiles_per_img * ca.layers;
+                if (__hip_atomic_load(ca.ctl + xc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < len)
+                    __hip_atomic_store(ca.ctl + 9, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             for (int i = 0; i < 9; ++i) __hip_atomic_store(ca.ctl + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }

@@ -104,20 +104,26 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     constexpr int J_STEP = 256 / TN > 0 ? 256 / TN : 1;
     const bool pvalid = tile_base + p_l < total_pix;
     int iy0 = 0, ix0 = 0;
-    const int8_t* px00 = x;  // this thread's pixel at tap (0, 0), octet 0 (only dereferenced where in bounds)
+    // this thread's pixel at tap (0, 0), octet 0, as a byte offset into the (group's slice of the) input; the loads go
+    // through a buffer descriptor, so that an out-of-image tap or a padded octet is an out-of-range offset (reads as
+    // zero) instead of a branch around the load
+    int px_ofs = 0;
     if (pvalid) {
         unsigned n, pix;
         locate((unsigned)p_l, n, pix);
-        const int8_t* xn = x + (size_t)n * Cs8 * HW * 8;
+        const int img = (int)n * Cs8 * HW * 8;
         if (pointwise) {
-            px00 = xn + (size_t)pix * 8;
+            px_ofs = img + (int)pix * 8;
         } else {
             const int oy = (int)(pix / (unsigned)g.OW), ox = (int)pix - oy * g.OW;
             iy0 = oy * g.sh - g.ph;
             ix0 = ox * g.sw - g.pw;
-            px00 = xn + ((ptrdiff_t)iy0 * g.W + ix0) * 8;
+            px_ofs = img + (iy0 * g.W + ix0) * 8;
         }
     }
+    constexpr unsigned IG_OOB = 0x80000000u;
+    const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t*>(x), 0, (int)((unsigned)g.N * (unsigned)Cs8 * (unsigned)HW * 8u - (unsigned)blockIdx.z * (unsigned)(g.C / 8) * (unsigned)HW * 8u), 0x00020000);
 
     v2i breg[KC][Cfg::B_V][2];
     v4i areg[KC][Cfg::A_V];
@@ -131,15 +137,14 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
             inb = pvalid && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
         }
-        const int8_t* px = px00 + ((ptrdiff_t)(u * g.dh) * g.W + v * g.dw) * 8;  // (uniform offset)
+        const int tap_ofs = ((u * g.dh) * g.W + v * g.dw) * 8;  // (uniform)
 #pragma unroll
         for (int r = 0; r < Cfg::B_V; ++r) {
             const int o0 = cgp * 8 + 2 * (j0 + r * J_STEP);
-            v2i lo = {0, 0}, hi = {0, 0};
-            if (inb && o0 < C8) lo = *reinterpret_cast<const v2i*>(px + (size_t)o0 * HW * 8);
-            if (inb && o0 + 1 < C8) hi = *reinterpret_cast<const v2i*>(px + (size_t)(o0 + 1) * HW * 8);
-            breg[q][r][0] = lo;
-            breg[q][r][1] = hi;
+            const unsigned v_lo = (unsigned)(px_ofs + tap_ofs + o0 * HW * 8);
+            breg[q][r][0] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(inb && o0 < C8 ? v_lo : IG_OOB), 0, 0));
+            breg[q][r][1] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(
+                rin, (int)(inb && o0 + 1 < C8 ? v_lo + (unsigned)(HW * 8) : IG_OOB), 0, 0));
         }
         const int8_t* wa = wpk + ((size_t)kc * m_tiles16 + mt0) * 1024;
 #pragma unroll

@@ -176,7 +176,7 @@ int otter_hip_conv_forward_residual(const otter_hip_conv_t* handle, const void* 
  * Net, Tensor/Net.cpp:413-505 runs them one after the other): out = layer[n-1](... layer[0](in)). The result is what
  * n calls of otter_hip_conv_forward give. The intermediate blobs live in `workspace`
  * (otter_hip_conv_chain_workspace_bytes, one buffer per intermediate blob). Where all layers are the same 3x3
- * stride-1 pad-1 geometry with 65..128 channels, the chain runs as ONE persistent launch in which a tile of a layer
+ * stride-1 pad-1 geometry with 33..128 channels, the chain runs as ONE persistent launch in which a tile of a layer
  * starts as soon as the tiles of the previous layer it reads are done; otherwise as n launches. The single launch
  * waits on flags between workgroups; every wait is bounded, and otter_hip_conv_chain_status reports (after
  * synchronizing the device) whether one ever gave up, in which case the outputs of the chain calls since the last
@@ -190,6 +190,12 @@ int otter_hip_conv_chain_status(int* gave_up);
 /* For tests and profiling: the number of convolution launches otter_hip_conv_chain_forward makes for this chain and
  * input (1: the single persistent launch; n_layers: layer by layer), or a negative status. */
 int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);
+/* Tuning / test hook with no counterpart in the reference: the single launch is only used where one layer's share
+ * of an XCD's tile list (images / 8 x tiles per image) is at least `tiles` (default 96: below that the tiles' producers
+ * are still running when they are reached, and the layers one by one are faster). 0 makes every chain that qualifies
+ * by shape a single launch (the tests do that on small shapes). Process-wide; returns the previous value; a negative
+ * argument only queries. */
+int otter_hip_conv_chain_set_min_tiles(int tiles);
 
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked

@@ -72,7 +72,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_forward_twin", "otter_hip_conv_forward_residual",
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
-           "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches"]
+           "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
+           "otter_hip_conv_chain_set_min_tiles"]
 
 
 def load_cdll():
@@ -255,6 +256,10 @@ class Library:
         r = self.lib.otter_hip_conv_chain_launches(hs, len(convs), n, h, w)
         self._check(min(r, 0))
         return r
+
+    def conv_chain_set_min_tiles(self, tiles):
+        """otter_hip_conv_chain_set_min_tiles: returns the previous threshold."""
+        return self.lib.otter_hip_conv_chain_set_min_tiles(int(tiles))
 
     def conv_chain_gave_up(self):
         """otter_hip_conv_chain_status: synchronizes; True if a chain launch since the last call gave up a wait."""

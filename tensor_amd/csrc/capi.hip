@@ -562,6 +562,8 @@ static bool chain_shapes(const otter_hip_conv_t* const* hs, int layers, int n, i
     return true;
 }
 
+static int g_chain_min_tiles = 96;  // see chain_single_launch
+
 // true when the chain runs as one persistent launch (conv3x3_chain.hip): every layer the same 3x3 stride-1 pad-1
 // geometry, same rounding and epilogue family
 static bool chain_single_launch(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {
@@ -580,7 +582,19 @@ static bool chain_single_launch(const otter_hip_conv_t* const* handles, int n_la
     for (int l = 1; l < n_layers; ++l)
         if (pick_epilogue(make_epilogue(handles[l], OTTER_HIP_I8_P8), g.K) != pick_epilogue(ep0, g.K)) return false;
     int plan[4];
-    return g.OH > 0 && g.OW > 0 && conv3x3_chain_applicable(g, ep0, n_layers, plan);
+    if (!(g.OH > 0 && g.OW > 0 && conv3x3_chain_applicable(g, ep0, n_layers, plan))) return false;
+    // The single launch pays only where a tile's producers are far enough back in an XCD's list to be finished when
+    // it is reached: 64 workgroups per XCD are in flight, and a layer's share of the list must be well above that
+    // (measured: 112 tiles per XCD and layer, the 128-channel 56x56 batch-64 stack, gains 8 %; 56 or 32 tiles lose
+    // 20-35 % against the layers one by one).
+    const long per_xcd_and_layer = (long)((n + 7) / 8) * plan[2];
+    return per_xcd_and_layer >= g_chain_min_tiles;
+}
+
+int otter_hip_conv_chain_set_min_tiles(int tiles) {
+    const int before = g_chain_min_tiles;
+    if (tiles >= 0) g_chain_min_tiles = tiles;
+    return before;
 }
 
 int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {

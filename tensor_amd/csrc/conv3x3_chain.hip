@@ -1,4 +1,4 @@
-// A chain of dense int8 3x3 stride-1 "same" convolutions (each int8 Byte8 -> int8 Byte8, same shape, 65..128 channels)
+// A chain of dense int8 3x3 stride-1 "same" convolutions (each int8 Byte8 -> int8 Byte8, same shape, 33..128 channels)
 // as ONE persistent launch of the LDS-halo kernel of conv3x3.hip.
 //
 // Launched one by one, every layer pays its own ramp and drain, and a layer whose tile count is not a multiple of the
@@ -71,18 +71,19 @@ __device__ __forceinline__ int chain_xcc_id() {
 
 }  // namespace
 
-// FM = 4 row fragments per wave, waves = 2 (channel halves) x 2 (pixel halves): 128 output channels x 32*FN pixels
-// per tile, the whole reduction staged at once (C <= 128 here). See conv3x3.hip for the data path.
-template <int FN, int EPI, int LOGP>
+// FM = 4 row fragments per wave; waves = WM (channel blocks of 64) x 4 / WM (pixel blocks): WM = 2 for 65..128 output
+// channels (128 channels x 32*FN pixels per tile), WM = 1 for 33..64 (64 channels x 64*FN pixels), the whole reduction
+// staged at once (C = K <= 128 here). See conv3x3.hip for the data path.
+template <int FN, int EPI, int LOGP, int WM>
 __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilogue ep0, ChainArgs ca, int m_tiles16,
                                                             int c_groups, int r_max, int tiles_per_img,
                                                             unsigned act_bytes) {
-    constexpr int FM = 4, WM = 2, WN = 2;
+    constexpr int FM = 4, WN = 4 / WM;
     constexpr bool NONNEG = EPI == EPI_I8_P8_NONNEG;
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     constexpr int PT = WN * FN * 16;
     constexpr int PITCH = 1 << LOGP;
-    constexpr int ROWS = WM * FM * 16;  // 128
+    constexpr int ROWS = WM * FM * 16;  // 128 or 64
     __shared__ __attribute__((aligned(16))) float lds_prm[3 * ROWS];
     __shared__ int lds_ctl[4];  // [0] next tile index (-1: none), [1] its producers are done
 
@@ -432,7 +433,7 @@ bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers,
     if (g.C != g.K || g.ph != 1 || g.pw != 1 || g.OH != g.H || g.OW != g.W) return false;
     if (g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1) return false;
     if ((g.W + 4) * 8 > 1024) return false;  // LDS lines of 512 and 1024 bytes only
-    if (igemm_padded_rows(g.K) != 128) return false;  // 65..128 output channels: one row block of four wave tiles
+    if (igemm_padded_rows(g.K) != 128 && igemm_padded_rows(g.K) != 64) return false;  // 33..128 channels: one row block
     if (!conv3x3_halo_supported(g, ep)) return false;
     const int epi = pick_epilogue(ep, g.K);
     if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG) return false;
@@ -489,9 +490,9 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
     const size_t lds_bytes = (size_t)(igemm_channel_groups(g.C) * 8) * r_max << logp;
     const long total = (long)layers * g.N * tpi;
     const int grid = (int)std::min<long>(512, std::max<long>(total, 8));
-#define OHIP_CHAIN(FN_, E_, P_)                                                                                        \
+#define OHIP_CHAIN_W(FN_, E_, P_, W_)                                                                                  \
     do {                                                                                                               \
-        auto kern = conv3x3_chain_kernel<FN_, E_, P_>;                                                                 \
+        auto kern = conv3x3_chain_kernel<FN_, E_, P_, W_>;                                                             \
         static bool attr_set = false;                                                                                  \
         if (!attr_set) {                                                                                               \
             hipError_t e2 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,        \
@@ -501,6 +502,11 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
         }                                                                                                              \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, g, eps[0], ca, igemm_padded_rows(g.K) / 16, \
                            igemm_channel_groups(g.C), r_max, tpi, act_bytes);                                          \
+    } while (0)
+#define OHIP_CHAIN(FN_, E_, P_)                                  \
+    do {                                                         \
+        if (igemm_padded_rows(g.K) == 128) OHIP_CHAIN_W(FN_, E_, P_, 2); \
+        else OHIP_CHAIN_W(FN_, E_, P_, 1);                       \
     } while (0)
 #define OHIP_CHAIN_P(FN_, E_)                   \
     do {                                        \
@@ -521,6 +527,7 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
 #undef OHIP_CHAIN_E
 #undef OHIP_CHAIN_P
 #undef OHIP_CHAIN
+#undef OHIP_CHAIN_W
     if (error_word_out) *error_word_out = 0;
     return hipGetLastError();
 }

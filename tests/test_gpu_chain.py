@@ -10,6 +10,15 @@ from tensor_amd import capi
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def every_qualifying_chain_as_one_launch(hip):
+    """By default the single launch is only taken for problems large enough to gain from it; the tests here exercise it
+    on small shapes, so the threshold is lifted for their duration."""
+    before = hip.conv_chain_set_min_tiles(0)
+    yield
+    hip.conv_chain_set_min_tiles(before)
+
+
 def quantize_weights(wf):
     K = wf.shape[0]
     ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
@@ -46,6 +55,9 @@ def _one_by_one(hip, convs, xd, n, h, w):
     (128, 64, 56, 56, 4, 1),     # the benchmark's chain
     (96, 9, 15, 55, 2, 0),       # odd width, no activation (signed results)
     (128, 3, 56, 56, 8, 1),      # fewer images than XCDs, the longest chain one launch takes
+    (64, 16, 28, 28, 4, 1),      # 64 channels: the 1 x 4 wave layout (64 channels x 64*FN pixels per tile)
+    (40, 5, 17, 30, 3, 0),       # 40 channels padded to 64 rows, ragged tiles, signed results
+    (64, 11, 56, 56, 2, 3),      # 64 channels at the benchmark's image size
 ])
 def test_same_shape_chain_is_one_launch_and_equals_the_layers_one_by_one(hip, oracle, C, N, H, W, L, act):
     rng = np.random.default_rng(C + N + H + L)
@@ -124,6 +136,19 @@ def test_chains_on_several_streams_at_once(hip):
     assert not hip.conv_chain_gave_up()  # (synchronizes the device)
     for (convs, xd, want, st), got in zip(jobs, outs):
         np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_default_rule_takes_the_single_launch_for_large_problems_only(hip):
+    """With the default threshold a chain is one launch only where a layer's share of an XCD's tile list is long (the
+    benchmark's stack: 8 images x 14 tiles = 112); small stacks of the same geometry run layer by layer."""
+    rng = np.random.default_rng(30)
+    convs, _ = _layers(hip, rng, [128] * 5, act=1)
+    hip.conv_chain_set_min_tiles(96)
+    assert hip.conv_chain_launches(convs, 64, 56, 56) == 1
+    assert hip.conv_chain_launches(convs, 16, 28, 28) == 4
+    assert hip.conv_chain_launches(convs, 8, 56, 56) == 4
+    hip.conv_chain_set_min_tiles(0)
+    assert hip.conv_chain_launches(convs, 16, 28, 28) == 1
 
 
 def test_chain_argument_checks(hip):

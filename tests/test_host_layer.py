@@ -85,6 +85,10 @@ def test_net_runs_a_stack_of_same_shape_3x3_layers_as_one_launch(oracle):
     net.set_conv("head", wh, bh, sh, scale)
     want["head"] = oracle.conv_layer_forward(cur, wh, sh, scale, bias=bh)
 
+    # (the library takes the single launch only for large problems by default: lift the threshold for this small one)
+    from tensor_amd import capi
+    int8lib = capi.load_cdll()
+    old_threshold = int8lib.otter_hip_conv_chain_set_min_tiles(0)
     # (Net.run makes two passes: one for the shape, one for the data)
     before = hostnet.chain_forward_count()
     np.testing.assert_allclose(net.run("data", x, "head"), want["head"], rtol=1e-5, atol=1e-30)
@@ -94,6 +98,9 @@ def test_net_runs_a_stack_of_same_shape_3x3_layers_as_one_launch(oracle):
     # a blob inside the run: every pass computes from scratch, the layers up to that blob one by one
     np.testing.assert_array_equal(net.run("data", x, "c2"), want["c2"])
     np.testing.assert_array_equal(net.run("data", x, "c1"), want["c1"])
+    assert hostnet.chain_forward_count() == before + 4
+    int8lib.otter_hip_conv_chain_set_min_tiles(old_threshold)
+    np.testing.assert_array_equal(net.run("data", x, "c3"), want["c3"])   # now layer by layer
     assert hostnet.chain_forward_count() == before + 4
 
 

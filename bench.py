@@ -143,7 +143,7 @@ def build_c3(hip, capi, rng):
     # the dominant kernel is the chain's one launch (all four layers' operations); when the library runs the chain
     # layer by layer it is one layer's launch
     one = launches == 1
-    return dict(name="c3", step=step, step_layers=step_layers, layer_fn=layer_fn, ops=L * ops_layer, launches=launches,
+    return dict(name="c3", step=step, step_layers=step_layers, layer_fn=layer_fn, layers=layers, ops=L * ops_layer, launches=launches,
                 dom_ops=L * ops_layer if one else ops_layer,
                 dom_bytes=2 * N * C * H * W + C * C * 9, bound="mfma",
                 workload="4 x int8 3x3 conv 128->128 s1 p1 @56x56, batch 64, int8 in/out, requantize+ReLU",

@@ -207,7 +207,8 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
  * MFMA implicit-GEMM kernel with a tile of tm output channels x tn pixels (tm in {32,64,128}, tn in
  * {64,128,256}; tn + 1 forces the kernel variant that stages one 64-deep slice of the reduction at a time, tn + 2 the
  * variant that stages several, tn alone leaves that choice automatic). tm < 0: keep the 3x3 halo kernel where it applies and force its pixel-fragment count to tn
- * (4..7, 0 = automatic). tm == -2 on a depthwise 3x3 layer: force the matrix-core kernel's strip height to tn
+ * (4..7, 0 = automatic; set on the first layer of a chain it also applies to otter_hip_conv_chain_forward's single
+ * launch). tm == -2 on a depthwise 3x3 layer: force the matrix-core kernel's strip height to tn
  * steps of 8 / stride output rows (0 = automatic). tm == -3: use the vector-ALU depthwise kernels instead, with a
  * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. tm == -4: the generic
  * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo kernel would be picked. */

@@ -571,7 +571,9 @@ static bool chain_single_launch(const otter_hip_conv_t* const* handles, int n_la
     const otter_hip_conv_desc& d0 = handles[0]->d;
     for (int l = 0; l < n_layers; ++l) {
         const otter_hip_conv_desc& d = handles[l]->d;
-        const bool same = handles[l]->w_igemm && !handles[l]->c_pad && handles[l]->force_tm == 0 && d.in_channels == d0.in_channels &&
+        // (a forced fragment count of the LDS-halo kernel on the first layer, force_tm == -1, carries over to the chain)
+        const bool tile_ok = handles[l]->force_tm == 0 || (l == 0 && handles[l]->force_tm == -1);
+        const bool same = handles[l]->w_igemm && !handles[l]->c_pad && tile_ok && d.in_channels == d0.in_channels &&
                           d.out_channels == d0.out_channels && d.kernel_h == 3 && d.kernel_w == 3 && d.stride_h == 1 &&
                           d.stride_w == 1 && d.pad_h == 1 && d.pad_w == 1 && d.dilation_h == 1 && d.dilation_w == 1 &&
                           d.groups == 1 && d.out_round_mode == d0.out_round_mode && d.out_kind == OTTER_HIP_OUT_I8;
@@ -582,7 +584,7 @@ static bool chain_single_launch(const otter_hip_conv_t* const* handles, int n_la
     for (int l = 1; l < n_layers; ++l)
         if (pick_epilogue(make_epilogue(handles[l], OTTER_HIP_I8_P8), g.K) != pick_epilogue(ep0, g.K)) return false;
     int plan[4];
-    if (!(g.OH > 0 && g.OW > 0 && conv3x3_chain_applicable(g, ep0, n_layers, plan))) return false;
+    if (!(g.OH > 0 && g.OW > 0 && conv3x3_chain_applicable(g, ep0, n_layers, plan, handles[0]->force_tm == -1 ? handles[0]->force_tn : 0))) return false;
     // The single launch pays only where a tile's producers are far enough back in an XCD's list to be finished when
     // it is reached: 64 workgroups per XCD are in flight, and a layer's share of the list must be well above that
     // (measured: 112 tiles per XCD and layer, the 128-channel 56x56 batch-64 stack, gains 8 %; 56 or 32 tiles lose
@@ -650,7 +652,8 @@ int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_l
             eps[l] = make_epilogue(handles[l], OTTER_HIP_I8_P8);
             wpk[l] = handles[l]->w_igemm;
         }
-        const hipError_t ce = run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream);
+        const hipError_t ce = run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream,
+                                                 handles[0]->force_tm == -1 ? handles[0]->force_tn : 0);
         if (ce == hipSuccess) return OTTER_HIP_OK;
         if (ce != hipErrorNotReady) OHIP_CHECK(ce);
         // (every flag set of this GPU belongs to another stream: this stream takes the layers one by one)

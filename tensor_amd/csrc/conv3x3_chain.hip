@@ -428,7 +428,7 @@ std::mutex g_chain_mutex;
 }  // namespace
 
 // can this chain of layers (same geometry g for all) run as one launch? `plan` receives {fragments, lds rows, tiles per image, line pitch log2}
-bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers, int plan[4]) {
+bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers, int plan[4], int force_fn) {
     if (layers < 2 || layers > CHAIN_MAX_LAYERS) return false;
     if (g.C != g.K || g.ph != 1 || g.pw != 1 || g.OH != g.H || g.OW != g.W) return false;
     if (g.sh != 1 || g.sw != 1 || g.dh != 1 || g.dw != 1) return false;
@@ -438,7 +438,7 @@ bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers,
     const int epi = pick_epilogue(ep, g.K);
     if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG) return false;
     int hp[8];
-    if (!conv3x3_halo_plan(g, 0, hp)) return false;
+    if (!conv3x3_halo_plan(g, force_fn, hp)) return false;  // (a forced fragment count that does not fit: the automatic one)
     if (hp[7] != igemm_channel_groups(g.C) * 64) return false;  // the whole reduction must fit one LDS stage
     if ((long)layers * g.N * hp[2] > CHAIN_MAX_FLAGS) return false;
     plan[0] = hp[0], plan[1] = hp[6], plan[2] = hp[2], plan[3] = (g.W + 4) * 8 <= 512 ? 9 : 10;
@@ -446,9 +446,9 @@ bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers,
 }
 
 hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_t* const* wpk, const int8_t* const* act,
-                             int layers, int* error_word_out, hipStream_t stream) {
+                             int layers, int* error_word_out, hipStream_t stream, int force_fn) {
     int plan[4];
-    if (!conv3x3_chain_applicable(g, eps[0], layers, plan)) return hipErrorInvalidValue;
+    if (!conv3x3_chain_applicable(g, eps[0], layers, plan, force_fn)) return hipErrorInvalidValue;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;

@@ -24,9 +24,9 @@ hipError_t run_conv3x3_halo(const int8_t* x, const int8_t* wpk, void* out, const
                             int force_fn, hipStream_t stream);
 
 // conv3x3_chain.hip: a chain of same-shape 3x3 int8 -> int8 layers as one persistent launch
-bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers, int plan[4]);
+bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers, int plan[4], int force_fn = 0);
 hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_t* const* wpk, const int8_t* const* act,
-                             int layers, int* error_word_out, hipStream_t stream);
+                             int layers, int* error_word_out, hipStream_t stream, int force_fn = 0);
 hipError_t conv3x3_chain_error(int* error_word);
 
 // conv_direct.hip

@@ -704,7 +704,12 @@ def main():
         # the same four layers as four launches of the per-layer entry point, and one of those launches alone
         msl, _ = timer.run(wl["step_layers"], a.steps, a.warmup)
         kl, _ = timer.run(wl["layer_fn"], max(a.steps * 4, 50), 5)
+        # the chain launch ran some thousand times above: its result must still be the four launches' result, and no
+        # workgroup may have given up a wait
+        same = bool((wl["step"]().cpu() == wl["step_layers"]().cpu()).all().item())
+        gave_up = hip.conv_chain_gave_up()
         layer_by_layer = dict(ms_per_step=msl, tops=wl["ops"] / (msl * 1e-3) / 1e12, launches_per_step=4,
+                              chain_equals_layers=same, chain_gave_up=gave_up,
                               kernel="conv3x3_halo_kernel (one layer per launch)", kernel_ms=kl,
                               frac=wl["layer_ops"] / (kl * 1e-3) / 1e12 / PEAK_INT8_TOPS)
     res = measure(wl, timer, a.steps, a.warmup, unit)

@@ -97,6 +97,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
     const int EW = g.W + 4;
     const int pair_bytes = r_max * 2 * PITCH;
     const int cb = c_groups * 64;
+    const unsigned inv_ow20 = ((1u << 20) + (unsigned)g.OW - 1u) / (unsigned)g.OW;  // ceil(2^20 / OW), uniform
 
     // ---- this XCD's tile list ------------------------------------------------------------------------------------
     const int xcd = __builtin_amdgcn_readfirstlane(chain_xcc_id() % ca.xcds);
@@ -127,9 +128,16 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
         if (tl.l == 0) return true;
         int t_lo, t_hi;
         producers(tl, t_lo, t_hi);
-        bool ok = true;
-        for (int t = t_lo; t <= t_hi; ++t)
-            ok = ok && __hip_atomic_load(flag_of(tl.l - 1, tl.n, t), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ca.epoch;
+        // at most three producers (a tile's rows +-1 reach into the tile before and the tile behind): their flags are
+        // requested together, one round trip to L2 instead of up to three in a row
+        const int* f = flag_of(tl.l - 1, tl.n, 0);
+        const int t_mid = min(t_lo + 1, t_hi);
+        const int v0 = __hip_atomic_load(f + t_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int v1 = __hip_atomic_load(f + t_mid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int v2 = __hip_atomic_load(f + t_hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool ok = v0 == ca.epoch && v1 == ca.epoch && v2 == ca.epoch;
+        for (int t = t_lo + 2; t < t_hi; ++t)  // (only tiles shorter than an image row have more producers)
+            ok = ok && __hip_atomic_load(f + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ca.epoch;
         return ok;
     };
     auto deps_wait = [&](const Tile& tl) {  // thread 0 only; bounded
@@ -225,12 +233,18 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
         ep.scale_in = ca.scale_in[tl.l], ep.bias = ca.bias[tl.l], ep.scale_out = ca.scale_out[tl.l];
         ep.act_hi = ca.act_hi[tl.l], ep.act_p0 = ca.act_p0[tl.l], ep.lrelu = ca.lrelu[tl.l] != 0;
 
+        // LDS offset of each fragment's pixel (tap 0, 0). Row and column relative to the tile's first row come from a
+        // multiplication by 2^20 / OW (exact: (column of the first pixel + offset in the tile) * OW < 2^20, both factors
+        // below 2^24), not from a division per fragment: seven 32-bit divisions were a tenth of a tile's vector work.
         int bcc[FN];
+        const int col0 = p0 - r_lo * g.OW;                 // column of the tile's first pixel (uniform)
+        const int rel_max = min(p0 + PT, OHW) - 1 - p0 + col0;  // lanes past the image end keep the last pixel
 #pragma unroll
         for (int f = 0; f < FN; ++f) {
-            const int pix = min(p0 + (wn * FN + f) * 16 + (lane & 15), OHW - 1);
-            const int oy = pix / g.OW, ox = pix % g.OW;
-            bcc[f] = (oy - r_lo) * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
+            const int rel = min(col0 + (wn * FN + f) * 16 + (lane & 15), rel_max);
+            const int oy_rel = (int)(__umul24((unsigned)rel, inv_ow20) >> 20);
+            const int ox = rel - oy_rel * g.OW;
+            bcc[f] = oy_rel * 2 * PITCH + (ox - g.pw + 2) * 8 + (lane >> 4) * pair_bytes;
         }
         v4i acc[FM][FN];
 #pragma unroll

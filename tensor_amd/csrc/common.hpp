@@ -278,6 +278,13 @@ __device__ __forceinline__ void epi8_load(Epi8& p, const Epilogue& ep, int ch0) 
 // epi8_clamp_init. Without an activation (!NONNEG) there is nothing to clamp but the int8 range.
 typedef short ohip_v2s __attribute__((ext_vector_type(2)));
 
+// the clamp of one channel pair, as epi8_clamp_init packs it (for kernels that keep the clamps of a row block in LDS)
+__device__ __forceinline__ unsigned epi8_clamp_pair(const Epilogue& ep, float so0, float so1) {
+    const int q0 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, so0), ep.round_half), 127);
+    const int q1 = min((int)__fadd_rn(__fmul_rn(ep.act_hi, so1), ep.round_half), 127);
+    return (unsigned)(q0 & 0xffff) | ((unsigned)q1 << 16);
+}
+
 __device__ __forceinline__ void epi8_clamp_init(const Epilogue& ep, Epi8& p) {
 #pragma unroll
     for (int h = 0; h < 4; ++h) {

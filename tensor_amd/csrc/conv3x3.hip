@@ -66,6 +66,15 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
         const float* src = which == 0 ? ep.scale_in : (which == 1 ? ep.bias : ep.scale_out);
         lds_prm[i] = src ? src[c] : 1.f;
     }
+    // (int8 result behind ReLU / clip: the upper clamp of the rounded value per channel, once per workgroup instead of
+    // once per tile and wave)
+    __shared__ __attribute__((aligned(16))) unsigned lds_qh[ROWS / 2];
+    if constexpr (EPI == EPI_I8_P8_NONNEG) {
+        for (int i = tid; i < ROWS / 2; i += 256) {
+            const int c = blockIdx.y * ROWS + 2 * i;
+            lds_qh[i] = epi8_clamp_pair(ep, ep.scale_out[c], ep.scale_out[c + 1]);
+        }
+    }
 
     const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x), 0, (int)in_bytes, 0x00020000);
 
@@ -314,7 +323,13 @@ __global__ void __launch_bounds__(256, 2) conv3x3_halo_kernel(const int8_t* __re
                     prm.so[e] = __int_as_float(r4[e]);
                     prm.so[4 + e] = __int_as_float(r5[e]);
                 }
-                if constexpr (EPI == EPI_I8_P8_NONNEG) epi8_clamp_init(ep, prm);
+                if constexpr (EPI == EPI_I8_P8_NONNEG) {
+                    const unsigned pq = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned*)lds_qh + (unsigned)cl * 2u;
+                    v4i r6;
+                    asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(r6) : "v"(pq));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) prm.qh[e] = (unsigned)r6[e];
+                }
             }
 #pragma unroll
             for (int f = 0; f < FN; ++f) {

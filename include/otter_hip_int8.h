@@ -182,7 +182,9 @@ int otter_hip_conv_forward_residual(const otter_hip_conv_t* handle, const void* 
  * synchronizing the device) whether one ever gave up, in which case the outputs of the chain calls since the last
  * status call are not valid. The flags live in static device memory, one set per stream for the first four streams
  * that call this on a GPU (calls on different streams may overlap); further streams run their chains as n launches.
- * Like every entry point here it allocates nothing. */
+ * Like every entry point here it allocates nothing, and after one eager call on a stream it may be captured into a
+ * HIP graph on that stream and replayed (a launch takes its sequence number from device memory, not from the kernel
+ * arguments). */
 size_t otter_hip_conv_chain_workspace_bytes(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);
 int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_layers, const void* in, int n, int in_h,
                                  int in_w, void* out, void* workspace, size_t workspace_bytes, void* stream);

@@ -49,7 +49,7 @@ constexpr int CHAIN_SPIN_LIMIT = 1 << 17;  // polls of a producer flag before gi
 // different streams may overlap and must not share them.
 constexpr int CHAIN_SLOTS = 4;
 __device__ int g_chain_flags[CHAIN_SLOTS * CHAIN_MAX_FLAGS];
-__device__ int g_chain_ctl[CHAIN_SLOTS * 16];  // per slot: [0..7] queue counters, [8] workgroups that have left, [9] error
+__device__ int g_chain_ctl[CHAIN_SLOTS * 16];  // per slot: [0..7] queue counters, [8] workgroups that have left, [9] error, [10] launches completed
 
 struct ChainArgs {
     const int8_t* act[CHAIN_MAX_LAYERS + 1];  // act[l]: input of layer l; act[l + 1]: its output
@@ -59,7 +59,7 @@ struct ChainArgs {
     const float* scale_out[CHAIN_MAX_LAYERS];
     float act_hi[CHAIN_MAX_LAYERS], act_p0[CHAIN_MAX_LAYERS];
     int lrelu[CHAIN_MAX_LAYERS];
-    int layers, xcds, epoch;
+    int layers, xcds;
     int* flags;
     int* ctl;
 };
@@ -99,6 +99,10 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
     const int cb = c_groups * 64;
     const unsigned inv_ow20 = ((1u << 20) + (unsigned)g.OW - 1u) / (unsigned)g.OW;  // ceil(2^20 / OW), uniform
 
+    // The launch's epoch number = the count of completed launches on this flag set + 1, kept in device memory (ctl[10],
+    // advanced by the last workgroup to leave): a launch replayed from a captured graph gets a fresh number like any other.
+    const int epoch = __builtin_amdgcn_readfirstlane(__hip_atomic_load(ca.ctl + 10, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) + 1;
+
     // ---- this XCD's tile list ------------------------------------------------------------------------------------
     const int xcd = __builtin_amdgcn_readfirstlane(chain_xcc_id() % ca.xcds);
     const int my_images = (g.N - xcd + ca.xcds - 1) / ca.xcds;  // images xcd, xcd + xcds, ...
@@ -135,9 +139,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
         const int v0 = __hip_atomic_load(f + t_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const int v1 = __hip_atomic_load(f + t_mid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const int v2 = __hip_atomic_load(f + t_hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bool ok = v0 == ca.epoch && v1 == ca.epoch && v2 == ca.epoch;
+        bool ok = v0 == epoch && v1 == epoch && v2 == epoch;
         for (int t = t_lo + 2; t < t_hi; ++t)  // (only tiles shorter than an image row have more producers)
-            ok = ok && __hip_atomic_load(f + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ca.epoch;
+            ok = ok && __hip_atomic_load(f + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == epoch;
         return ok;
     };
     auto deps_wait = [&](const Tile& tl) {  // thread 0 only; bounded
@@ -279,7 +283,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
         // every wave's stores of the previous tile have been acknowledged: publish it
         if (tid == 0 && done_i >= 0) {
             const Tile d = tile_at(done_i);
-            __hip_atomic_store(flag_of(d.l, d.n, d.t), ca.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(flag_of(d.l, d.n, d.t), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         done_i = -1;
         // the epilogue constants of this tile's layer (nobody reads the old ones any more; the barrier behind the
@@ -386,7 +390,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
             __builtin_amdgcn_s_waitcnt(0);
             __syncthreads();
             if (tid == 0) {
-                __hip_atomic_store(flag_of(tl.l, tl.n, tl.t), ca.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(flag_of(tl.l, tl.n, tl.t), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 deps_wait(tile_at(nxt_i));
             }
             done_i = -1;
@@ -401,7 +405,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
     if (tid == 0) {
         if (done_i >= 0) {
             const Tile d = tile_at(done_i);
-            __hip_atomic_store(flag_of(d.l, d.n, d.t), ca.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(flag_of(d.l, d.n, d.t), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         // the last workgroup to leave rewinds the queues for the next launch
         const int left = __hip_atomic_fetch_add(ca.ctl + 8, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -414,6 +418,7 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
                     __hip_atomic_store(ca.ctl + 9, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             for (int i = 0; i < 9; ++i) __hip_atomic_store(ca.ctl + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(ca.ctl + 10, epoch == 0x7ffffffe ? 0 : epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
@@ -431,10 +436,9 @@ struct ChainDevice {
     int* flags = nullptr;
     int* ctl = nullptr;
     int xcds = 0;
-    // slot -> the stream that owns it (first come, for the life of the process) and that stream's launch count
+    // slot -> the stream that owns it (first come, for the life of the process)
     hipStream_t stream[CHAIN_SLOTS] = {};
     bool used[CHAIN_SLOTS] = {};
-    int epoch[CHAIN_SLOTS] = {};
 };
 ChainDevice g_chain_dev[16];
 std::mutex g_chain_mutex;
@@ -468,7 +472,7 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     ChainDevice& cd = g_chain_dev[dev];
-    int slot = -1, epoch = 0;
+    int slot = -1;
     {
         std::lock_guard<std::mutex> lock(g_chain_mutex);
         if (!cd.flags) {
@@ -485,8 +489,6 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
         for (int i = 0; i < CHAIN_SLOTS && slot < 0; ++i)
             if (!cd.used[i]) cd.used[i] = true, cd.stream[i] = stream, slot = i;
         if (slot < 0) return hipErrorNotReady;  // more streams than slots: the caller runs the layers one by one
-        epoch = ++cd.epoch[slot];
-        if (cd.epoch[slot] == 0x7fffffff) cd.epoch[slot] = 0;  // (flags of 2^31 launches ago could alias; unreachable)
     }
     ChainArgs ca;
     for (int l = 0; l < layers; ++l) {
@@ -496,7 +498,7 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
         ca.act_hi[l] = eps[l].act_hi, ca.act_p0[l] = eps[l].act_p0, ca.lrelu[l] = eps[l].lrelu ? 1 : 0;
     }
     ca.act[layers] = act[layers];
-    ca.layers = layers, ca.xcds = cd.xcds, ca.epoch = epoch;
+    ca.layers = layers, ca.xcds = cd.xcds;
     ca.flags = cd.flags + (size_t)slot * CHAIN_MAX_FLAGS, ca.ctl = cd.ctl + slot * 16;
     const int fn = plan[0], r_max = plan[1], tpi = plan[2], logp = plan[3];
     const int epi = pick_epilogue(eps[0], g.K);
@@ -561,9 +563,10 @@ hipError_t conv3x3_chain_error(int* error_word) {
         *error_word |= ctl[s * 16 + 9];
         dirty = dirty || ctl[s * 16 + 9] || ctl[s * 16 + 8] || ctl[s * 16];
     }
-    if (dirty) {  // a launch that gave up (or was cut short) leaves the counters dirty: rewind
-        int zeros[CHAIN_SLOTS * 16] = {0};
-        if ((e = hipMemcpy(g_chain_dev[dev].ctl, zeros, sizeof(zeros), hipMemcpyHostToDevice)) != hipSuccess) return e;
+    if (dirty) {  // a launch that gave up (or was cut short) leaves the counters dirty: rewind them, keep the launch counts
+        for (int s = 0; s < CHAIN_SLOTS; ++s)
+            for (int i = 0; i < 10; ++i) ctl[s * 16 + i] = 0;
+        if ((e = hipMemcpy(g_chain_dev[dev].ctl, ctl, sizeof(ctl), hipMemcpyHostToDevice)) != hipSuccess) return e;
     }
     return hipSuccess;
 }

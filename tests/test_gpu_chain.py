@@ -151,6 +151,41 @@ def test_default_rule_takes_the_single_launch_for_large_problems_only(hip):
     assert hip.conv_chain_launches(convs, 16, 28, 28) == 1
 
 
+def test_chain_replayed_from_a_captured_graph(hip):
+    """The single launch captured into a graph and replayed: every replay must take a fresh epoch number (it lives in
+    device memory, not in the kernel arguments), so replays on new inputs, with eager work and synchronisations in
+    between, all equal the layers one by one."""
+    torch = hip.torch
+    rng = np.random.default_rng(40)
+    N, C, H, W, L = 16, 128, 28, 28, 3
+    convs, _ = _layers(hip, rng, [C] * (L + 1), act=1)
+    xs = [hip.to_device(capi.pack_np(rng.integers(-127, 128, size=(N, C, H, W), dtype=np.int8), 8)) for _ in range(3)]
+    wants = [_one_by_one(hip, convs, x, N, H, W).clone() for x in xs]
+    x_static = xs[0].clone()
+    out = hip.empty(N * C * H * W, np.int8)
+    ws = hip.empty(2 * N * C * H * W + 1024, np.int8)
+    assert hip.conv_chain_launches(convs, N, H, W) == 1
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        hip.conv_chain(convs, x_static, N, H, W, out=out, workspace=ws)  # (first call on this stream: takes its flag set)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        hip.conv_chain(convs, x_static, N, H, W, out=out, workspace=ws)
+    for rep in range(2):
+        for x, want in zip(xs, wants):
+            x_static.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert bool((out == want.view(-1)).all().item())
+            # eager work on the same flag set between replays
+            with torch.cuda.stream(side):
+                eager = hip.conv_chain(convs, x, N, H, W)
+            side.synchronize()
+            assert bool((eager == want.view(-1)).all().item())
+    assert not hip.conv_chain_gave_up()
+
+
 def test_chain_argument_checks(hip):
     rng = np.random.default_rng(6)
     convs, _ = _layers(hip, rng, [16, 32])

@@ -201,7 +201,7 @@ int otter_hip_conv_chain_set_min_tiles(int tiles);
 
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
- * blob). For tests and profiling. */
+ * blob), 5 streamed 1x1 kernel (int8 -> int8 over at most 64 input channels). For tests and profiling. */
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, int n, int in_h, int in_w,
                                int out_layout);
 
@@ -213,7 +213,9 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
  * launch). tm == -2 on a depthwise 3x3 layer: force the matrix-core kernel's strip height to tn
  * steps of 8 / stride output rows (0 = automatic). tm == -3: use the vector-ALU depthwise kernels instead, with a
  * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. tm == -4: the generic
- * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo kernel would be picked. */
+ * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo or the streamed 1x1 kernel would be picked.
+ * tm == -5 on a layer the streamed 1x1 kernel takes: tn = groups | slices << 3 forces the 16-pixel groups a wave owns
+ * (2 or 4) and the slices the output channels are cut into (0 = automatic for either). */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
 /* Test hook with no counterpart in the reference, host arithmetic only (no GPU needed): the launch plan of the 3x3

@@ -100,6 +100,7 @@ struct otter_hip_conv {
     float* scale_in = nullptr;   // [Kpad]
     float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
     float* scale_out = nullptr;  // [Kpad] or null
+    unsigned* clamp_hi = nullptr; // [Kpad / 2] upper clamps of the rounded int8 results (ReLU / clip, dense layers) or null
     float* in_scale = nullptr;   // [1]
     int c_pad = 0;               // > 0: C is not a multiple of 8; the MFMA path runs on C zero-padded to c_pad
     int force_tm = 0, force_tn = 0;
@@ -191,6 +192,7 @@ int otter_hip_conv_destroy(otter_hip_conv_t* h) {
     (void)hipFree(h->scale_in);
     (void)hipFree(h->bias);
     (void)hipFree(h->scale_out);
+    (void)hipFree(h->clamp_hi);
     (void)hipFree(h->in_scale);
     delete h;
     return OTTER_HIP_OK;
@@ -234,6 +236,14 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
                 if (!(so[i] > 0.f) || std::isinf(so[i])) h->so_positive = false;
             }
             if ((rc = upload<float>(&h->scale_out, so.data(), K, kpad, 1.f))) break;
+            if (g == 1 && h->so_positive && (d.activation_type == 1 || d.activation_type == 3)) {
+                // the streamed 1x1 kernel reads the clamps of its ReLU / clip epilogue instead of deriving them per wave
+                so.resize(kpad, 1.f);
+                std::vector<unsigned> qh(kpad / 2);
+                conv_pw_stream_clamps(d.activation_type == 3 ? 6.f : __builtin_inff(),
+                                      d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f, so.data(), kpad, qh.data());
+                if ((rc = upload<unsigned>(&h->clamp_hi, qh.data(), qh.size(), qh.size(), 0u))) break;
+            }
         }
         if ((rc = upload<float>(&h->in_scale, &in_scale, 1, 1, 0.f))) break;
         if (h->depthwise && C % 8) {
@@ -359,13 +369,15 @@ static bool use_stem(const otter_hip_conv* h, int in_layout, const ConvGeom& g_i
     return h->w_stem && h->force_tm == 0 && conv_stem_applicable(g_in, ep, in_layout);
 }
 
-// 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS, 4 few-channel 3x3 (image stem)
+// 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS, 4 few-channel 3x3 (image stem),
+// 5 streamed 1x1 over few input channels
 static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g, const Epilogue& ep) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
         if (h->w_igemm && g.groups > 1) return igemm_grouped_applicable(g, ep) ? 1 : 0;  // else the scalar catch-all
         if (h->w_igemm) {
             if (h->force_tm > 0 || h->force_tm == -4) return 1;  // forced generic kernel (-4: with automatic tiles)
+            if (conv_pw_stream_applicable(g, ep)) return 5;
             if (g.OH > 0 && g.OW > 0 && conv3x3_halo_supported(g, ep)) return 3;
             return 1;
         }
@@ -500,6 +512,11 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
         }
         break;
     }
+    case 5:
+        // set_tile(-5, groups | slices << 3): force the pixel groups per wave and the slices of the output channels
+        OHIP_CHECK(run_conv_pw_stream(xq, h->w_igemm, h->clamp_hi, out, g, ep, h->force_tm == -5 ? (h->force_tn & 7) : 0,
+                                      h->force_tm == -5 ? (h->force_tn >> 3) : 0, stream));
+        break;
     case 1:
         OHIP_CHECK(run_conv_igemm(xq, h->w_igemm, out, g, ep, h->force_tm > 0 ? h->force_tm : 0,
                                   h->force_tm > 0 ? h->force_tn : 0, stream));

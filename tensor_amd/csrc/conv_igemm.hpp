@@ -17,6 +17,13 @@ void igemm_pack_weights_grouped(const int8_t* w, int K, int C, int groups, int k
 hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep, int tm,
                           int tn, hipStream_t stream);
 
+// conv_pw.hip: 1x1 stride-1 int8 -> int8 over at most 64 input channels, streamed (reads the implicit-GEMM weight packing)
+bool conv_pw_stream_applicable(const ConvGeom& g, const Epilogue& ep);
+void conv_pw_stream_plan(const ConvGeom& g, int* groups, int* slices);
+void conv_pw_stream_clamps(float act_hi, float round_half, const float* scale_out, int n, unsigned* dst);
+hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned* qh, void* out, const ConvGeom& g,
+                              const Epilogue& ep, int force_groups, int force_slices, hipStream_t stream);
+
 // conv3x3.hip
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep);
 bool conv3x3_halo_plan(const ConvGeom& g, int force_fn, int plan[8]);

@@ -1,0 +1,198 @@
+// Pointwise (1x1, stride 1) int8 -> int8 convolution over at most 64 input channels, as a streaming kernel.
+//
+// With one MFMA reduction step per output the layer is an elementwise pass: read C bytes per pixel, write K bytes,
+// and the time goes into the requantization of the K results, not into the product. The implicit-GEMM kernel pays
+// for its generality here (output rows padded to its row tile, the pixels' round trip through LDS and two barriers
+// per workgroup for one MFMA step, a workgroup prologue per tile). This kernel has no tile grid and one barrier:
+//   - a wave owns G groups of 16 consecutive pixels of one image and loads their bytes straight into the MFMA's
+//     B operand (lane (q, p): channels 16q..16q+15 of pixel p = two 8-byte elements of the Byte8 blob);
+//   - it walks the output channels in pairs of 16-row tiles (32 channels); the A operands (the implicit-GEMM weight
+//     packing as it lies in memory, 16 bytes per lane and tile) and the per-channel constants of the workgroup's
+//     pairs sit in LDS, copied there once per workgroup, and are read once per pair for all G groups;
+//   - after the two MFMAs of a pair each lane holds 8 consecutive output channels of one pixel (the row
+//     permutation of igemm_row_channel), requantizes them and stores one Byte8 element: 16 lanes cover 128
+//     contiguous bytes.
+// Only whole channel octets are stored, so K need not be a multiple of 32; the padded rows cost their MFMA only.
+#include "common.hpp"
+#include "conv_igemm.hpp"
+
+#include <algorithm>
+
+namespace ohip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v2u_store __attribute__((__vector_size__(2 * sizeof(unsigned))));
+
+constexpr unsigned PW_OOB = 0x80000000u;  // past any buffer: the load returns zero, the store is dropped
+
+// LDS image of one pair of row tiles: the two A operands in lane order, then scale_in, bias, scale_out (32 floats
+// each) and the clamps (16 dwords) of the pair's 32 channels
+constexpr int PW_PAIR_V4 = 128 + 8 + 8 + 8 + 4;  // 16-byte units
+constexpr int PW_MAX_PAIRS = 24;
+
+// grid: x = chunks of 4 waves x G groups x 16 pixels of an image, y = image, z = slice of the channel pairs
+// qh (EPI_I8_P8_NONNEG): the upper clamps of the rounded results, one 16-bit value per padded channel
+// (conv_pw_stream_clamps)
+// The four waves of a workgroup share one copy of their slice's weights and constants in LDS: read from there a
+// lane group's constants are one broadcast each, where 64 lanes loading them from memory keep the texture
+// addresser busy for longer than the requantization of two pixel groups takes.
+template <int EPI, int G>
+__global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
+                                                             int8_t* __restrict__ out, Epilogue ep,
+                                                             const unsigned* __restrict__ qh, int C8, int K, int HW,
+                                                             int pairs_per_slice) {
+    extern __shared__ v4i pw_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane >> 4, p = lane & 15;
+    const int n = blockIdx.y;
+    const int pix0 = (blockIdx.x * 4 + wave) * (16 * G);
+
+    const size_t in_img = (size_t)C8 * HW * 8, out_img = (size_t)K * HW;
+    const __amdgpu_buffer_rsrc_t rin =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x) + (size_t)n * in_img, 0, (int)in_img, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(out + (size_t)n * out_img, 0, (int)out_img, 0x00020000);
+
+    // B operands of the G groups (all out of range for a wave past the image: zeros, and nothing is stored)
+    v4i b[G];
+    const bool plane0 = 2 * q < C8, plane1 = 2 * q + 1 < C8;
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+        const int pix = pix0 + 16 * gi + p;
+        const unsigned o0 = ((unsigned)(2 * q) * HW + pix) * 8u;
+        const bool in = pix < HW;
+        const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && plane0 ? o0 : PW_OOB), 0, 0));
+        const v2i hi = __builtin_bit_cast(
+            v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && plane1 ? o0 + (unsigned)HW * 8u : PW_OOB), 0, 0));
+        b[gi] = v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+
+    const int pairs = (K + 31) / 32;
+    const int pr0 = blockIdx.z * pairs_per_slice;
+    const int pr1 = min(pr0 + pairs_per_slice, pairs);
+    {
+        // the per-channel arrays are padded to the weight rows, so every pair is whole in memory
+        const v4i* wg = reinterpret_cast<const v4i*>(wpk);
+        const v4i* sg = reinterpret_cast<const v4i*>(ep.scale_in);
+        const v4i* bg = reinterpret_cast<const v4i*>(ep.bias);
+        const v4i* og = reinterpret_cast<const v4i*>(ep.scale_out);
+        const v4i* cg = reinterpret_cast<const v4i*>(qh);
+        const int total = (pr1 - pr0) * PW_PAIR_V4;
+        for (int i = threadIdx.x; i < total; i += 256) {
+            const int pr = pr0 + i / PW_PAIR_V4, r = i % PW_PAIR_V4;
+            v4i v;
+            if (r < 128) v = wg[pr * 128 + r];
+            else if (r < 136) v = sg[pr * 8 + r - 128];
+            else if (r < 144) v = bg[pr * 8 + r - 136];
+            else if (r < 152) v = og[pr * 8 + r - 144];
+            else if constexpr (EPI == EPI_I8_P8_NONNEG) v = cg[pr * 4 + r - 152];
+            else v = v4i{0, 0, 0, 0};
+            pw_lds[i] = v;
+        }
+    }
+    __syncthreads();
+    if (pix0 >= HW) return;
+
+    for (int pr = pr0; pr < pr1; ++pr) {
+        const v4i* l = pw_lds + (pr - pr0) * PW_PAIR_V4;
+        const v4i a0 = l[lane], a1 = l[64 + lane];
+        Epi8 prm;
+        {
+            const v4i s0 = l[128 + 2 * q], s1 = l[129 + 2 * q], b0 = l[136 + 2 * q], b1 = l[137 + 2 * q];
+            const v4i o0 = l[144 + 2 * q], o1 = l[145 + 2 * q], c = l[152 + q];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
+                prm.bi[e] = __int_as_float(b0[e]), prm.bi[4 + e] = __int_as_float(b1[e]);
+                prm.so[e] = __int_as_float(o0[e]), prm.so[4 + e] = __int_as_float(o1[e]);
+                prm.qh[e] = (unsigned)c[e];
+            }
+        }
+        const int ch0 = 32 * pr + 8 * q;
+        const bool live = ch0 < K;
+        const unsigned orow = (unsigned)(ch0 >> 3) * HW;
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) {
+            const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b[gi], v4i{0, 0, 0, 0}, 0, 0, 0);
+            const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b[gi], v4i{0, 0, 0, 0}, 0, 0, 0);
+            const int a8[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+            const v2i r = epi8_quant_i8p8<EPI == EPI_I8_P8_NONNEG>(ep, prm, a8);
+            const int pix = pix0 + 16 * gi + p;
+            const unsigned oo = (orow + pix) * 8u;
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, r), rout, (int)(live && pix < HW ? oo : PW_OOB),
+                                                  0, 0);
+        }
+    }
+}
+
+// The upper clamp of the rounded result per channel for the ReLU / clip epilogue, as epi8_clamp_pair packs it: two
+// 16-bit values per dword. Host arithmetic in the order the kernels use (one multiplication, one addition, toward zero).
+void conv_pw_stream_clamps(float act_hi, float round_half, const float* scale_out, int n, unsigned* dst) {
+    auto one = [&](float so) {
+        float t = act_hi * so;
+        t = t + round_half;
+        return t >= 127.f ? 127u : (unsigned)(int)t;
+    };
+    for (int i = 0; i + 1 < n; i += 2) dst[i / 2] = one(scale_out[i]) | one(scale_out[i + 1]) << 16;
+}
+
+bool conv_pw_stream_applicable(const ConvGeom& g, const Epilogue& ep) {
+    if (g.groups != 1 || g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph != 0 || g.pw != 0) return false;
+    if (g.Cs || g.Ks || g.C % 8 || g.C > 64 || g.K % 8 || g.N < 1 || g.N > 65535) return false;
+    if ((size_t)std::max(g.C, g.K) * g.H * g.W >= (1ull << 31)) return false;  // 32-bit offsets inside an image
+    const int epi = pick_epilogue(ep, g.K);
+    return epi == EPI_I8_P8 || epi == EPI_I8_P8_NONNEG;
+}
+
+// Pixel groups per wave and slices of the channel pairs. Four groups per wave amortize a pair's operand reads best
+// and are taken while they still leave every SIMD a few waves; below that two groups, and the channel pairs cut
+// into slices (each slice re-reads the pixels, which are few bytes next to what it writes) until there are about
+// two waves per SIMD or a slice is down to two pairs.
+void conv_pw_stream_plan(const ConvGeom& g, int* groups, int* slices) {
+    const int HW = g.H * g.W, pairs = (g.K + 31) / 32;
+    auto waves = [&](int G, int s) { return (long)g.N * ((HW + 16 * G - 1) / (16 * G)) * s; };
+    const int G = waves(4, 1) >= 8192 ? 4 : 2;
+    int s = 1;
+    const int smax = std::max(1, pairs / 2);
+    while (s < smax && waves(G, s) < 8192) ++s;
+    while ((pairs + s - 1) / s > PW_MAX_PAIRS) ++s;  // a slice's LDS image stays under 64 KB
+    const int per = (pairs + s - 1) / s;
+    *groups = G, *slices = (pairs + per - 1) / per;
+}
+
+template <int EPI, int G>
+static hipError_t launch_pw(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                            const unsigned* qh, int slices, hipStream_t stream) {
+    const int HW = g.H * g.W, pairs = (g.K + 31) / 32;
+    const int per = (pairs + slices - 1) / slices;
+    const dim3 grid((HW + 64 * G - 1) / (64 * G), g.N, (pairs + per - 1) / per);
+    hipLaunchKernelGGL((conv_pw_stream_kernel<EPI, G>), grid, dim3(256), (size_t)per * PW_PAIR_V4 * 16, stream, x, wpk,
+                       (int8_t*)out, ep, qh, g.C / 8, g.K, HW, per);
+    return hipGetLastError();
+}
+
+// qh: conv_pw_stream_clamps of the layer's output scales (read by the ReLU / clip epilogue only)
+// force_groups / force_slices: 0 = automatic
+hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned* qh, void* out, const ConvGeom& g,
+                              const Epilogue& ep, int force_groups, int force_slices, hipStream_t stream) {
+    if (!conv_pw_stream_applicable(g, ep)) return hipErrorInvalidValue;
+    int G, s;
+    conv_pw_stream_plan(g, &G, &s);
+    if (force_groups) G = force_groups;
+    if (force_slices) s = force_slices;
+    const int pairs = (g.K + 31) / 32;
+    if ((G != 2 && G != 4) || s < 1 || s > pairs) return hipErrorInvalidValue;
+    while ((pairs + s - 1) / s > PW_MAX_PAIRS) ++s;  // a slice's LDS image stays under 64 KB
+    const bool nonneg = pick_epilogue(ep, g.K) == EPI_I8_P8_NONNEG;
+    if (nonneg && !qh) return hipErrorInvalidValue;
+#define OHIP_PW(G_) \
+    if (G == G_) \
+        return nonneg ? launch_pw<EPI_I8_P8_NONNEG, G_>(x, wpk, out, g, ep, qh, s, stream) \
+                      : launch_pw<EPI_I8_P8, G_>(x, wpk, out, g, ep, qh, s, stream);
+    OHIP_PW(4)
+    OHIP_PW(2)
+#undef OHIP_PW
+    return hipErrorInvalidValue;
+}
+
+}  // namespace ohip

@@ -214,7 +214,8 @@ def build_bench(hip, capi, rng, batch=64, hw=224, calib=32):
                 shape=(batch, 3, hw, hw), _keep=(net, sess))
 
 
-KERNEL_NAMES = {0: "direct", 1: "implicit GEMM (MFMA)", 2: "depthwise", 3: "3x3 LDS-halo (MFMA)", 4: "few-channel 3x3"}
+KERNEL_NAMES = {0: "direct", 1: "implicit GEMM (MFMA)", 2: "depthwise", 3: "3x3 LDS-halo (MFMA)", 4: "few-channel 3x3",
+                5: "streamed 1x1 (MFMA)"}
 
 
 def per_layer(hip, capi, rng, time_fn, batch=64, hw=224, calib=32):

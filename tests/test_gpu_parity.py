@@ -346,6 +346,36 @@ def test_random_shapes_against_oracle(hip, oracle, C, K, k, s, p, d, g, N, H, W)
             assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("groups_slices", [(0, 0), (4, 1), (2, 2), (2, 3), (2, 1), (4, 5)],
+                         ids=["auto", "g4s1", "g2s2", "g2s3", "g2s1", "g4s5"])
+def test_streamed_pointwise_kernel(hip, oracle, groups_slices):
+    """The streamed 1x1 int8 -> int8 kernel (at most 64 input channels): 1 to 8 input octets (a half-used operand
+    register, a full one), output channel counts that end inside a pair of row tiles (8, 24, 40, 144) and on one,
+    pixel counts that are not whole groups of 16 (and images smaller than one group), every epilogue the fast int8
+    path has (none, ReLU, clip, LeakyReLU), with and without bias, forced pixel groups per wave and channel slices.
+    fp32 output and more than 64 input channels stay on the implicit-GEMM kernel."""
+    G, S = groups_slices
+    rng = np.random.default_rng(100 + 8 * G + S)
+    for (C, K, N, H, W) in [(16, 96, 2, 19, 23), (24, 144, 1, 28, 28), (32, 16, 3, 9, 11), (8, 8, 2, 3, 3),
+                            (64, 384, 1, 14, 14), (40, 24, 2, 16, 16), (56, 40, 1, 5, 41), (32, 192, 2, 1, 70)]:
+        pairs = (K + 31) // 32
+        tile = (-5, G | min(S, pairs) << 3) if G else None
+        x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W)
+        in_scale = 25.0
+        for act, b in [(0, bias), (1, bias), (3, None), (2, bias)]:
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, bias=b, top_scale=11.0, int8_out=True, act_type=act,
+                                             act_params=[0.1] if act == 2 else [0.0, 6.0])
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, bias=b, top_scale=11.0, act=act, act_p0=0.1,
+                                 out_kind=capi.OUT_I8, tile=tile)
+            assert kind == 5, (C, K, act)
+            np.testing.assert_array_equal(out, want)
+        out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, bias=bias, act=1, out_kind=capi.OUT_F32)
+        assert kind == 1
+    x, wq, ws, bias = _rand_problem(rng, 72, 32, 1, 1, 1, 6, 6)
+    _, kind = run_conv(hip, oracle, x, wq, ws, 25.0, bias=bias, top_scale=11.0, act=1, out_kind=capi.OUT_I8)
+    assert kind == 1
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_drawn_geometries_against_oracle(hip, oracle, seed):
     """Eight geometries per seed drawn from the whole domain of the layer (kernel 1..5, stride 1..2, dilation 1..2,
@@ -434,7 +464,8 @@ def test_depthwise5x5_and_wide_padding(hip, oracle, family, s):
 
 @pytest.mark.parametrize("C,K,k,s,p,g,N,H,W,kind", [
     (64, 96, 3, 1, 1, 1, 2, 14, 16, 3),     # 3x3 LDS-halo kernel
-    (48, 72, 1, 1, 0, 1, 2, 13, 11, 1),     # 1x1 implicit GEMM
+    (80, 72, 1, 1, 0, 1, 2, 13, 11, 1),     # 1x1 implicit GEMM
+    (48, 72, 1, 1, 0, 1, 2, 13, 11, 5),     # 1x1 streamed (int8 result; the fp32 one takes the implicit GEMM)
     (32, 64, 3, 2, 1, 1, 2, 15, 15, 1),     # 3x3 stride 2 implicit GEMM
     (40, 40, 3, 1, 1, 40, 3, 12, 20, 2),    # depthwise stride 1
     (24, 24, 3, 2, 1, 24, 3, 13, 18, 2),    # depthwise stride 2
@@ -449,7 +480,7 @@ def test_leaky_relu_fast_epilogues(hip, oracle, C, K, k, s, p, g, N, H, W, kind)
                                          int8_out=int8_out, act_type=2, act_params=[0.1])
         out, got_kind = run_conv(hip, oracle, x, wq, ws, 18.0, stride=s, pad=p, groups=g, bias=bias, top_scale=13.0,
                                  act=2, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
-        assert got_kind == kind
+        assert got_kind == (1 if kind == 5 and not int8_out else kind)
         if int8_out:
             np.testing.assert_array_equal(out, want)
         else:

@@ -199,6 +199,29 @@ int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_
  * argument only queries. */
 int otter_hip_conv_chain_set_min_tiles(int tiles);
 
+/* An inverted-residual block as networks spell it -- a 1x1 Convolution (int8 result), a depthwise 3x3 Convolution
+ * (int8 result) and a 1x1 Convolution, each read only by the next (Tensor/Net.cpp:413-505 runs them one after the other,
+ * ConvolutionLayer::forward_int8, Tensor/ConvolutionLayer.cpp:754-847, three times), optionally followed by the Eltwise
+ * sum with the block's shortcut (Tensor/EltwiseLayer.cpp:48-80). `in` is the Byte8 input of the first layer; out is the
+ * last layer's result: fp32 in OTTER_HIP_F32_P4 (then `residual`, or NULL, is a blob of that layout added to it, and
+ * out_q, or NULL, receives the Byte8 quantization float2int8(out * q_scale) with q_round_mode, as in
+ * otter_hip_conv_forward_residual / _twin) or int8 Byte8 (residual and out_q NULL). The result is what the three (four)
+ * calls give, bit for bit. Where the depthwise layer is stride 1 pad 1 on an image at most 64 pixels wide, the first
+ * layer reads at most 192 channels and the activations are none / ReLU / clip, the block runs as ONE launch that keeps
+ * the expanded tensor in LDS (otter_hip_conv_block_launches says 1) and needs no workspace; otherwise as three launches
+ * with the two intermediate blobs in `workspace` (otter_hip_conv_block_workspace_bytes). */
+int otter_hip_conv_block_launches(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
+                                  const otter_hip_conv_t* project, int n, int in_h, int in_w);
+size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
+                                            const otter_hip_conv_t* project, int n, int in_h, int in_w);
+int otter_hip_conv_block_forward(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
+                                 const otter_hip_conv_t* project, const void* in, int n, int in_h, int in_w,
+                                 const float* residual, void* out, int out_layout, void* out_q, float q_scale,
+                                 int q_round_mode, void* workspace, size_t workspace_bytes, void* stream);
+/* Tuning / test hook with no counterpart in the reference: force the single launch's output rows per band and the
+ * expanded channels per LDS slice (64 or 128) of blocks whose first layer is `expand`; 0 = automatic. */
+int otter_hip_conv_block_set_plan(otter_hip_conv_t* expand, int rows_per_band, int slice_channels);
+
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
  * blob), 5 streamed 1x1 kernel (int8 -> int8 over at most 64 input channels). For tests and profiling. */

@@ -73,7 +73,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
-           "otter_hip_conv_chain_set_min_tiles"]
+           "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
+           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan"]
 
 
 def load_cdll():
@@ -95,6 +96,7 @@ class Library:
         L.otter_hip_last_error.restype = C.c_char_p
         L.otter_hip_conv_workspace_bytes.restype = C.c_size_t
         L.otter_hip_conv_chain_workspace_bytes.restype = C.c_size_t
+        L.otter_hip_conv_block_workspace_bytes.restype = C.c_size_t
         self.device = torch.device("cuda", device)
         self._check(L.otter_hip_init(C.c_int(device)))
 
@@ -251,6 +253,28 @@ class Library:
                                                           C.c_size_t(ws_bytes), self.stream()))
         return out
 
+    def conv_block(self, expand, dw, project, x, n, h, w, residual=None, q_scale=None, q_round_mode=ROUND_SSE):
+        """otter_hip_conv_block_forward: x (int8 Byte8) through expand -> depthwise -> project (+ residual), and with
+        q_scale the Byte8 quantization of the result. Returns (out, q or None)."""
+        oh, ow = dw.out_hw(*expand.out_hw(h, w))
+        oh, ow = project.out_hw(oh, ow)
+        f32 = project.out_kind == OUT_F32
+        out_layout = F32_P4 if f32 else I8_P8
+        out = self.empty(n * project.K * oh * ow, np.float32 if f32 else np.int8)
+        q = self.empty(n * project.K * oh * ow, np.int8) if q_scale is not None else None
+        ws_bytes = self.lib.otter_hip_conv_block_workspace_bytes(expand.h, dw.h, project.h, n, h, w)
+        workspace = self.empty(ws_bytes, np.int8) if ws_bytes else None
+        self._check(self.lib.otter_hip_conv_block_forward(
+            expand.h, dw.h, project.h, self.ptr(x), n, h, w, self.ptr(residual) if residual is not None else None,
+            self.ptr(out), out_layout, self.ptr(q) if q is not None else None, C.c_float(q_scale or 0.0), q_round_mode,
+            self.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.stream()))
+        return out, q
+
+    def conv_block_launches(self, expand, dw, project, n, h, w):
+        r = self.lib.otter_hip_conv_block_launches(expand.h, dw.h, project.h, n, h, w)
+        self._check(min(r, 0))
+        return r
+
     def conv_chain_launches(self, convs, n, h, w):
         hs = (C.c_void_p * len(convs))(*[c.h for c in convs])
         r = self.lib.otter_hip_conv_chain_launches(hs, len(convs), n, h, w)
@@ -305,6 +329,9 @@ class Conv:
 
     def set_tile(self, tm, tn):
         self.L._check(self.L.lib.otter_hip_conv_set_tile(self.h, tm, tn))
+
+    def set_block_plan(self, rows_per_band, slice_channels):
+        self.L._check(self.L.lib.otter_hip_conv_block_set_plan(self.h, rows_per_band, slice_channels))
 
     def forward(self, x, in_layout, n, h, w, out_layout=None, out=None, workspace=None):
         out_layout = self.default_out_layout() if out_layout is None else out_layout

@@ -104,6 +104,7 @@ struct otter_hip_conv {
     float* in_scale = nullptr;   // [1]
     int c_pad = 0;               // > 0: C is not a multiple of 8; the MFMA path runs on C zero-padded to c_pad
     int force_tm = 0, force_tn = 0;
+    int block_rb = 0, block_sl = 0;  // forced plan of the fused block launch this layer heads (0 = automatic)
 };
 
 extern "C" {
@@ -716,6 +717,124 @@ int otter_hip_conv_forward_twin(const otter_hip_conv_t* h, const void* in, int i
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_twin: unknown rounding mode");
     return conv_forward(h, in, in_layout, n, in_h, in_w, out, out_layout, workspace, workspace_bytes, stream, (int8_t*)out_q,
                         q_scale, q_round_mode);
+}
+
+// ---- an inverted-residual block ----------------------------------------------------------------------------------
+
+static int block_check(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p, int n, int in_h,
+                       int in_w, const char* who) {
+    if (!e || !d || !p) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": null layer");
+    if (e->d.out_kind != OTTER_HIP_OUT_I8 || d->d.out_kind != OTTER_HIP_OUT_I8 || p->d.out_kind == OTTER_HIP_OUT_I32)
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": the first two layers must write int8, the last int8 or fp32");
+    if (e->d.in_channels % 8 || e->d.out_channels % 8 || d->d.out_channels % 8)
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": the blobs inside the block must be Byte8 (channels in octets)");
+    if (e->d.out_channels != d->d.in_channels || d->d.out_channels != p->d.in_channels)
+        return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": channel counts of consecutive layers do not match");
+    if (n < 0 || in_h < 1 || in_w < 1) return fail(OTTER_HIP_ERR_INVALID, std::string(who) + ": bad shape");
+    return OTTER_HIP_OK;
+}
+
+// geometry of the three layers on this input; false on an empty blob
+static bool block_geoms(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p, int n, int in_h,
+                        int in_w, ConvGeom g[3]) {
+    g[0] = make_geom(e->d, n, in_h, in_w);
+    if (g[0].OH < 1 || g[0].OW < 1) return false;
+    g[1] = make_geom(d->d, n, g[0].OH, g[0].OW);
+    if (g[1].OH < 1 || g[1].OW < 1) return false;
+    g[2] = make_geom(p->d, n, g[1].OH, g[1].OW);
+    return g[2].OH >= 1 && g[2].OW >= 1;
+}
+
+static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
+                                const ConvGeom g[3], int out_layout) {
+    if (!e->w_igemm || e->c_pad || e->force_tm || !d->depthwise || !d->w_dw_mfma || d->c_pad || d->force_tm || !p->w_igemm ||
+        p->c_pad || p->force_tm)
+        return false;
+    const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8), e3 = make_epilogue(p, out_layout);
+    if (!conv_block_applicable(g[0], e1, g[1], e2, g[2], e3)) return false;
+    int plan[4];
+    return conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, plan);
+}
+
+static int block_default_out_layout(const otter_hip_conv_t* p) {
+    return p->d.out_kind == OTTER_HIP_OUT_F32 ? OTTER_HIP_F32_P4 : OTTER_HIP_I8_P8;
+}
+
+int otter_hip_conv_block_launches(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p, int n,
+                                  int in_h, int in_w) {
+    int rc = block_check(e, d, p, n, in_h, in_w, "otter_hip_conv_block_launches");
+    if (rc) return rc;
+    ConvGeom g[3];
+    if (!block_geoms(e, d, p, n, in_h, in_w, g)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_launches: empty output");
+    return n >= 1 && p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p)) ? 1 : 3;
+}
+
+size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
+                                            int n, int in_h, int in_w) {
+    if (!e || !d || !p || n < 1 || in_h < 1 || in_w < 1) return 0;
+    ConvGeom g[3];
+    if (!block_geoms(e, d, p, n, in_h, in_w, g)) return 0;
+    if (p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p))) return 0;
+    const size_t b0 = (size_t)n * g[0].K * g[0].OH * g[0].OW, b1 = (size_t)n * g[1].K * g[1].OH * g[1].OW;
+    return (b0 + 255) / 256 * 256 + (b1 + 255) / 256 * 256;
+}
+
+int otter_hip_conv_block_set_plan(otter_hip_conv_t* e, int rows_per_band, int slice_channels) {
+    if (!e || rows_per_band < 0 || (slice_channels != 0 && slice_channels != 64 && slice_channels != 128))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_set_plan: bad argument");
+    e->block_rb = rows_per_band, e->block_sl = slice_channels;
+    return OTTER_HIP_OK;
+}
+
+int otter_hip_conv_block_forward(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
+                                 const void* in, int n, int in_h, int in_w, const float* residual, void* out, int out_layout,
+                                 void* out_q, float q_scale, int q_round_mode, void* workspace, size_t workspace_bytes,
+                                 void* stream_) {
+    if (!in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: null");
+    int rc = block_check(e, d, p, n, in_h, in_w, "otter_hip_conv_block_forward");
+    if (rc) return rc;
+    const bool f32 = p->d.out_kind == OTTER_HIP_OUT_F32;
+    if (!valid_layout(out_layout) || layout_elem(out_layout) != (f32 ? 0 : 1) || p->d.out_channels % layout_pack(out_layout))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: output layout does not match the last layer");
+    if ((residual || out_q) && !f32)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: a shortcut sum or a quantized twin needs an fp32 result");
+    if (out_q && p->d.out_channels % 8)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: the quantized result needs K % 8 == 0");
+    if (out_q && q_round_mode != OTTER_HIP_ROUND_SSE && q_round_mode != OTTER_HIP_ROUND_EXACT)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: unknown rounding mode");
+    if (residual == out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: out must not be the residual");
+    ConvGeom g[3];
+    if (!block_geoms(e, d, p, n, in_h, in_w, g)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: empty output");
+    for (int l = 0; l < 3; ++l)
+        if ((size_t)n * g[l].C * g[l].H * g[l].W >= (1ull << 31) || (size_t)n * g[l].K * g[l].OH * g[l].OW >= (1ull << 31))
+            return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_block_forward: tensor exceeds 2^31 elements; split the batch");
+    if (n == 0) return OTTER_HIP_OK;
+    hipStream_t stream = (hipStream_t)stream_;
+
+    if (p->d.out_channels % 8 == 0 && out_layout == block_default_out_layout(p) && block_single_launch(e, d, p, g, out_layout)) {
+        const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8);
+        Epilogue e3 = make_epilogue(p, out_layout);
+        e3.residual = residual;
+        e3.twin = (int8_t*)out_q, e3.twin_scale = q_scale;
+        e3.twin_half = q_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+        OHIP_CHECK(run_conv_block((const int8_t*)in, e->w_igemm, d->w_dw_mfma, p->w_igemm, out, g[0], e1, g[1], e2, g[2], e3,
+                                  e->block_rb, e->block_sl, stream));
+        return OTTER_HIP_OK;
+    }
+    // the layers one after the other, the intermediate blobs in the workspace
+    const size_t b0 = (size_t)n * g[0].K * g[0].OH * g[0].OW, b1 = (size_t)n * g[1].K * g[1].OH * g[1].OW;
+    const size_t need = (b0 + 255) / 256 * 256 + (b1 + 255) / 256 * 256;
+    if (!workspace || workspace_bytes < need)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: needs the workspace reported by "
+                                           "otter_hip_conv_block_workspace_bytes");
+    void* t0 = workspace;
+    void* t1 = (char*)workspace + (b0 + 255) / 256 * 256;
+    rc = conv_forward(e, in, OTTER_HIP_I8_P8, n, in_h, in_w, t0, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
+    if (rc) return rc;
+    rc = conv_forward(d, t0, OTTER_HIP_I8_P8, n, g[1].H, g[1].W, t1, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
+    if (rc) return rc;
+    return conv_forward(p, t1, OTTER_HIP_I8_P8, n, g[2].H, g[2].W, out, out_layout, nullptr, 0, stream_, (int8_t*)out_q, q_scale,
+                        q_round_mode, residual);
 }
 
 // -----------------------------------------------------------------------------------------------------

@@ -24,6 +24,15 @@ void conv_pw_stream_clamps(float act_hi, float round_half, const float* scale_ou
 hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned* qh, void* out, const ConvGeom& g,
                               const Epilogue& ep, int force_groups, int force_slices, hipStream_t stream);
 
+// conv_block.hip: 1x1 expand -> depthwise 3x3 -> 1x1 project (+ shortcut sum, + int8 twin) as one launch
+bool conv_block_applicable(const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
+                           const Epilogue& e3);
+struct BlockArgs;
+bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int force_sl, int plan[4], BlockArgs* out = nullptr);
+hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int8_t* w_dw, const int8_t* w_prj, void* out,
+                          const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
+                          const Epilogue& e3, int force_rb, int force_sl, hipStream_t stream);
+
 // conv3x3.hip
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep);
 bool conv3x3_halo_plan(const ConvGeom& g, int force_fn, int plan[8]);

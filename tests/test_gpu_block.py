@@ -1,0 +1,131 @@
+"""otter_hip_conv_block_forward: an inverted-residual block (1x1 expand -> depthwise 3x3 -> 1x1 project, optionally
++ shortcut and the quantized twin of the result) as one launch that keeps the expanded tensor in LDS. The result must
+be, bit for bit, what the three layers give one by one through otter_hip_conv_forward (+ _residual / _twin), and what
+the oracle gives for the three layers (int8 blobs bit-exact, the fp32 result within FP32_RTOL, in fact bitwise)."""
+import numpy as np
+import pytest
+
+from tensor_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+FP32_RTOL = 1e-5
+
+
+def quantize_weights(wf):
+    K = wf.shape[0]
+    ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
+    wq = np.clip(np.round(wf * ws[:, None, None, None]), -127, 127).astype(np.int8)
+    return wq, ws
+
+
+def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1):
+    """The three layers as a MobileNetV2 block has them: expand and depthwise with `act` and int8 results, a linear
+    project layer with an fp32 or int8 result."""
+    layers = []
+    in_scale = np.float32(rng.uniform(20, 60))
+    specs = [(cin, ce, 1, 1, 0, 1, act, True), (ce, ce, 3, stride, 1, ce, act, True), (ce, cout, 1, 1, 0, 1, 0, not f32_out)]
+    for (ci, co, k, s, pad, groups, a, i8) in specs:
+        wq, ws = quantize_weights(rng.normal(0, 0.3 if groups > 1 else 2.0 / np.sqrt(ci), (co, ci // groups, k, k)).astype(np.float32))
+        bias = rng.normal(0, 0.05, co).astype(np.float32)
+        out_scale = np.float32(rng.uniform(15, 40))
+        si = (np.float32(1.0) / (in_scale * ws)).astype(np.float32)
+        conv = hip.conv(wq=wq, scale_in=si, bias=bias, in_scale=float(in_scale), out_scale=[out_scale] if i8 else None,
+                        stride=(s, s), pad=(pad, pad), groups=groups, act=a,
+                        out_kind=capi.OUT_I8 if i8 else capi.OUT_F32, out_round=capi.ROUND_SSE)
+        layers.append(dict(conv=conv, wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale), k=k,
+                           stride=s, pad=pad, groups=groups, act=a, int8_out=i8))
+        in_scale = out_scale
+    return layers
+
+
+def one_by_one(hip, layers, xd, n, h, w, residual, q_scale):
+    e, d, p = (l["conv"] for l in layers)
+    t = e.forward(xd, capi.I8_P8, n, h, w, capi.I8_P8)
+    t = d.forward(t, capi.I8_P8, n, h, w, capi.I8_P8)
+    oh, ow = d.out_hw(h, w)
+    if residual is not None:
+        return p.forward_residual(t, capi.I8_P8, n, oh, ow, residual, q_scale=q_scale)
+    if q_scale is not None:
+        return p.forward_twin(t, capi.I8_P8, n, oh, ow, q_scale, capi.ROUND_SSE)
+    return p.forward(t, capi.I8_P8, n, oh, ow), None
+
+
+CASES = [
+    # cin, ce, cout, N, H, W, act, f32_out, residual, twin, plan
+    (64, 384, 64, 5, 14, 14, 3, True, True, True, None),      # a 14x14 MobileNetV2 block, automatic plan
+    (64, 384, 64, 3, 14, 14, 3, True, True, True, (4, 128)),  # four bands, 128-channel slices
+    (64, 384, 64, 3, 14, 14, 3, True, True, True, (8, 64)),   # two bands of unequal height
+    (160, 960, 160, 3, 7, 7, 3, True, True, True, None),      # 7x7: one band, three reduction steps in the expand layer
+    (160, 960, 320, 2, 7, 7, 3, False, False, False, None),   # int8 result, ten channel pairs in the project layer
+    (32, 192, 32, 3, 28, 28, 3, True, True, True, None),      # 28x28
+    (24, 144, 24, 2, 56, 56, 3, True, True, True, None),      # 56x56, 24 channels (padded reduction), 144 = 2.25 slices
+    (96, 576, 96, 3, 14, 14, 1, True, True, False, None),     # ReLU, 4.5 slices of 128, no twin
+    (64, 384, 96, 3, 14, 14, 3, True, False, True, None),     # no shortcut (channel count changes), twin only
+    (40, 136, 24, 2, 11, 13, 0, True, False, False, None),    # no activation (signed blobs), odd sizes, nothing fused behind
+    (16, 96, 24, 2, 9, 64, 3, True, False, False, None),      # the widest image the launch takes
+    (8, 48, 8, 1, 1, 1, 3, True, True, True, None),           # a single pixel
+]
+
+
+@pytest.mark.parametrize("cin,ce,cout,N,H,W,act,f32_out,with_res,with_twin,plan", CASES)
+def test_block_equals_the_three_layers(hip, oracle, cin, ce, cout, N, H, W, act, f32_out, with_res, with_twin, plan):
+    rng = np.random.default_rng(cin * 1000 + ce + H)
+    layers = make_block(hip, rng, cin, ce, cout, act, f32_out)
+    e, d, p = (l["conv"] for l in layers)
+    if plan is not None:
+        e.set_block_plan(*plan)
+    assert hip.conv_block_launches(e, d, p, N, H, W) == 1
+    x = rng.integers(-127, 128, (N, cin, H, W)).astype(np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    res = resd = None
+    if with_res:
+        res = rng.normal(0, 1, (N, cout, H, W)).astype(np.float32)
+        resd = hip.to_device(capi.pack_np(res, 4))
+    q_scale = 21.5 if with_twin else None
+    for _ in range(2):  # twice: nothing may depend on what the previous call left in LDS or memory
+        got, got_q = hip.conv_block(e, d, p, xd, N, H, W, residual=resd, q_scale=q_scale)
+        hip.torch.cuda.synchronize()
+        want, want_q = one_by_one(hip, layers, xd, N, H, W, resd, q_scale)
+        hip.torch.cuda.synchronize()
+        assert hip.torch.equal(got, want)
+        if with_twin:
+            assert hip.torch.equal(got_q, want_q)
+    # against the oracle, layer by layer
+    cur = x
+    for l in layers:
+        cur = oracle.conv_layer_forward(cur, l["wq"], l["ws"], l["in_scale"], stride=(l["stride"],) * 2, pad=(l["pad"],) * 2,
+                                        groups=l["groups"], bias=l["bias"], top_scale=l["out_scale"], int8_out=l["int8_out"],
+                                        act_type=l["act"])
+    if with_res:
+        cur = oracle.eltwise_add(cur, res)
+    out = capi.unpack_np(got.cpu().numpy(), 4 if f32_out else 8, (N, cout, H, W))
+    if f32_out:
+        np.testing.assert_allclose(out, cur, rtol=FP32_RTOL, atol=0)
+        assert (out.view(np.int32) == cur.view(np.int32)).all()
+        if with_twin:
+            q = oracle.quantize(cur, np.float32(q_scale), capi.ROUND_SSE)
+            assert (capi.unpack_np(got_q.cpu().numpy(), 8, (N, cout, H, W)) == q).all()
+    else:
+        assert (out == cur).all()
+    for l in layers:
+        l["conv"].close()
+
+
+def test_block_falls_back_to_three_launches(hip):
+    """A stride-2 depthwise layer is not what the single launch takes: the same call runs the layers one by one."""
+    rng = np.random.default_rng(5)
+    layers = make_block(hip, rng, 32, 192, 64, 3, True, stride=2)
+    e, d, p = (l["conv"] for l in layers)
+    N, H, W = 2, 28, 28
+    assert hip.conv_block_launches(e, d, p, N, H, W) == 3
+    x = rng.integers(-127, 128, (N, 32, H, W)).astype(np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    got, got_q = hip.conv_block(e, d, p, xd, N, H, W, q_scale=30.0)
+    t = e.forward(xd, capi.I8_P8, N, H, W, capi.I8_P8)
+    t = d.forward(t, capi.I8_P8, N, H, W, capi.I8_P8)
+    want, want_q = p.forward_twin(t, capi.I8_P8, N, 14, 14, 30.0, capi.ROUND_SSE)
+    hip.torch.cuda.synchronize()
+    assert hip.torch.equal(got, want) and hip.torch.equal(got_q, want_q)
+    for l in layers:
+        l["conv"].close()

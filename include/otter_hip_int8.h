@@ -207,9 +207,12 @@ int otter_hip_conv_chain_set_min_tiles(int tiles);
  * out_q, or NULL, receives the Byte8 quantization float2int8(out * q_scale) with q_round_mode, as in
  * otter_hip_conv_forward_residual / _twin) or int8 Byte8 (residual and out_q NULL). The result is what the three (four)
  * calls give, bit for bit. Where the depthwise layer is stride 1 pad 1 on an image at most 64 pixels wide, the first
- * layer reads at most 192 channels and the activations are none / ReLU / clip, the block runs as ONE launch that keeps
- * the expanded tensor in LDS (otter_hip_conv_block_launches says 1) and needs no workspace; otherwise as three launches
- * with the two intermediate blobs in `workspace` (otter_hip_conv_block_workspace_bytes). */
+ * layer reads at most 192 channels and the activations are none / ReLU / clip, the block can run as ONE launch that
+ * keeps the expanded tensor in LDS and needs no workspace; it does (otter_hip_conv_block_launches says 1) for the
+ * shapes where that was measured faster than the three launches (at most 64 input channels, images up to 28 pixels
+ * wide, 128..512 bands of rows over the batch), or for every shape that qualifies after
+ * otter_hip_conv_block_set_always(1) / a forced plan. Otherwise the call makes three launches with the two intermediate
+ * blobs in `workspace` (otter_hip_conv_block_workspace_bytes). */
 int otter_hip_conv_block_launches(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
                                   const otter_hip_conv_t* project, int n, int in_h, int in_w);
 size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
@@ -218,6 +221,10 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* expand, const otter_hip
                                  const otter_hip_conv_t* project, const void* in, int n, int in_h, int in_w,
                                  const float* residual, void* out, int out_layout, void* out_q, float q_scale,
                                  int q_round_mode, void* workspace, size_t workspace_bytes, void* stream);
+/* Tuning / test hook with no counterpart in the reference: 1 = every block that qualifies by shape runs as the single
+ * launch, 0 = only the shapes measured faster that way (default). Process-wide; returns the previous value; a negative
+ * argument only queries. */
+int otter_hip_conv_block_set_always(int on);
 /* Tuning / test hook with no counterpart in the reference: force the single launch's output rows per band and the
  * expanded channels per LDS slice (64 or 128) of blocks whose first layer is `expand`; 0 = automatic. */
 int otter_hip_conv_block_set_plan(otter_hip_conv_t* expand, int rows_per_band, int slice_channels);

@@ -74,7 +74,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
-           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan"]
+           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always"]
 
 
 def load_cdll():
@@ -269,6 +269,10 @@ class Library:
             self.ptr(out), out_layout, self.ptr(q) if q is not None else None, C.c_float(q_scale or 0.0), q_round_mode,
             self.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.stream()))
         return out, q
+
+    def conv_block_set_always(self, on):
+        """otter_hip_conv_block_set_always: returns the previous setting."""
+        return self.lib.otter_hip_conv_block_set_always(int(on))
 
     def conv_block_launches(self, expand, dw, project, n, h, w):
         r = self.lib.otter_hip_conv_block_launches(expand.h, dw.h, project.h, n, h, w)

@@ -96,6 +96,7 @@ struct otter_hip_conv {
     int8_t* w_stem = nullptr;    // MFMA lane order of the few-channel 3x3 kernel (C <= 5, K <= 64)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
     int8_t* w_dw_mfma = nullptr; // block-diagonal MFMA operands (depthwise 3x3, C % 8 == 0)
+    int32_t* blk_consts = nullptr; // the layer's constants (and depthwise 3x3 weights) as the fused block launch keeps them in LDS
     bool so_positive = true;     // every output scale is finite and > 0
     float* scale_in = nullptr;   // [Kpad]
     float* bias = nullptr;       // [Kpad]; -0.0f everywhere when the layer has no bias
@@ -190,6 +191,7 @@ int otter_hip_conv_destroy(otter_hip_conv_t* h) {
     (void)hipFree(h->w_stem);
     (void)hipFree(h->w_dw);
     (void)hipFree(h->w_dw_mfma);
+    (void)hipFree(h->blk_consts);
     (void)hipFree(h->scale_in);
     (void)hipFree(h->bias);
     (void)hipFree(h->scale_out);
@@ -246,6 +248,23 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
                 if ((rc = upload<unsigned>(&h->clamp_hi, qh.data(), qh.size(), qh.size(), 0u))) break;
             }
         }
+        if (d.out_kind == OTTER_HIP_OUT_I8 && K % 8 == 0 && C % 8 == 0 &&
+            (g == 1 || (h->depthwise && d.kernel_h == 3 && d.kernel_w == 3))) {
+            // what the fused block launch (conv_block.hip) copies into LDS: the per-channel arrays as uploaded above
+            // (padded the same way), the upper clamps of a ReLU / clip epilogue, a depthwise layer's weights
+            const int kp = (K + 31) / 32 * 32;
+            std::vector<float> si(kp, 0.f), bi(kp, -0.0f), so(kp, 1.f);
+            std::memcpy(si.data(), scale_in, (size_t)K * sizeof(float));
+            if (bias) std::memcpy(bi.data(), bias, (size_t)K * sizeof(float));
+            for (int i = 0; i < K; ++i) so[i] = n_out_scale == 1 ? out_scale[0] : out_scale[i];
+            const bool nonneg = h->so_positive && (d.activation_type == 1 || d.activation_type == 3);
+            const float hi = d.activation_type == 3 ? 6.f : __builtin_inff();
+            const float half = d.out_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+            std::vector<int32_t> kc((g == 1 ? block_expand_const_bytes(K) : block_dw_const_bytes(K)) / sizeof(int32_t));
+            if (g == 1) block_pack_expand_consts(si.data(), bi.data(), so.data(), K, nonneg, hi, half, kc.data());
+            else block_pack_dw_consts(weight, si.data(), bi.data(), so.data(), K, nonneg, hi, half, kc.data());
+            if ((rc = upload<int32_t>(&h->blk_consts, kc.data(), kc.size(), kc.size(), 0))) break;
+        }
         if ((rc = upload<float>(&h->in_scale, &in_scale, 1, 1, 0.f))) break;
         if (h->depthwise && C % 8) {
             // depthwise on a channel count that is not whole octets: the channels are zero-padded to the next octet on the
@@ -267,6 +286,7 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
                 dw_mfma_pack_weights(weight, C, d.stride_w, d.pad_w, d.kernel_w, wa.data());
                 if ((rc = upload<int8_t>(&h->w_dw_mfma, wa.data(), wa.size(), wa.size(), 0))) break;
             }
+
         } else if (g == 1 && C % 8 == 0) {
             std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
             igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
@@ -745,15 +765,25 @@ static bool block_geoms(const otter_hip_conv_t* e, const otter_hip_conv_t* d, co
     return g[2].OH >= 1 && g[2].OW >= 1;
 }
 
+static int g_block_always = 0;  // see block_single_launch
+
 static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
                                 const ConvGeom g[3], int out_layout) {
-    if (!e->w_igemm || e->c_pad || e->force_tm || !d->depthwise || !d->w_dw_mfma || d->c_pad || d->force_tm || !p->w_igemm ||
+    if (!e->w_igemm || e->c_pad || e->force_tm || !e->blk_consts || !d->depthwise || !d->blk_consts || d->c_pad || d->force_tm || !p->w_igemm ||
         p->c_pad || p->force_tm)
         return false;
     const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8), e3 = make_epilogue(p, out_layout);
     if (!conv_block_applicable(g[0], e1, g[1], e2, g[2], e3)) return false;
     int plan[4];
-    return conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, plan);
+    if (!conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, plan)) return false;
+    if (g_block_always || e->block_rb || e->block_sl) return true;
+    // The single launch pays where the three layers are short, latency-bound launches and its workgroups (a band of
+    // rows of one image each) about fill the 256 compute units once. Measured at batch 64 against the three launches:
+    // 14x14 64 -> 384 -> 64 13.2 us against 17.8 us, 28x28 32 -> 192 -> 32 16.8 against 21.8; 56x56 (896 workgroups
+    // of 13 us each) 56 against 45, 7x7 (64 workgroups, the requantization of a whole image on one compute unit's
+    // vector ALUs) 38 against 20, more than 64 input channels (reduction steps in registers, spills) 24 against 23.5.
+    const long wgs = (long)g[0].N * plan[1];
+    return g[0].C <= 64 && g[0].W <= 28 && wgs >= 128 && wgs <= 512;
 }
 
 static int block_default_out_layout(const otter_hip_conv_t* p) {
@@ -777,6 +807,12 @@ size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const ott
     if (p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p))) return 0;
     const size_t b0 = (size_t)n * g[0].K * g[0].OH * g[0].OW, b1 = (size_t)n * g[1].K * g[1].OH * g[1].OW;
     return (b0 + 255) / 256 * 256 + (b1 + 255) / 256 * 256;
+}
+
+int otter_hip_conv_block_set_always(int on) {
+    const int before = g_block_always;
+    if (on >= 0) g_block_always = on ? 1 : 0;
+    return before;
 }
 
 int otter_hip_conv_block_set_plan(otter_hip_conv_t* e, int rows_per_band, int slice_channels) {
@@ -817,7 +853,7 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* e, const otter_hip_conv
         e3.residual = residual;
         e3.twin = (int8_t*)out_q, e3.twin_scale = q_scale;
         e3.twin_half = q_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
-        OHIP_CHECK(run_conv_block((const int8_t*)in, e->w_igemm, d->w_dw_mfma, p->w_igemm, out, g[0], e1, g[1], e2, g[2], e3,
+        OHIP_CHECK(run_conv_block((const int8_t*)in, e->w_igemm, e->blk_consts, d->blk_consts, p->w_igemm, out, g[0], e1, g[1], e2, g[2], e3,
                                   e->block_rb, e->block_sl, stream));
         return OTTER_HIP_OK;
     }

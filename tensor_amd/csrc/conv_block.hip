@@ -16,6 +16,8 @@
 // Two barriers per slice (A|B, B|C); C of one slice and A of the next run without one.
 // Every intermediate value is the one the three layers would have written: same accumulators, same epilogue code.
 #include <algorithm>
+#include <cstring>
+#include <vector>
 
 #include "common.hpp"
 #include "conv_igemm.hpp"
@@ -25,12 +27,16 @@ namespace ohip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
-constexpr int BLK_WAVES = 8;
-constexpr int BLK_NI = 5;    // (channel pair, pixel group) items of the project layer per wave, at most
+constexpr int BLK_WAVES = 16;
+constexpr int BLK_NI = 3;    // (channel pair, pixel group) items of the project layer per wave, at most
 constexpr int BLK_CGE = 3;   // 64-channel reduction steps of the expand layer, at most (192 input channels)
+constexpr int BLK_PAIR_DW = 112;  // LDS dwords of one expand channel pair's constants: scale_in, bias, scale_out (32 each), 16 clamps
+constexpr int BLK_OCT_DW = 52;    // LDS dwords of one depthwise octet: 3 x 8 weight words, scale_in, bias, scale_out (8 each), 4 clamps
 
 struct BlockArgs {
-    const int8_t *x, *w_exp, *w_dw, *w_prj;
+    const int8_t *x, *w_exp, *w_prj;
+    const int32_t* k1;  // expand layer: [channel pair][BLK_PAIR_DW] constants (block_pack_expand_consts)
+    const int32_t* k2;  // depthwise layer: [octet][BLK_OCT_DW] weights and constants (block_pack_dw_consts)
     void* out;
     Epilogue e1, e2, e3;
     int Cin8, cgE, mtE;   // input octets; reduction steps and (padded) 16-row tiles of the expand weights
@@ -38,38 +44,70 @@ struct BlockArgs {
     int cgP, mtP, Cout;   // project: reduction steps, (padded) 16-row tiles, output channels
     int H, W, HW;
     int RB, bands;        // output rows per band, bands per image
-    int SL, slices;       // expanded channels per slice, slices
+    int slices;           // slices of SL expanded channels
     int cpr, rpi;         // depthwise: lane columns (of 4 pixels) per row, rows per wave item
     int ER, pitch;        // LDS lines per octet (RB + 2), bytes per line
     int GA, GD;           // 16-pixel groups: the band's input rows, the band's output rows
     int npairsP, itemsP;  // project: channel pairs (32 channels), pairs x GD
     unsigned inv_w;       // ceil(2^20 / W)
-    int lds_e, lds_d;     // byte offsets of the two intermediate arrays (the input operands start at 0)
+    int lds_e, lds_d, lds_c1, lds_c2;  // byte offsets: expanded lines, depthwise results, constants of the two layers
+    int lds_c3, lds_r;                 // constants of the project layer, the band's shortcut elements (fp32 result only)
 };
 
+// LDS visibility between the phases needs the LDS counter only: the weight loads requested ahead stay in flight
+__device__ __forceinline__ void blk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // EPI3: EPI_F32_P4_FUSED (fp32 Float4, optional residual and twin in e3) or EPI_I8_P8 (signed int8 Byte8)
-template <bool NONNEG, int EPI3>
+// SL: expanded channels per slice; NI: project items per wave; CGE: reduction steps of the expand layer (at least cgE)
+template <bool NONNEG, int EPI3, int SL, int NI, int CGE>
 __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockArgs a) {
     extern __shared__ v4i blk_lds[];
     char* const lds = reinterpret_cast<char*>(blk_lds);
     char* const ldsE = lds + a.lds_e;
     char* const ldsD = lds + a.lds_d;
+    const int* const ldsC1 = reinterpret_cast<const int*>(lds + a.lds_c1);
+    const int* const ldsC2 = reinterpret_cast<const int*>(lds + a.lds_c2);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 15, q = lane >> 4;
     const int band = blockIdx.x, n = blockIdx.y;
-    const int r0 = band * a.RB, rows = min(a.RB, a.H - r0);
+    // bands of nearly equal height (at most RB rows): band b owns rows [b * H / bands, (b + 1) * H / bands)
+    const int r0 = band * a.H / a.bands, rows = (band + 1) * a.H / a.bands - r0;
     const int in_row0 = max(r0 - 1, 0), in_row1 = min(r0 + rows, a.H - 1);
     const int in_pix0 = in_row0 * a.W, in_pixN = (in_row1 + 1) * a.W - in_pix0;
     const int out_pixN = rows * a.W;
 
-    // ---- prologue: zero the expanded lines (their borders are never written), stage the input as MFMA B operands ----
+    constexpr int npairsE = SL / 32, noct = SL / 8, kqs = SL / 16, KSS = SL / 64;
+    static_assert(BLK_WAVES % noct == 0, "a wave keeps one octet of the slice");
+    // A: pair of the slice and first pixel group of this wave
+    const int prE = wave % npairsE, gaE0 = wave / npairsE;
+    constexpr int gaEs = BLK_WAVES / npairsE;
+
+    // the expand weights of a slice: this wave's channel pair, every reduction step
+    v4i wA[CGE][2];
+    // (every load is issued whatever the shape -- indices past the end are clamped to the last valid one -- so that the
+    // wait in front of a weight's first use counts the loads requested after it instead of waiting for all of them)
+    auto load_wA = [&](int s) {
+        const int pair_abs = min(s * npairsE + prE, (a.Ce - 1) / 32);
+        const v4i* wg = reinterpret_cast<const v4i*>(a.w_exp) + (size_t)(2 * pair_abs) * 64 + lane;
+#pragma unroll
+        for (int cg = 0; cg < CGE; ++cg) {
+            const size_t o = (size_t)min(cg, a.cgE - 1) * a.mtE * 64;
+            wA[cg][0] = wg[o];
+            wA[cg][1] = wg[o + 64];
+        }
+    };
+    load_wA(0);
+
+    // ---- prologue: zero the expanded lines (their borders are never written), stage the input as MFMA B operands,
+    // the per-channel constants of the expand and depthwise layers and the depthwise weights ---------------------------
     {
-        const int e16 = (a.SL / 8) * a.ER * a.pitch / 16;
+        const int e16 = noct * a.ER * a.pitch / 16;
         v4i* e = reinterpret_cast<v4i*>(ldsE);
         for (int i = tid; i < e16; i += 64 * BLK_WAVES) e[i] = v4i{0, 0, 0, 0};
         const int total = a.GA * a.cgE * 64;
         const int8_t* xi = a.x + (size_t)n * a.Cin8 * a.HW * 8;
+#pragma unroll 2
         for (int i = tid; i < total; i += 64 * BLK_WAVES) {
             const int l = i & 63, t = i >> 6;
             const int ga = t / a.cgE, cg = t - ga * a.cgE;
@@ -82,43 +120,109 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
             }
             blk_lds[i] = v4i{lo[0], lo[1], hi[0], hi[1]};
         }
+        // the two layers' constants and the depthwise weights, as the host laid them out (straight copies)
+        v4i* c1 = reinterpret_cast<v4i*>(lds + a.lds_c1);
+        const v4i* g1 = reinterpret_cast<const v4i*>(a.k1);
+        const int n1 = ((a.Ce + 31) / 32) * (BLK_PAIR_DW / 4);
+#pragma unroll 2
+        for (int i = tid; i < n1; i += 64 * BLK_WAVES) c1[i] = g1[i];
+        v4i* c2 = reinterpret_cast<v4i*>(lds + a.lds_c2);
+        const v4i* g2 = reinterpret_cast<const v4i*>(a.k2);
+        const int n2 = a.Ce8 * (BLK_OCT_DW / 4);
+#pragma unroll 4
+        for (int i = tid; i < n2; i += 64 * BLK_WAVES) c2[i] = g2[i];
+        if constexpr (EPI3 != EPI_I8_P8) {
+            // project: [channel pair][scale_in 32][bias 32] (the arrays are padded to whole pairs), and the band's elements
+            // of the shortcut blob as [channel quad][pixel of the band]
+            int* c3 = reinterpret_cast<int*>(lds + a.lds_c3);
+            const int n3 = a.npairsP * 64;
+            for (int i = tid; i < n3; i += 64 * BLK_WAVES) {
+                const int pr = i >> 6, r = i & 63;
+                c3[i] = __float_as_int(r < 32 ? a.e3.scale_in[32 * pr + r] : a.e3.bias[32 * pr + r - 32]);
+            }
+            if (a.e3.residual != nullptr) {  // uniform
+                v4i* rl = reinterpret_cast<v4i*>(lds + a.lds_r);
+                const v4i* rg = reinterpret_cast<const v4i*>(a.e3.residual) + (size_t)n * (a.Cout / 4) * a.HW + r0 * a.W;
+                const int n4 = (a.Cout / 4) * out_pixN;
+#pragma unroll 2
+                for (int i = tid; i < n4; i += 64 * BLK_WAVES) {
+                    const int c4 = i / out_pixN, px = i - c4 * out_pixN;
+                    rl[i] = rg[(size_t)c4 * a.HW + px];
+                }
+            }
+        }
     }
 
-    // ---- lane constants of the three phases ------------------------------------------------------------------------
-    const int npairsE = a.SL / 32, noct = a.SL / 8, kqs = a.SL / 16;
-    // A: pair of the slice and first pixel group of this wave
-    const int prE = wave % npairsE, gaE0 = wave / npairsE, gaEs = BLK_WAVES / npairsE;
-    // B: lane column -> (row within the item, column chunk)
+    // B: lane column -> (row within the item, column chunk); selectors that move a row's tap into the lane's byte of
+    // the block-diagonal weight operand (dw_mfma_pack_weights: lane (r, g) holds, for pixel slot e, the tap
+    // dx = 2g + e - 1 - r/4 of channel 4t + r%4 at byte 8e + 4t + r%4, zero when dx is outside the window)
     const int row_sub = p / a.cpr, nx = p - row_sub * a.cpr;
     const bool laneB = row_sub < a.rpi;
     const int oxB = 4 * nx + q;
-    // C: accumulators
-    v4i acc[BLK_NI][2];
+    unsigned selB[2];
 #pragma unroll
-    for (int i = 0; i < BLK_NI; ++i) acc[i][0] = acc[i][1] = v4i{0, 0, 0, 0};
-
-    __syncthreads();
+    for (int e = 0; e < 2; ++e) {
+        const int dx = 2 * q + e - 1 - (p >> 2);
+        const unsigned none = 0x0c0c0c0cu;
+        selB[e] = (dx >= 0 && dx <= 2) ? (none & ~(0xffu << (8 * (p & 3)))) | ((unsigned)dx << (8 * (p & 3))) : none;
+    }
+    // the depthwise weight operands: only two of an operand's four dwords ever hold a tap, the others stay zero for the
+    // whole kernel; and a zero tuple that every fresh accumulation starts from (kept in registers: the compiler would
+    // otherwise write four zeros in front of every first matrix instruction)
+    v4i wB[3][2];
+#pragma unroll
+    for (int dy = 0; dy < 3; ++dy) wB[dy][0] = wB[dy][1] = v4i{0, 0, 0, 0};
+    v4i zero4 = {0, 0, 0, 0};
+    asm volatile("" : "+v"(zero4));
+    // C: accumulators and the weights requested a phase ahead
+    v4i acc[NI][2];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) acc[i][0] = acc[i][1] = v4i{0, 0, 0, 0};
+    constexpr bool PFP = NI == 1;  // the project weights are requested a phase ahead where the registers allow
+    v4i wP[NI][KSS][2];
+    auto load_wP = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int prP = min(wave + BLK_WAVES * i, a.itemsP - 1) % a.npairsP;
+#pragma unroll
+            for (int ks = 0; ks < KSS; ++ks) {
+                const int cgp = min(s * KSS + ks, a.cgP - 1);
+                const v4i* wg = reinterpret_cast<const v4i*>(a.w_prj) + ((size_t)cgp * a.mtP + 2 * prP) * 64 + lane;
+                wP[i][ks][0] = wg[0], wP[i][ks][1] = wg[64];
+            }
+        }
+    };
+    blk_barrier();
 
     for (int s = 0; s < a.slices; ++s) {
         // ================= A: expand =================
+        if constexpr (PFP) load_wP(s);
         {
             const int pair_abs = s * npairsE + prE;
             if (32 * pair_abs < a.Ce) {  // wave-uniform
-                v4i wA[BLK_CGE][2];
-                const v4i* wg = reinterpret_cast<const v4i*>(a.w_exp) + (size_t)(2 * pair_abs) * 64 + lane;
-#pragma unroll
-                for (int cg = 0; cg < BLK_CGE; ++cg)
-                    if (cg < a.cgE) {
-                        wA[cg][0] = wg[(size_t)cg * a.mtE * 64];
-                        wA[cg][1] = wg[(size_t)cg * a.mtE * 64 + 64];
-                    }
                 Epi8 prm;
-                epi8_load<NONNEG ? EPI_I8_P8_NONNEG : EPI_I8_P8>(prm, a.e1, 32 * pair_abs + 8 * q);
+                {
+                    const v4i* c = reinterpret_cast<const v4i*>(ldsC1 + pair_abs * BLK_PAIR_DW);
+                    const v4i s0 = c[2 * q], s1 = c[2 * q + 1], b0 = c[8 + 2 * q], b1 = c[9 + 2 * q];
+                    const v4i o0 = c[16 + 2 * q], o1 = c[17 + 2 * q], ch = c[24 + q];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
+                        prm.bi[e] = __int_as_float(b0[e]), prm.bi[4 + e] = __int_as_float(b1[e]);
+                        prm.so[e] = __int_as_float(o0[e]), prm.so[4 + e] = __int_as_float(o1[e]);
+                        prm.qh[e] = (unsigned)ch[e];
+                    }
+                }
                 char* const eo = ldsE + (size_t)((4 * prE + q) * a.ER) * a.pitch;
                 for (int ga = gaE0; ga < a.GA; ga += gaEs) {
-                    v4i c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+                    v4i c0, c1;
+                    {
+                        const v4i b = blk_lds[(ga * a.cgE) * 64 + lane];
+                        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wA[0][0], b, zero4, 0, 0, 0);
+                        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wA[0][1], b, zero4, 0, 0, 0);
+                    }
 #pragma unroll
-                    for (int cg = 0; cg < BLK_CGE; ++cg)
+                    for (int cg = 1; cg < CGE; ++cg)
                         if (cg < a.cgE) {
                             const v4i b = blk_lds[(ga * a.cgE + cg) * 64 + lane];
                             c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wA[cg][0], b, c0, 0, 0, 0);
@@ -137,32 +241,44 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
                 }
             }
         }
-        __syncthreads();
+        blk_barrier();
         // ================= B: depthwise =================
+        if (s + 1 < a.slices) load_wA(s + 1);
         {
             const int nrc = (rows + a.rpi - 1) / a.rpi;
-            for (int ol = wave; ol < noct; ol += BLK_WAVES) {
-                const int oct_abs = s * noct + ol;
-                if (oct_abs >= a.Ce8) break;  // wave-uniform
-                v4i wB[3][2];
-                const v4i* wg = reinterpret_cast<const v4i*>(a.w_dw) + (size_t)oct_abs * 6 * 64 + lane;
+            const int ol = wave % noct;
+            const int oct_abs = s * noct + ol;
+            if (oct_abs < a.Ce8) {  // wave-uniform
+                const int* const c = ldsC2 + oct_abs * BLK_OCT_DW;
 #pragma unroll
-                for (int dy = 0; dy < 3; ++dy)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) wB[dy][t] = wg[(dy * 2 + t) * 64];
+                for (int dy = 0; dy < 3; ++dy) {
+                    const unsigned w0 = (unsigned)c[dy * 8 + (p & 3)], w1 = (unsigned)c[dy * 8 + 4 + (p & 3)];
+                    wB[dy][0][0] = (int)__builtin_amdgcn_perm(0u, w0, selB[0]), wB[dy][0][2] = (int)__builtin_amdgcn_perm(0u, w0, selB[1]);
+                    wB[dy][1][1] = (int)__builtin_amdgcn_perm(0u, w1, selB[0]), wB[dy][1][3] = (int)__builtin_amdgcn_perm(0u, w1, selB[1]);
+                }
                 Epi8 prm;
-                epi8_load<NONNEG ? EPI_I8_P8_NONNEG : EPI_I8_P8>(prm, a.e2, 8 * oct_abs);
+                {
+                    const v4i* cv = reinterpret_cast<const v4i*>(c + 24);
+                    const v4i s0 = cv[0], s1 = cv[1], b0 = cv[2], b1 = cv[3], o0 = cv[4], o1 = cv[5], ch = cv[6];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
+                        prm.bi[e] = __int_as_float(b0[e]), prm.bi[4 + e] = __int_as_float(b1[e]);
+                        prm.so[e] = __int_as_float(o0[e]), prm.so[4 + e] = __int_as_float(o1[e]);
+                        prm.qh[e] = (unsigned)ch[e];
+                    }
+                }
                 const char* const ei = ldsE + (size_t)(ol * a.ER) * a.pitch + (4 * nx + 2 * q) * 8;
                 char* const dout = ldsD + (size_t)(ol >> 1) * 256 + (ol & 1) * 8;
-                for (int rc = 0; rc < nrc; ++rc) {
+                for (int rc = wave / noct; rc < nrc; rc += BLK_WAVES / noct) {
                     const int orow = rc * a.rpi + row_sub;
                     const int orc = min(orow, a.RB - 1);
-                    v4i c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+                    v4i c0 = zero4, c1 = zero4;
 #pragma unroll
                     for (int dy = 0; dy < 3; ++dy) {
                         const v4i b = *reinterpret_cast<const v4i*>(ei + (orc + dy) * a.pitch);
-                        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wB[dy][0], b, c0, 0, 0, 0);
-                        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wB[dy][1], b, c1, 0, 0, 0);
+                        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wB[dy][0], b, dy ? c0 : zero4, 0, 0, 0);
+                        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(wB[dy][1], b, dy ? c1 : zero4, 0, 0, 0);
                     }
                     const int a8[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
                     const v2i r = epi8_quant_i8p8<NONNEG, 0>(a.e2, prm, a8);
@@ -173,32 +289,28 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
                 }
             }
         }
-        __syncthreads();
+        blk_barrier();
         // ================= C: project =================
-        {
-            const int kss = a.SL / 64;
+        if constexpr (!PFP) load_wP(s);
 #pragma unroll
-            for (int i = 0; i < BLK_NI; ++i) {
-                const int it = wave + BLK_WAVES * i;
-                if (it < a.itemsP) {  // wave-uniform
-                    const int prP = it % a.npairsP, gd = it / a.npairsP;
-                    for (int ks = 0; ks < kss; ++ks) {
-                        const int cgp = s * kss + ks;
-                        if (cgp >= a.cgP) break;
-                        const v4i* wg = reinterpret_cast<const v4i*>(a.w_prj) + ((size_t)cgp * a.mtP + 2 * prP) * 64 + lane;
-                        const v4i w0 = wg[0], w1 = wg[64];
+        for (int i = 0; i < NI; ++i) {
+            const int it = wave + BLK_WAVES * i;
+            if (it < a.itemsP) {  // wave-uniform
+                const int gd = it / a.npairsP;
+#pragma unroll
+                for (int ks = 0; ks < KSS; ++ks) {
+                    if (s * KSS + ks < a.cgP) {
                         const v4i b = *reinterpret_cast<const v4i*>(ldsD + (size_t)((gd * kqs + 4 * ks + q) * 16 + p) * 16);
-                        acc[i][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, b, acc[i][0], 0, 0, 0);
-                        acc[i][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, b, acc[i][1], 0, 0, 0);
+                        acc[i][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wP[i][ks][0], b, acc[i][0], 0, 0, 0);
+                        acc[i][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wP[i][ks][1], b, acc[i][1], 0, 0, 0);
                     }
                 }
             }
         }
     }
-
-    // ---- the project layer's epilogue ------------------------------------------------------------------------------
+    // ---- the project layer's epilogue (fp32: its constants and the band's shortcut elements wait in LDS) --------------
 #pragma unroll
-    for (int i = 0; i < BLK_NI; ++i) {
+    for (int i = 0; i < NI; ++i) {
         const int it = wave + BLK_WAVES * i;
         if (it >= a.itemsP) break;  // wave-uniform
         const int prP = it % a.npairsP, gd = it / a.npairsP;
@@ -214,14 +326,40 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
             const v2i r = epi8_quant_i8p8<false, 0>(a.e3, prm, a8);
             *reinterpret_cast<v2i*>((int8_t*)a.out + ((size_t)(n * (a.Cout / 8) + ch0 / 8) * a.HW + opix) * 8) = r;
         } else {
-            epi8_load<EPI_F32_P4>(prm, a.e3, ch0);
-            const size_t img = (size_t)n * a.Cout * a.HW;  // floats
-            const size_t elem = img + ((size_t)(ch0 / 4) * a.HW + opix) * 4;
+            // epi4_store_f32p4<true, 0> with the shortcut element and the constants read from LDS
+            {
+                const v4i* c = reinterpret_cast<const v4i*>(lds + a.lds_c3) + prP * 16 + 2 * q;
+                const v4i s0 = c[0], s1 = c[1], b0 = c[8], b1 = c[9];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
+                    prm.bi[e] = __int_as_float(b0[e]), prm.bi[4 + e] = __int_as_float(b1[e]);
+                }
+            }
+            const v4i* const rl = reinterpret_cast<const v4i*>(lds + a.lds_r) + (ch0 / 4) * out_pixN + pix;
+            const size_t elem = (size_t)n * a.Cout * a.HW + ((size_t)(ch0 / 4) * a.HW + opix) * 4;
             v2i tw = {0, 0};
-            tw[0] = (int)epi4_store_f32p4<true, 0>((float*)a.out, a.e3, prm.si, prm.bi, elem, a8[0], a8[1], a8[2], a8[3]);
-            if (ch0 + 4 < a.Cout)
-                tw[1] = (int)epi4_store_f32p4<true, 0>((float*)a.out, a.e3, prm.si + 4, prm.bi + 4, elem + (size_t)a.HW * 4,
-                                                       a8[4], a8[5], a8[6], a8[7]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (h == 1 && ch0 + 4 >= a.Cout) break;
+                v4i r, res = {0, 0, 0, 0};
+                if (a.e3.residual != nullptr) res = rl[h * out_pixN];  // wave-uniform
+                unsigned qv = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v = __fmaf_rn((float)a8[4 * h + e], prm.si[4 * h + e], prm.bi[4 * h + e]);
+                    v = fminf(fmaxf(v, a.e3.act_lo), a.e3.act_hi);
+                    if (a.e3.residual != nullptr) v = __fadd_rn(v, __int_as_float(res[e]));
+                    if (a.e3.twin != nullptr) {  // wave-uniform
+                        const float t = __fmul_rn(v, a.e3.twin_scale);
+                        const int k = (int)__fadd_rn(t, __builtin_copysignf(a.e3.twin_half, t));
+                        qv |= (unsigned)(min(max(k, -127), 127) & 0xff) << (8 * e);
+                    }
+                    r[e] = __float_as_int(v);
+                }
+                *reinterpret_cast<v4i*>((float*)a.out + elem + (size_t)h * a.HW * 4) = r;
+                tw[h] = (int)qv;
+            }
             if (a.e3.twin != nullptr)  // Cout % 8 == 0 then
                 *reinterpret_cast<v2i*>(a.e3.twin + ((size_t)(n * (a.Cout / 8) + ch0 / 8) * a.HW + opix) * 8) = tw;
         }
@@ -242,35 +380,42 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
     if (cgE > BLK_CGE) return false;
     const int npairsP = (Cout + 31) / 32;
     const int pitch = (4 * cpr + 4) * 8;
-    constexpr int kLdsMax = 64 * 1024;
-    auto fits = [&](int RB, int SL, int* lds_e, int* lds_d, int* total) {
+    constexpr int kLdsMax = 160 * 1024;
+    int off[6];  // expanded lines, depthwise results, expand / depthwise / project constants, shortcut elements
+    auto fits = [&](int RB, int SL, int* total) {
         const int rows_in = std::min(RB + 2, H);
         const int GA = (rows_in * W + 15) / 16, GD = (RB * W + 15) / 16;
         if (npairsP * GD > BLK_WAVES * BLK_NI) return false;
         const int x = GA * cgE * 1024;
         const int e = (SL / 8) * (RB + 2) * pitch;
         const int d = GD * (SL / 16) * 256;
-        *lds_e = x, *lds_d = x + (e + 255) / 256 * 256, *total = *lds_d + d;
+        const int c1 = ((Ce + 31) / 32) * BLK_PAIR_DW * 4, c2 = (Ce / 8) * BLK_OCT_DW * 4;
+        off[0] = x, off[1] = off[0] + (e + 255) / 256 * 256, off[2] = off[1] + d, off[3] = off[2] + c1;
+        off[4] = off[3] + c2, off[5] = off[4] + npairsP * 256;
+        *total = off[5] + (Cout / 4) * RB * W * 16;
         return *total <= kLdsMax;
     };
-    int RB = 0, SL = 0, le = 0, ld = 0, tot = 0;
+    int RB = 0, SL = 0, tot = 0;
     if (force_rb > 0 || force_sl > 0) {
         RB = force_rb > 0 ? std::min(force_rb, H) : std::min(H, std::max(rpi, 4));
         SL = force_sl == 64 || force_sl == 128 ? force_sl : 64;
-        if (!fits(RB, SL, &le, &ld, &tot)) return false;
+        if (!fits(RB, SL, &tot)) return false;
     } else {
         // the tallest band that still gives every compute unit a workgroup (fewer halo rows to expand twice), in steps
-        // of the depthwise item's rows; the wider slice where the expanded channels fill it and LDS allows
+        // of the depthwise item's rows; the wider slice where the expanded channels fill it. Two workgroups share a
+        // compute unit's LDS where there are more workgroups than compute units.
         const int sl_first = Ce > 64 ? 128 : 64;
         bool found = false;
         for (int rb = (H + rpi - 1) / rpi * rpi; rb >= 1 && !found; rb -= (rb > rpi ? rpi : 1)) {
             const int rbc = std::min(rb, H);
             const long wgs = (long)ge.N * ((H + rbc - 1) / rbc);
             if (wgs < 256 && rbc > std::max(rpi, 4)) continue;
+            const int budget = wgs > 256 ? 80 * 1024 : kLdsMax;
             for (int sl = sl_first; sl >= 64 && !found; sl -= 64)
-                if (fits(rbc, sl, &le, &ld, &tot)) RB = rbc, SL = sl, found = true;
+                if (fits(rbc, sl, &tot) && tot <= budget) RB = rbc, SL = sl, found = true;
         }
         if (!found) return false;
+        fits(RB, SL, &tot);
     }
     plan[0] = RB, plan[1] = (H + RB - 1) / RB, plan[2] = SL, plan[3] = tot;
     if (out) {
@@ -279,12 +424,12 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
         a.Ce = Ce, a.Ce8 = Ce / 8;
         a.cgP = igemm_channel_groups(Ce), a.mtP = igemm_padded_rows(Cout) / 16, a.Cout = Cout;
         a.H = H, a.W = W, a.HW = H * W;
-        a.RB = RB, a.bands = plan[1], a.SL = SL, a.slices = (Ce + SL - 1) / SL;
+        a.RB = RB, a.bands = plan[1], a.slices = (Ce + SL - 1) / SL;
         a.cpr = cpr, a.rpi = rpi, a.ER = RB + 2, a.pitch = pitch;
         a.GA = (std::min(RB + 2, H) * W + 15) / 16, a.GD = (RB * W + 15) / 16;
         a.npairsP = npairsP, a.itemsP = npairsP * a.GD;
         a.inv_w = ((1u << 20) + W - 1) / W;
-        a.lds_e = le, a.lds_d = ld;
+        a.lds_e = off[0], a.lds_d = off[1], a.lds_c1 = off[2], a.lds_c2 = off[3], a.lds_c3 = off[4], a.lds_r = off[5];
     }
     return true;
 }
@@ -310,25 +455,81 @@ bool conv_block_applicable(const ConvGeom& ge, const Epilogue& e1, const ConvGeo
     return p3 == EPI_F32_P4;
 }
 
-hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int8_t* w_dw, const int8_t* w_prj, void* out,
+// The per-channel constants of the expand layer as the kernel keeps them in LDS: per pair of 16-row tiles (32 channels)
+// [scale_in 32][bias 32][scale_out 32][16 words of two 16-bit upper clamps each]. si / bi / so hold `kpad` (a multiple
+// of 32) entries. nonneg: the layer clamps at zero (ReLU / clip) and every output scale is positive.
+size_t block_expand_const_bytes(int K) { return (size_t)((K + 31) / 32) * BLK_PAIR_DW * sizeof(int32_t); }
+void block_pack_expand_consts(const float* si, const float* bi, const float* so, int K, bool nonneg, float act_hi,
+                              float round_half, int32_t* dst) {
+    const int pairs = (K + 31) / 32;
+    std::vector<unsigned> qh(pairs * 16, 0u);
+    if (nonneg) conv_pw_stream_clamps(act_hi, round_half, so, pairs * 32, qh.data());
+    for (int pr = 0; pr < pairs; ++pr) {
+        int32_t* d = dst + (size_t)pr * BLK_PAIR_DW;
+        std::memcpy(d, si + 32 * pr, 128);
+        std::memcpy(d + 32, bi + 32 * pr, 128);
+        std::memcpy(d + 64, so + 32 * pr, 128);
+        std::memcpy(d + 96, qh.data() + 16 * pr, 64);
+    }
+}
+
+// The depthwise 3x3 layer as the kernel keeps it in LDS: per channel octet [kernel row 3][channel 8] words holding the
+// row's three taps in bytes 0..2, then [scale_in 8][bias 8][scale_out 8][4 words of two upper clamps each].
+size_t block_dw_const_bytes(int C) { return (size_t)(C / 8) * BLK_OCT_DW * sizeof(int32_t); }
+void block_pack_dw_consts(const int8_t* w, const float* si, const float* bi, const float* so, int C, bool nonneg, float act_hi,
+                          float round_half, int32_t* dst) {
+    std::vector<unsigned> qh(C / 2, 0u);
+    if (nonneg) conv_pw_stream_clamps(act_hi, round_half, so, C, qh.data());
+    for (int o = 0; o < C / 8; ++o) {
+        int32_t* d = dst + (size_t)o * BLK_OCT_DW;
+        for (int dy = 0; dy < 3; ++dy)
+            for (int c = 0; c < 8; ++c) {
+                const int8_t* t = w + (size_t)(8 * o + c) * 9 + dy * 3;
+                d[dy * 8 + c] = (int32_t)((uint32_t)(uint8_t)t[0] | (uint32_t)(uint8_t)t[1] << 8 | (uint32_t)(uint8_t)t[2] << 16);
+            }
+        std::memcpy(d + 24, si + 8 * o, 32);
+        std::memcpy(d + 32, bi + 8 * o, 32);
+        std::memcpy(d + 40, so + 8 * o, 32);
+        std::memcpy(d + 48, qh.data() + 4 * o, 16);
+    }
+}
+
+template <bool NN, int E3, int SL, int NI, int CGE>
+static hipError_t launch_block(const BlockArgs& a, const dim3& grid, size_t lds, hipStream_t stream) {
+    static bool raised = false;  // more than the default 64 KB of dynamic LDS has to be asked for, once per kernel
+    if (lds > 64 * 1024 && !raised) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<NN, E3, SL, NI, CGE>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL((conv_block_kernel<NN, E3, SL, NI, CGE>), grid, dim3(64 * BLK_WAVES), lds, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int32_t* k1, const int32_t* k2, const int8_t* w_prj, void* out,
                           const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
                           const Epilogue& e3, int force_rb, int force_sl, hipStream_t stream) {
     if (!conv_block_applicable(ge, e1, gd, e2, gp, e3)) return hipErrorInvalidValue;
     BlockArgs a;
     int plan[4];
     if (!conv_block_plan(ge, gp, force_rb, force_sl, plan, &a)) return hipErrorInvalidValue;
-    a.x = x, a.w_exp = w_exp, a.w_dw = w_dw, a.w_prj = w_prj, a.out = out;
+    a.x = x, a.w_exp = w_exp, a.k1 = k1, a.k2 = k2, a.w_prj = w_prj, a.out = out;
     a.e1 = e1, a.e2 = e2, a.e3 = e3;
-    const dim3 grid((unsigned)a.bands, (unsigned)ge.N), block(64 * BLK_WAVES);
+    const dim3 grid((unsigned)a.bands, (unsigned)ge.N);
     const bool nonneg = pick_epilogue(e1, ge.K) == EPI_I8_P8_NONNEG;
     const bool i8 = pick_epilogue(e3, gp.K) == EPI_I8_P8;
-#define OHIP_BLK(NN_, E3_) hipLaunchKernelGGL((conv_block_kernel<NN_, E3_>), grid, block, (size_t)plan[3], stream, a)
-    if (nonneg && i8) OHIP_BLK(true, EPI_I8_P8);
-    else if (nonneg) OHIP_BLK(true, EPI_F32_P4_FUSED);
-    else if (i8) OHIP_BLK(false, EPI_I8_P8);
-    else OHIP_BLK(false, EPI_F32_P4_FUSED);
-#undef OHIP_BLK
-    return hipGetLastError();
+    const bool wide = plan[2] == 128, few = a.itemsP <= BLK_WAVES;
+#define OHIP_BLK4(NN_, E3_, SL_, NI_) (a.cgE == 1 ? launch_block<NN_, E3_, SL_, NI_, 1>(a, grid, (size_t)plan[3], stream) \
+                                                  : launch_block<NN_, E3_, SL_, NI_, BLK_CGE>(a, grid, (size_t)plan[3], stream))
+#define OHIP_BLK3(NN_, E3_, SL_) (few ? OHIP_BLK4(NN_, E3_, SL_, 1) : OHIP_BLK4(NN_, E3_, SL_, BLK_NI))
+#define OHIP_BLK2(NN_, E3_) (wide ? OHIP_BLK3(NN_, E3_, 128) : OHIP_BLK3(NN_, E3_, 64))
+    if (nonneg) return i8 ? OHIP_BLK2(true, EPI_I8_P8) : OHIP_BLK2(true, EPI_F32_P4_FUSED);
+    return i8 ? OHIP_BLK2(false, EPI_I8_P8) : OHIP_BLK2(false, EPI_F32_P4_FUSED);
+#undef OHIP_BLK2
+#undef OHIP_BLK3
+#undef OHIP_BLK4
 }
 
 }  // namespace ohip
+

@@ -294,6 +294,7 @@ int otter_host_net_load_weight(void* net, const char* path, int ncnn) {
 // its weights as load_model will ask for them: "... K C groups kh kw bias_term int8_scale_term".
 // how many runs of convolution layers went through the chain entry point as one launch, in this process
 long otter_host_chain_forward_count(void) { return ConvolutionLayer::chain_forward_count(); }
+long otter_host_block_forward_count(void) { return ConvolutionLayer::block_forward_count(); }
 
 long otter_host_net_describe(void* net, char* buf, size_t capacity) {
     try {

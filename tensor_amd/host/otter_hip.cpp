@@ -706,6 +706,54 @@ int ConvolutionLayer::forward_chain(const std::vector<const ConvolutionLayer*>& 
     return 0;
 }
 
+static std::atomic<long> g_block_forwards{0};
+long ConvolutionLayer::block_forward_count() { return g_block_forwards.load(); }
+
+int ConvolutionLayer::forward_block(const ConvolutionLayer* e, const ConvolutionLayer* d, const ConvolutionLayer* p,
+                                    const Tensor& bottom, const Tensor* shortcut, float q_scale, int q_round, Tensor& top,
+                                    const NetOption& opt) {
+    if (!opt.use_packing_layout || !bottom.defined() || bottom.dim() != 4 || bottom.scalar_type() != ScalarType::Byte8) return 1;
+    if (!e->handle_ || !d->handle_ || !p->handle_ || e->int8_scale_term <= 100 || d->int8_scale_term <= 100 || !p->int8_scale_term)
+        return 1;
+    if (e->force_out_layout >= 0 || d->force_out_layout >= 0 || p->force_out_layout >= 0) return 1;
+    const int N = (int)bottom.size(0), H = (int)bottom.size(2), W = (int)bottom.size(3);
+    if (bottom.channels() != e->in_channels || p->out_channels % 8) return 1;
+    if (otter_hip_conv_block_launches(e->handle_, d->handle_, p->handle_, N, H, W) != 1) return 1;
+    int oh = H, ow = W;
+    for (const ConvolutionLayer* c : {e, d, p}) {
+        int h2 = 0, w2 = 0;
+        if (otter_hip_conv_output_shape(c->handle_, oh, ow, &h2, &w2)) return 1;
+        oh = h2, ow = w2;
+    }
+    const bool f32 = p->int8_scale_term <= 100;
+    const ScalarType odt = f32 ? ScalarType::Float4 : ScalarType::Byte8;
+    if (shortcut) {
+        if (!f32 || shortcut->scalar_type() != odt || shortcut->dim() != 4 || shortcut->size(0) != N ||
+            shortcut->channels() != p->out_channels || shortcut->size(2) != oh || shortcut->size(3) != ow)
+            return 1;
+    }
+    try {
+        top = Tensor::empty_device({N, p->out_channels / elempack_of(odt), oh, ow}, odt);
+        const bool with_q = f32 && q_scale > 0.f;
+        Tensor q;
+        if (with_q) q = Tensor::empty_device({N, p->out_channels / 8, oh, ow}, ScalarType::Byte8);
+        const int rc = otter_hip_conv_block_forward(e->handle_, d->handle_, p->handle_, bottom.device_ptr(), N, H, W,
+                                                    shortcut ? (const float*)shortcut->device_ptr() : nullptr, top.device_ptr(),
+                                                    f32 ? OTTER_HIP_F32_P4 : OTTER_HIP_I8_P8, with_q ? q.device_ptr() : nullptr,
+                                                    q_scale, q_round, nullptr, 0, nullptr);
+        if (rc) return rc;
+        top.mark_device_written();
+        if (with_q) {
+            q.mark_device_written();
+            top.attach_quantized(q, q_scale, q_round);
+        }
+        ++g_block_forwards;
+    } catch (const Error&) {
+        return -100;
+    }
+    return 0;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // functional API
 // ---------------------------------------------------------------------------------------------------
@@ -1589,6 +1637,15 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
         }
     }
     {
+        const auto unit = block_units_.find(li);
+        // only when neither blob inside the block has been computed (or set by the caller) yet
+        if (unit != block_units_.end() && !blobs[layers_[unit->second.expand]->tops[0]].defined() &&
+            !blobs[layers_[unit->second.depthwise]->tops[0]].defined()) {
+            const int rc = forward_block_unit(unit->second, li, -1, blobs, opt);
+            if (rc <= 0) return rc;
+        }
+    }
+    {
         const auto unit = chain_units_.find(li);
         if (unit != chain_units_.end()) {
             // only when nothing inside the run has been computed (or set by the caller) yet
@@ -1723,6 +1780,26 @@ void Net::plan_fused_quantize() const {
         shuffle_units_[lo] = u;
         shuffle_units_[hi] = u;
     }
+    // Inverted-residual blocks: 1x1 (int8 result) -> depthwise (int8 result) -> 1x1, each blob with one reader
+    block_units_.clear();
+    for (size_t li = 0; li < layers_.size(); ++li) {
+        const auto* pc = dynamic_cast<const ConvolutionLayer*>(layers_[li]);
+        auto pointwise = [](const ConvolutionLayer* c) {
+            return c->groups == 1 && c->kernel_height == 1 && c->kernel_width == 1 && c->stride_height == 1 &&
+                   c->stride_width == 1 && c->padding_height == 0 && c->padding_width == 0 && c->bottoms.size() == 1 &&
+                   c->tops.size() == 1 && c->force_out_layout < 0;
+        };
+        if (!pc || !pc->int8_scale_term || !pointwise(pc) || pc->out_channels % 8) continue;
+        const int di = blobs_[pc->bottoms[0]].producer;
+        const auto* dc = di < 0 ? nullptr : dynamic_cast<const ConvolutionLayer*>(layers_[di]);
+        if (!dc || dc->int8_scale_term <= 100 || dc->groups != dc->in_channels || dc->groups != dc->out_channels ||
+            dc->bottoms.size() != 1 || dc->force_out_layout >= 0 || sole_reader(dc->tops[0]) != (int)li)
+            continue;
+        const int ei = blobs_[dc->bottoms[0]].producer;
+        const auto* ec = ei < 0 ? nullptr : dynamic_cast<const ConvolutionLayer*>(layers_[ei]);
+        if (!ec || ec->int8_scale_term <= 100 || !pointwise(ec) || ec->in_channels % 8 || sole_reader(ec->tops[0]) != di) continue;
+        block_units_[(int)li] = BlockUnit{ei, di, (int)li};
+    }
     // Runs of int8 -> int8 convolutions, each blob read by the next convolution only (no Split: one reader), at most 8 long
     chain_units_.clear();
     auto chainable = [&](int li) {
@@ -1774,11 +1851,50 @@ int Net::forward_chain_unit(const std::vector<int>& run, std::vector<Tensor>& bl
     return 0;
 }
 
+// An inverted-residual block (and the sum with its shortcut) in one launch (ConvolutionLayer::forward_block). Returns 1
+// when the layers or the blobs at hand do not allow it; the caller then runs the layers one by one.
+int Net::forward_block_unit(const BlockUnit& u, int out_layer, int shortcut, std::vector<Tensor>& blobs,
+                            const NetOption& opt) const {
+    const auto* ec = static_cast<const ConvolutionLayer*>(layers_[u.expand]);
+    const auto* dc = static_cast<const ConvolutionLayer*>(layers_[u.depthwise]);
+    const auto* pc = static_cast<const ConvolutionLayer*>(layers_[u.project]);
+    const int in_blob = ec->bottoms[0];
+    for (int b : {shortcut, in_blob})
+        if (b >= 0 && !blobs[b].defined()) {
+            const int rc = forward_layer(blobs_[b].producer, blobs, opt);
+            if (rc) return rc;
+        }
+    // the block reads Byte8: the blob itself, or the int8 twin its producer made with the first layer's scale
+    Tensor bottom = blobs[in_blob], twin;
+    if (bottom.defined() && base_of(bottom.scalar_type()) == ScalarType::Float &&
+        bottom.quantized_twin(ec->bottom_blob_int8_scales.data_ptr<float>()[0], ec->input_round_mode(opt), twin))
+        bottom = twin;
+    const Layer* out = layers_[out_layer];
+    Tensor top;
+    const int rc = ConvolutionLayer::forward_block(ec, dc, pc, bottom, shortcut >= 0 ? &blobs[shortcut] : nullptr, out->fuse_scale,
+                                                   out->fuse_round, top, opt);
+    if (rc) return rc;
+    blobs[out->tops[0]] = top;
+    if (opt.lightmode)
+        for (int b : {shortcut, in_blob})
+            if (b >= 0 && blobs_[b].consumers.size() == 1) blobs[b] = Tensor();
+    return 0;
+}
+
 // Convolution and Eltwise sum in one launch (otter_hip_conv_forward_residual). Returns 1 when the blobs at hand do not
 // allow it; the caller then runs the layers one by one.
 int Net::forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const {
     const auto* conv = static_cast<const ConvolutionLayer*>(layers_[u.conv]);
     const Layer* e = layers_[u.eltwise];
+    {
+        // the convolution may be the last layer of an inverted-residual block: then the whole block and the sum in one launch
+        const auto bu = block_units_.find(u.conv);
+        if (bu != block_units_.end() && !blobs[layers_[bu->second.expand]->tops[0]].defined() &&
+            !blobs[layers_[bu->second.depthwise]->tops[0]].defined()) {
+            const int rc = forward_block_unit(bu->second, u.eltwise, u.shortcut, blobs, opt);
+            if (rc <= 0) return rc;
+        }
+    }
     for (int b : {u.shortcut, conv->bottoms[0]})
         if (!blobs[b].defined()) {
             const int rc = forward_layer(blobs_[b].producer, blobs, opt);

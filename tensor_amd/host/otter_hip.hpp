@@ -220,6 +220,12 @@ public:
     static int forward_chain(const std::vector<const ConvolutionLayer*>& run, const Tensor& bottom_blob, Tensor& top,
                              const NetOption& opt);
     static long chain_forward_count();  // runs executed that way so far in this process (for tests)
+    // expand (1x1, int8 result) -> depthwise (int8 result) -> project (1x1) [+ shortcut] as one launch
+    // (otter_hip_conv_block_forward). Returns 1 when the layers or the blobs at hand do not allow the single launch.
+    static int forward_block(const ConvolutionLayer* expand, const ConvolutionLayer* depthwise, const ConvolutionLayer* project,
+                             const Tensor& bottom_blob, const Tensor* shortcut, float q_scale, int q_round, Tensor& top,
+                             const NetOption& opt);
+    static long block_forward_count();  // blocks executed that way so far in this process (for tests)
 
 private:
     int create_pipeline_int8(const NetOption& opt);
@@ -319,6 +325,18 @@ private:
     int forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
     // Runs of 2..8 int8 -> int8 convolution layers, each read only by the next, found by the plan: last layer's index ->
     // the run; forward_layer hands the run to ConvolutionLayer::forward_chain when none of its blobs exists yet.
+    // Inverted-residual blocks, found by the plan: a 1x1 convolution whose only input is the int8 result of a depthwise
+    // convolution read by nothing else, which in turn reads the int8 result of a 1x1 convolution read by nothing else.
+    // Last layer's index -> the three; forward_layer (and the residual unit the last layer may be part of) hands them to
+    // ConvolutionLayer::forward_block when neither inner blob exists yet.
+    struct BlockUnit {
+        int expand, depthwise, project;
+    };
+    mutable std::map<int, BlockUnit> block_units_;
+    // out_layer: the layer whose top blob receives the result (the project layer, or the Eltwise sum behind it when
+    // shortcut >= 0)
+    int forward_block_unit(const BlockUnit& u, int out_layer, int shortcut, std::vector<Tensor>& blobs,
+                           const NetOption& opt) const;
     mutable std::map<int, std::vector<int>> chain_units_;
     int forward_chain_unit(const std::vector<int>& run, std::vector<Tensor>& blobs, const NetOption& opt) const;
 };

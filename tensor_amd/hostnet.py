@@ -14,7 +14,7 @@ EXPORTS = ["otter_host_last_error", "otter_host_net_create", "otter_host_net_des
            "otter_host_session_pass", "otter_host_session_fetch", "otter_host_session_destroy",
            "otter_host_functional_chain", "otter_host_net_load_otter", "otter_host_net_load_weight",
            "otter_host_net_describe", "otter_host_net_conv_fp32_probe", "otter_host_net_eval", "otter_host_otter_dump", "otter_host_ncnn_read",
-           "otter_host_chain_forward_count"]
+           "otter_host_chain_forward_count", "otter_host_block_forward_count"]
 
 
 def load_cdll():
@@ -29,7 +29,13 @@ def load_cdll():
     lib.otter_host_otter_dump.restype = C.c_long
     lib.otter_host_ncnn_read.restype = C.c_long
     lib.otter_host_chain_forward_count.restype = C.c_long
+    lib.otter_host_block_forward_count.restype = C.c_long
     return lib
+
+
+def block_forward_count():
+    """Inverted-residual blocks the Nets of this process have run as one launch so far."""
+    return load_cdll().otter_host_block_forward_count()
 
 
 def chain_forward_count():

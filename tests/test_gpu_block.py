@@ -12,6 +12,15 @@ pytestmark = pytest.mark.gpu
 FP32_RTOL = 1e-5
 
 
+@pytest.fixture(autouse=True)
+def every_qualifying_block_as_one_launch(hip):
+    """By default the single launch is only taken for the shapes it was measured faster on; the tests here exercise it
+    on every shape it can run."""
+    before = hip.conv_block_set_always(1)
+    yield
+    hip.conv_block_set_always(before)
+
+
 def quantize_weights(wf):
     K = wf.shape[0]
     ws = (np.float32(127) / np.abs(wf).reshape(K, -1).max(axis=1)).astype(np.float32)
@@ -110,6 +119,18 @@ def test_block_equals_the_three_layers(hip, oracle, cin, ce, cout, N, H, W, act,
         assert (out == cur).all()
     for l in layers:
         l["conv"].close()
+
+
+def test_default_policy_takes_the_measured_shapes_only(hip):
+    hip.conv_block_set_always(0)
+    rng = np.random.default_rng(3)
+    for (cin, ce, cout, n, hw, want) in [(64, 384, 64, 64, 14, 1), (32, 192, 32, 64, 28, 1), (24, 144, 24, 64, 56, 3),
+                                          (160, 960, 160, 64, 7, 3), (96, 576, 96, 64, 14, 3), (64, 384, 64, 4, 14, 3)]:
+        layers = make_block(hip, rng, cin, ce, cout, 3, True)
+        e, d, p = (l["conv"] for l in layers)
+        assert hip.conv_block_launches(e, d, p, n, hw, hw) == want
+        for l in layers:
+            l["conv"].close()
 
 
 def test_block_falls_back_to_three_launches(hip):

@@ -35,3 +35,41 @@ def test_network_matches_oracle_layer_by_layer(hip, oracle):
             np.testing.assert_allclose(got, want[name], rtol=1e-5, atol=1e-30, err_msg=name)
     got = net.run("data", x, "fc").reshape(batch, -1)
     np.testing.assert_allclose(got, want["fc"], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_network_with_blocks_as_single_launches(hip, oracle):
+    """The same network with every inverted-residual block that qualifies by shape run as one launch
+    (otter_hip_conv_block_forward through Net's block units): the blobs behind the blocks equal the oracle's and, bit
+    for bit, those of the layers one by one; a blob asked for inside a block still comes from the layers one by one."""
+    rng = np.random.default_rng(0)
+    hw, batch = 64, 2
+    layers = mobilenet.describe(num_classes=50)
+    params = mobilenet.init_weights(layers, rng)
+    mobilenet.calibrate(hip, capi, layers, params, rng.uniform(0, 1, (4, 3, hw, hw)).astype(np.float32))
+    net = mobilenet.build_net(hostnet, layers, params, batch, hw, num_classes=50)
+    x = rng.uniform(0, 1, (batch, 3, hw, hw)).astype(np.float32)
+    want = mobilenet.oracle_forward(oracle, layers, params, x)
+    names = ("b2_add", "b5_add", "b9_add", "b10_project", "b12_add", "b15_add", "b16_project", "head")
+    plain = {name: net.run("data", x, name) for name in names}
+    before = hip.conv_block_set_always(1)
+    try:
+        count0 = hostnet.block_forward_count()
+        for name in names:
+            got = net.run("data", x, name)
+            assert got.tobytes() == plain[name].tobytes(), name
+            if got.dtype == np.int8:
+                np.testing.assert_array_equal(got, want[name], err_msg=name)
+            else:
+                np.testing.assert_allclose(got, want[name], rtol=1e-5, atol=1e-30, err_msg=name)
+        # the stride-1 blocks with an expand layer: b2, b4, b5, b7..b12, b14, b15, b16 = 12 of them up to the head
+        # (Net.run makes two passes: one for the shape, one to fetch)
+        count1 = hostnet.block_forward_count()
+        assert count1 > count0
+        net.run("data", x, "head")
+        assert hostnet.block_forward_count() - count1 == 2 * 12
+        # a blob inside a block: the layers run one by one up to it, same bytes as before
+        inner = net.run("data", x, "b8_dw")
+        np.testing.assert_array_equal(inner, want["b8_dw"])
+    finally:
+        hip.conv_block_set_always(before)

@@ -209,7 +209,7 @@ int otter_hip_conv_chain_set_min_tiles(int tiles);
  * calls give, bit for bit. Where the depthwise layer is stride 1 pad 1 on an image at most 64 pixels wide, the first
  * layer reads at most 192 channels and the activations are none / ReLU / clip, the block can run as ONE launch that
  * keeps the expanded tensor in LDS and needs no workspace; it does (otter_hip_conv_block_launches says 1) for the
- * shapes where that was measured faster than the three launches (at most 64 input channels, images up to 28 pixels
+ * shapes where that was measured faster than the three launches (at most 128 input channels, images up to 28 pixels
  * wide, 128..512 bands of rows over the batch), or for every shape that qualifies after
  * otter_hip_conv_block_set_always(1) / a forced plan. Otherwise the call makes three launches with the two intermediate
  * blobs in `workspace` (otter_hip_conv_block_workspace_bytes). */

@@ -226,6 +226,14 @@ class Library:
                                                   int(align_corner), self.ptr(dst), dst_layout, self.stream()))
         return dst
 
+    def inner_product(self, x, n, in_features, weight, bias, out_features):
+        """otter_hip_inner_product: y[n][o] = sum_i x[n][i] * weight[o][i] + bias[o] (device tensors; bias may be None)."""
+        y = self.empty(n * out_features, np.float32)
+        self._check(self.lib.otter_hip_inner_product(self.ptr(x), n, in_features, self.ptr(weight),
+                                                     self.ptr(bias) if bias is not None else None, out_features,
+                                                     self.ptr(y), self.stream()))
+        return y
+
     def eltwise_add_quantize(self, a, b, layout, shape, scale, round_mode):
         n, c, h, w = shape
         out = self.empty(n * c * h * w, np.float32)

@@ -781,9 +781,10 @@ static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_
     // rows of one image each) about fill the 256 compute units once. Measured at batch 64 against the three launches:
     // 14x14 64 -> 384 -> 64 13.2 us against 17.8 us, 28x28 32 -> 192 -> 32 16.8 against 21.8; 56x56 (896 workgroups
     // of 13 us each) 56 against 45, 7x7 (64 workgroups, the requantization of a whole image on one compute unit's
-    // vector ALUs) 38 against 20, more than 64 input channels (reduction steps in registers, spills) 24 against 23.5.
+    // vector ALUs) 38 against 20; 14x14 96 -> 576 -> 96 21.8 against 23.5 (29.8 inside a network, where the three
+    // launches start on cold inputs).
     const long wgs = (long)g[0].N * plan[1];
-    return g[0].C <= 64 && g[0].W <= 28 && wgs >= 128 && wgs <= 512;
+    return g[0].C <= 128 && g[0].W <= 28 && wgs >= 128 && wgs <= 512;
 }
 
 static int block_default_out_layout(const otter_hip_conv_t* p) {

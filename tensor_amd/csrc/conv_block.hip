@@ -97,60 +97,77 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
             wA[cg][1] = wg[o + 64];
         }
     };
-    load_wA(0);
 
-    // ---- prologue: zero the expanded lines (their borders are never written), stage the input as MFMA B operands,
-    // the per-channel constants of the expand and depthwise layers and the depthwise weights ---------------------------
+    // ---- prologue: stage the input as MFMA B operands, the per-channel constants of the three layers, the depthwise
+    // weights and the band's shortcut elements; zero the expanded lines (their borders are never written). Every array's
+    // first round of loads is requested before any is waited for: one memory latency for the lot. ----------------------
     {
-        const int e16 = noct * a.ER * a.pitch / 16;
-        v4i* e = reinterpret_cast<v4i*>(ldsE);
-        for (int i = tid; i < e16; i += 64 * BLK_WAVES) e[i] = v4i{0, 0, 0, 0};
-        const int total = a.GA * a.cgE * 64;
+        constexpr int T = 64 * BLK_WAVES;
+        const int nX = a.GA * a.cgE * 64;
         const int8_t* xi = a.x + (size_t)n * a.Cin8 * a.HW * 8;
-#pragma unroll 2
-        for (int i = tid; i < total; i += 64 * BLK_WAVES) {
+        auto load_x = [&](int i, v2i& lo, v2i& hi) {
             const int l = i & 63, t = i >> 6;
             const int ga = t / a.cgE, cg = t - ga * a.cgE;
             const int pix = ga * 16 + (l & 15), oct = 8 * cg + 2 * (l >> 4);
-            v2i lo = {0, 0}, hi = {0, 0};
-            if (pix < in_pixN) {
+            lo = hi = v2i{0, 0};
+            if (i < nX && pix < in_pixN) {
                 const int8_t* s = xi + ((size_t)oct * a.HW + in_pix0 + pix) * 8;
                 if (oct < a.Cin8) lo = *reinterpret_cast<const v2i*>(s);
                 if (oct + 1 < a.Cin8) hi = *reinterpret_cast<const v2i*>(s + (size_t)a.HW * 8);
             }
-            blk_lds[i] = v4i{lo[0], lo[1], hi[0], hi[1]};
-        }
-        // the two layers' constants and the depthwise weights, as the host laid them out (straight copies)
+        };
         v4i* c1 = reinterpret_cast<v4i*>(lds + a.lds_c1);
         const v4i* g1 = reinterpret_cast<const v4i*>(a.k1);
         const int n1 = ((a.Ce + 31) / 32) * (BLK_PAIR_DW / 4);
-#pragma unroll 2
-        for (int i = tid; i < n1; i += 64 * BLK_WAVES) c1[i] = g1[i];
         v4i* c2 = reinterpret_cast<v4i*>(lds + a.lds_c2);
         const v4i* g2 = reinterpret_cast<const v4i*>(a.k2);
         const int n2 = a.Ce8 * (BLK_OCT_DW / 4);
-#pragma unroll 4
-        for (int i = tid; i < n2; i += 64 * BLK_WAVES) c2[i] = g2[i];
-        if constexpr (EPI3 != EPI_I8_P8) {
-            // project: [channel pair][scale_in 32][bias 32] (the arrays are padded to whole pairs), and the band's elements
-            // of the shortcut blob as [channel quad][pixel of the band]
-            int* c3 = reinterpret_cast<int*>(lds + a.lds_c3);
-            const int n3 = a.npairsP * 64;
-            for (int i = tid; i < n3; i += 64 * BLK_WAVES) {
-                const int pr = i >> 6, r = i & 63;
-                c3[i] = __float_as_int(r < 32 ? a.e3.scale_in[32 * pr + r] : a.e3.bias[32 * pr + r - 32]);
-            }
-            if (a.e3.residual != nullptr) {  // uniform
-                v4i* rl = reinterpret_cast<v4i*>(lds + a.lds_r);
-                const v4i* rg = reinterpret_cast<const v4i*>(a.e3.residual) + (size_t)n * (a.Cout / 4) * a.HW + r0 * a.W;
-                const int n4 = (a.Cout / 4) * out_pixN;
-#pragma unroll 2
-                for (int i = tid; i < n4; i += 64 * BLK_WAVES) {
-                    const int c4 = i / out_pixN, px = i - c4 * out_pixN;
-                    rl[i] = rg[(size_t)c4 * a.HW + px];
-                }
-            }
+        // project (fp32 result): [channel pair][scale_in 32][bias 32] (the arrays are padded to whole pairs), and the
+        // band's elements of the shortcut blob as [channel quad][pixel of the band]
+        constexpr bool F32 = EPI3 != EPI_I8_P8;
+        int* c3 = reinterpret_cast<int*>(lds + a.lds_c3);
+        const int n3 = F32 ? a.npairsP * 64 : 0;
+        auto load_c3 = [&](int i) {
+            const int pr = i >> 6, r = i & 63;
+            return __float_as_int(r < 32 ? a.e3.scale_in[32 * pr + r] : a.e3.bias[32 * pr + r - 32]);
+        };
+        v4i* rl = reinterpret_cast<v4i*>(lds + a.lds_r);
+        const bool with_res = F32 && a.e3.residual != nullptr;
+        const v4i* rg = reinterpret_cast<const v4i*>(a.e3.residual) + (size_t)n * (a.Cout / 4) * a.HW + r0 * a.W;
+        const int n4 = with_res ? (a.Cout / 4) * out_pixN : 0;
+        auto load_res = [&](int i) {
+            const int c4 = i / out_pixN, px = i - c4 * out_pixN;
+            return rg[(size_t)c4 * a.HW + px];
+        };
+        // first round
+        v2i xlo, xhi;
+        load_x(tid, xlo, xhi);
+        v4i k1v = {0, 0, 0, 0}, k2v = {0, 0, 0, 0}, rv = {0, 0, 0, 0};
+        int k3v = 0;
+        if (tid < n1) k1v = g1[tid];
+        if (tid < n2) k2v = g2[tid];
+        if (tid < n3) k3v = load_c3(tid);
+        if (tid < n4) rv = load_res(tid);
+        load_wA(0);
+        const int e16 = noct * a.ER * a.pitch / 16;
+        v4i* e = reinterpret_cast<v4i*>(ldsE);
+        for (int i = tid; i < e16; i += T) e[i] = v4i{0, 0, 0, 0};
+        if (tid < nX) blk_lds[tid] = v4i{xlo[0], xlo[1], xhi[0], xhi[1]};
+        if (tid < n1) c1[tid] = k1v;
+        if (tid < n2) c2[tid] = k2v;
+        if (tid < n3) c3[tid] = k3v;
+        if (tid < n4) rl[tid] = rv;
+        // the rest
+        for (int i = tid + T; i < nX; i += T) {
+            load_x(i, xlo, xhi);
+            blk_lds[i] = v4i{xlo[0], xlo[1], xhi[0], xhi[1]};
         }
+        for (int i = tid + T; i < n1; i += T) c1[i] = g1[i];
+#pragma unroll 2
+        for (int i = tid + T; i < n2; i += T) c2[i] = g2[i];
+        for (int i = tid + T; i < n3; i += T) c3[i] = load_c3(i);
+#pragma unroll 2
+        for (int i = tid + T; i < n4; i += T) rl[i] = load_res(i);
     }
 
     // B: lane column -> (row within the item, column chunk); selectors that move a row's tap into the lane's byte of
@@ -521,7 +538,8 @@ hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int32_t* k
     const bool i8 = pick_epilogue(e3, gp.K) == EPI_I8_P8;
     const bool wide = plan[2] == 128, few = a.itemsP <= BLK_WAVES;
 #define OHIP_BLK4(NN_, E3_, SL_, NI_) (a.cgE == 1 ? launch_block<NN_, E3_, SL_, NI_, 1>(a, grid, (size_t)plan[3], stream) \
-                                                  : launch_block<NN_, E3_, SL_, NI_, BLK_CGE>(a, grid, (size_t)plan[3], stream))
+                                      : a.cgE == 2 ? launch_block<NN_, E3_, SL_, NI_, 2>(a, grid, (size_t)plan[3], stream) \
+                                                   : launch_block<NN_, E3_, SL_, NI_, BLK_CGE>(a, grid, (size_t)plan[3], stream))
 #define OHIP_BLK3(NN_, E3_, SL_) (few ? OHIP_BLK4(NN_, E3_, SL_, 1) : OHIP_BLK4(NN_, E3_, SL_, BLK_NI))
 #define OHIP_BLK2(NN_, E3_) (wide ? OHIP_BLK3(NN_, E3_, 128) : OHIP_BLK3(NN_, E3_, 64))
     if (nonneg) return i8 ? OHIP_BLK2(true, EPI_I8_P8) : OHIP_BLK2(true, EPI_F32_P4_FUSED);

@@ -192,49 +192,44 @@ hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, fl
 }
 
 // The same product on the fp32 matrix cores, for the shapes of a classifier (a batch of up to a few hundred rows, IN a
-// multiple of 16): the kernel above re-reads the weights once per 8 rows of x; here a workgroup owns 16 outputs, reads
-// their weight rows ONCE and multiplies them with up to 64 rows of x per pass. v_mfma_f32_16x16x4f32: lane (i, kq)
+// multiple of 16): the kernel above re-reads the weights once per 8 rows of x and multiplies on the vector ALU; here a
+// workgroup multiplies 16 weight rows with 16 rows of x. v_mfma_f32_16x16x4f32: lane (i, kq)
 // supplies A[i][kq] and B[kq][i]; with one 16-byte load per lane (4 consecutive inputs of weight row i / x row i) four
-// instructions cover 16 inputs. The four waves split the inputs and add their accumulators up through LDS.
+// instructions cover 16 inputs. The waves split the inputs and add their accumulators up through LDS.
 typedef float ip_v4f __attribute__((ext_vector_type(4)));
-__global__ void __launch_bounds__(256) inner_product_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                                 const float* __restrict__ b, float* __restrict__ y, int N,
-                                                                 int IN, int OUT) {
-    __shared__ ip_v4f part[4][4][64];
+constexpr int IPM_WAVES = 16;  // the inputs are dealt to 16 waves: a wave requests all its loads at once (one memory latency)
+// A workgroup owns 16 outputs x 16 rows of x: enough workgroups to put every compute unit's memory pipeline to work
+// (1000 outputs x 64 rows: 252 of them), each weight row read once per 16 rows of x.
+__global__ void __launch_bounds__(64 * IPM_WAVES) inner_product_mfma_kernel(const float* __restrict__ x,
+                                                                            const float* __restrict__ w,
+                                                                            const float* __restrict__ b, float* __restrict__ y,
+                                                                            int N, int IN, int OUT) {
+    __shared__ ip_v4f part[IPM_WAVES][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, kq = lane >> 4;
-    const int o0 = blockIdx.x * 16, n0 = blockIdx.y * 64;
+    const int o0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
     const float* wr = w + (size_t)min(o0 + i, OUT - 1) * IN + 4 * kq;  // clamped rows are computed, not stored
-    const float* xr[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) xr[g] = x + (size_t)min(n0 + 16 * g + i, N - 1) * IN + 4 * kq;
-    ip_v4f acc[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) acc[g] = ip_v4f{0.f, 0.f, 0.f, 0.f};
+    const float* xr = x + (size_t)min(n0 + i, N - 1) * IN + 4 * kq;
+    ip_v4f acc = {0.f, 0.f, 0.f, 0.f};
     const int steps = IN / 16;
-#pragma unroll 2
-    for (int st = wave; st < steps; st += 4) {
+#pragma unroll 5
+    for (int st = wave; st < steps; st += IPM_WAVES) {
         const ip_v4f a = *reinterpret_cast<const ip_v4f*>(wr + 16 * st);
-        ip_v4f bv[4];
+        const ip_v4f bv = *reinterpret_cast<const ip_v4f*>(xr + 16 * st);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) bv[g] = *reinterpret_cast<const ip_v4f*>(xr[g] + 16 * st);
-#pragma unroll
-        for (int m = 0; m < 4; ++m)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m], bv[g][m], acc[g], 0, 0, 0);
+        for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m], bv[m], acc, 0, 0, 0);
     }
-#pragma unroll
-    for (int g = 0; g < 4; ++g) part[wave][g][lane] = acc[g];
+    part[wave][lane] = acc;
     __syncthreads();
-    // wave g adds up image group g: lane (i, kq) holds outputs o0 + 4 kq + r of x row n0 + 16 g + i
-    const int g = wave;
-    ip_v4f s = part[0][g][lane];
+    if (wave) return;
+    // lane (i, kq) holds outputs o0 + 4 kq + r of x row n0 + i
+    ip_v4f s = part[0][lane];
 #pragma unroll
-    for (int v = 1; v < 4; ++v) {
-        const ip_v4f t = part[v][g][lane];
+    for (int v = 1; v < IPM_WAVES; ++v) {
+        const ip_v4f t = part[v][lane];
         s = ip_v4f{s[0] + t[0], s[1] + t[1], s[2] + t[2], s[3] + t[3]};
     }
-    const int n = n0 + 16 * g + i;
+    const int n = n0 + i;
     if (n < N) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -248,7 +243,7 @@ hipError_t run_inner_product(const float* x, const float* w, const float* b, flo
                              hipStream_t stream) {
     if (N * OUT == 0) return hipSuccess;
     if (IN % 16 == 0 && IN >= 64 && N >= 16 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
-        hipLaunchKernelGGL(inner_product_mfma_kernel, dim3((OUT + 15) / 16, (N + 63) / 64), dim3(256), 0, stream, x, w, b, y,
+        hipLaunchKernelGGL(inner_product_mfma_kernel, dim3((OUT + 15) / 16, (N + 15) / 16), dim3(64 * IPM_WAVES), 0, stream, x, w, b, y,
                            N, IN, OUT);
         return hipGetLastError();
     }

@@ -208,11 +208,14 @@ int otter_hip_conv_chain_set_min_tiles(int tiles);
  * otter_hip_conv_forward_residual / _twin) or int8 Byte8 (residual and out_q NULL). The result is what the three (four)
  * calls give, bit for bit. Where the depthwise layer is stride 1 pad 1 on an image at most 64 pixels wide, the first
  * layer reads at most 192 channels and the activations are none / ReLU / clip, the block can run as ONE launch that
- * keeps the expanded tensor in LDS and needs no workspace; it does (otter_hip_conv_block_launches says 1) for the
- * shapes where that was measured faster than the three launches (at most 128 input channels, images up to 28 pixels
- * wide, 128..512 bands of rows over the batch), or for every shape that qualifies after
- * otter_hip_conv_block_set_always(1) / a forced plan. Otherwise the call makes three launches with the two intermediate
- * blobs in `workspace` (otter_hip_conv_block_workspace_bytes). */
+ * keeps the expanded tensor in LDS; it does (otter_hip_conv_block_launches says 1) for the
+ * shapes where that was measured faster than the three launches (images up to 28 pixels wide, 128..512 workgroups
+ * over the batch, at most 24 tiles of 32 channels x 16 pixels of the last layer per band), or for every shape that qualifies after
+ * otter_hip_conv_block_set_always(1) / a forced plan. Where a batch has fewer bands than half the compute units, the
+ * expanded channels of a band are dealt to several workgroups whose accumulators meet in `workspace` (the last to
+ * arrive adds them up: integer sums, the same result). Otherwise the call makes three launches with the two
+ * intermediate blobs in `workspace`. otter_hip_conv_block_workspace_bytes gives the size either way (0 for a single
+ * launch with one workgroup per band). */
 int otter_hip_conv_block_launches(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
                                   const otter_hip_conv_t* project, int n, int in_h, int in_w);
 size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
@@ -225,9 +228,10 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* expand, const otter_hip
  * launch, 0 = only the shapes measured faster that way (default). Process-wide; returns the previous value; a negative
  * argument only queries. */
 int otter_hip_conv_block_set_always(int on);
-/* Tuning / test hook with no counterpart in the reference: force the single launch's output rows per band and the
- * expanded channels per LDS slice (64 or 128) of blocks whose first layer is `expand`; 0 = automatic. */
-int otter_hip_conv_block_set_plan(otter_hip_conv_t* expand, int rows_per_band, int slice_channels);
+/* Tuning / test hook with no counterpart in the reference: force the single launch's output rows per band, the
+ * expanded channels per LDS slice (64 or 128) and the workgroups a band's slices are dealt to, for blocks whose first
+ * layer is `expand`; 0 = automatic. */
+int otter_hip_conv_block_set_plan(otter_hip_conv_t* expand, int rows_per_band, int slice_channels, int split);
 
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked

@@ -342,8 +342,8 @@ class Conv:
     def set_tile(self, tm, tn):
         self.L._check(self.L.lib.otter_hip_conv_set_tile(self.h, tm, tn))
 
-    def set_block_plan(self, rows_per_band, slice_channels):
-        self.L._check(self.L.lib.otter_hip_conv_block_set_plan(self.h, rows_per_band, slice_channels))
+    def set_block_plan(self, rows_per_band, slice_channels, split=0):
+        self.L._check(self.L.lib.otter_hip_conv_block_set_plan(self.h, rows_per_band, slice_channels, split))
 
     def forward(self, x, in_layout, n, h, w, out_layout=None, out=None, workspace=None):
         out_layout = self.default_out_layout() if out_layout is None else out_layout

@@ -105,7 +105,7 @@ struct otter_hip_conv {
     float* in_scale = nullptr;   // [1]
     int c_pad = 0;               // > 0: C is not a multiple of 8; the MFMA path runs on C zero-padded to c_pad
     int force_tm = 0, force_tn = 0;
-    int block_rb = 0, block_sl = 0;  // forced plan of the fused block launch this layer heads (0 = automatic)
+    int block_rb = 0, block_sl = 0, block_split = 0;  // forced plan of the fused block launch this layer heads (0 = automatic)
 };
 
 extern "C" {
@@ -768,23 +768,25 @@ static bool block_geoms(const otter_hip_conv_t* e, const otter_hip_conv_t* d, co
 static int g_block_always = 0;  // see block_single_launch
 
 static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
-                                const ConvGeom g[3], int out_layout) {
+                                const ConvGeom g[3], int out_layout, int plan[6]) {
     if (!e->w_igemm || e->c_pad || e->force_tm || !e->blk_consts || !d->depthwise || !d->blk_consts || d->c_pad || d->force_tm || !p->w_igemm ||
         p->c_pad || p->force_tm)
         return false;
     const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8), e3 = make_epilogue(p, out_layout);
     if (!conv_block_applicable(g[0], e1, g[1], e2, g[2], e3)) return false;
-    int plan[4];
-    if (!conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, plan)) return false;
-    if (g_block_always || e->block_rb || e->block_sl) return true;
+    if (!conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, e->block_split, plan)) return false;
+    if (g_block_always || e->block_rb || e->block_sl || e->block_split) return true;
     // The single launch pays where the three layers are short, latency-bound launches and its workgroups (a band of
-    // rows of one image each) about fill the 256 compute units once. Measured at batch 64 against the three launches:
-    // 14x14 64 -> 384 -> 64 13.2 us against 17.8 us, 28x28 32 -> 192 -> 32 16.8 against 21.8; 56x56 (896 workgroups
-    // of 13 us each) 56 against 45, 7x7 (64 workgroups, the requantization of a whole image on one compute unit's
-    // vector ALUs) 38 against 20; 14x14 96 -> 576 -> 96 21.8 against 23.5 (29.8 inside a network, where the three
-    // launches start on cold inputs).
-    const long wgs = (long)g[0].N * plan[1];
-    return g[0].C <= 128 && g[0].W <= 28 && wgs >= 128 && wgs <= 512;
+    // rows of one image each, or a share of a band's expanded channels) about fill the 256 compute units once.
+    // Measured at batch 64 against the three launches (kernel trace; in brackets the three launches inside a network,
+    // where each starts on cold inputs): 14x14 64 -> 384 -> 64 13.2 us against 17.8, 14x14 96 -> 576 -> 96 21.8 against
+    // 23.5 (29.8), 28x28 32 -> 192 -> 32 16.8 against 21.8, 7x7 160 -> 960 -> 160 with the slices of an image dealt to
+    // four workgroups 18.5 against 20 (23.4). Not taken: 56x56 24 -> 144 -> 24 (896 workgroups of 13 us each on 256
+    // compute units) 56 against 45, 7x7 160 -> 960 -> 320 (more project items per wave than registers for their
+    // weights) 23.9 against 24.4.
+    const long wgs = (long)g[0].N * plan[1] * plan[4];
+    const int items = ((g[2].K + 31) / 32) * ((plan[0] * g[0].W + 15) / 16);
+    return g[0].C <= 192 && g[0].W <= 28 && wgs >= 128 && wgs <= 512 && items <= 24;
 }
 
 static int block_default_out_layout(const otter_hip_conv_t* p) {
@@ -797,7 +799,8 @@ int otter_hip_conv_block_launches(const otter_hip_conv_t* e, const otter_hip_con
     if (rc) return rc;
     ConvGeom g[3];
     if (!block_geoms(e, d, p, n, in_h, in_w, g)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_launches: empty output");
-    return n >= 1 && p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p)) ? 1 : 3;
+    int plan[6];
+    return n >= 1 && p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p), plan) ? 1 : 3;
 }
 
 size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
@@ -805,7 +808,9 @@ size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const ott
     if (!e || !d || !p || n < 1 || in_h < 1 || in_w < 1) return 0;
     ConvGeom g[3];
     if (!block_geoms(e, d, p, n, in_h, in_w, g)) return 0;
-    if (p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p))) return 0;
+    int plan[6];
+    if (p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p), plan))
+        return (size_t)plan[5] * sizeof(int);  // the accumulators of a band's workgroups, when there are several
     const size_t b0 = (size_t)n * g[0].K * g[0].OH * g[0].OW, b1 = (size_t)n * g[1].K * g[1].OH * g[1].OW;
     return (b0 + 255) / 256 * 256 + (b1 + 255) / 256 * 256;
 }
@@ -816,10 +821,10 @@ int otter_hip_conv_block_set_always(int on) {
     return before;
 }
 
-int otter_hip_conv_block_set_plan(otter_hip_conv_t* e, int rows_per_band, int slice_channels) {
-    if (!e || rows_per_band < 0 || (slice_channels != 0 && slice_channels != 64 && slice_channels != 128))
+int otter_hip_conv_block_set_plan(otter_hip_conv_t* e, int rows_per_band, int slice_channels, int split) {
+    if (!e || rows_per_band < 0 || split < 0 || (slice_channels != 0 && slice_channels != 64 && slice_channels != 128))
         return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_set_plan: bad argument");
-    e->block_rb = rows_per_band, e->block_sl = slice_channels;
+    e->block_rb = rows_per_band, e->block_sl = slice_channels, e->block_split = split;
     return OTTER_HIP_OK;
 }
 
@@ -848,14 +853,19 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* e, const otter_hip_conv
     if (n == 0) return OTTER_HIP_OK;
     hipStream_t stream = (hipStream_t)stream_;
 
-    if (p->d.out_channels % 8 == 0 && out_layout == block_default_out_layout(p) && block_single_launch(e, d, p, g, out_layout)) {
+    int plan[6];
+    if (p->d.out_channels % 8 == 0 && out_layout == block_default_out_layout(p) && block_single_launch(e, d, p, g, out_layout, plan)) {
+        const size_t need1 = (size_t)plan[5] * sizeof(int);
+        if (need1 && (!workspace || workspace_bytes < need1))
+            return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_forward: needs the workspace reported by "
+                                               "otter_hip_conv_block_workspace_bytes");
         const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8);
         Epilogue e3 = make_epilogue(p, out_layout);
         e3.residual = residual;
         e3.twin = (int8_t*)out_q, e3.twin_scale = q_scale;
         e3.twin_half = q_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
         OHIP_CHECK(run_conv_block((const int8_t*)in, e->w_igemm, e->blk_consts, d->blk_consts, p->w_igemm, out, g[0], e1, g[1], e2, g[2], e3,
-                                  e->block_rb, e->block_sl, stream));
+                                  e->block_rb, e->block_sl, e->block_split, (int*)workspace, stream));
         return OTTER_HIP_OK;
     }
     // the layers one after the other, the intermediate blobs in the workspace

@@ -17,6 +17,7 @@
 // Every intermediate value is the one the three layers would have written: same accumulators, same epilogue code.
 #include <algorithm>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "common.hpp"
@@ -26,9 +27,9 @@ namespace ohip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v4u_blk __attribute__((__vector_size__(4 * sizeof(unsigned))));
 
-constexpr int BLK_WAVES = 16;
-constexpr int BLK_NI = 3;    // (channel pair, pixel group) items of the project layer per wave, at most
+constexpr int BLK_NI8 = 6;   // (channel pair, pixel group) items of the project layer per wave, at most (8 waves)
 constexpr int BLK_CGE = 3;   // 64-channel reduction steps of the expand layer, at most (192 input channels)
 constexpr int BLK_PAIR_DW = 112;  // LDS dwords of one expand channel pair's constants: scale_in, bias, scale_out (32 each), 16 clamps
 constexpr int BLK_OCT_DW = 52;    // LDS dwords of one depthwise octet: 3 x 8 weight words, scale_in, bias, scale_out (8 each), 4 clamps
@@ -52,15 +53,23 @@ struct BlockArgs {
     unsigned inv_w;       // ceil(2^20 / W)
     int lds_e, lds_d, lds_c1, lds_c2;  // byte offsets: expanded lines, depthwise results, constants of the two layers
     int lds_c3, lds_r;                 // constants of the project layer, the band's shortcut elements (fp32 result only)
+    // The slices of a band dealt to `split` workgroups (grid.z), `spp` consecutive slices each: each adds its slices
+    // into accumulators of its own, writes them to `partial` and counts itself in at counters[band of the batch]; the
+    // last one to arrive adds the others' up and runs the epilogue.
+    int split, spp;
+    int* partial;        // [band of the batch][split][item][tile 2][lane 64][4] accumulators
+    int partial_bytes;
+    unsigned* counters;  // zero before the launch, and again after it
 };
 
 // LDS visibility between the phases needs the LDS counter only: the weight loads requested ahead stay in flight
 __device__ __forceinline__ void blk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // EPI3: EPI_F32_P4_FUSED (fp32 Float4, optional residual and twin in e3) or EPI_I8_P8 (signed int8 Byte8)
-// SL: expanded channels per slice; NI: project items per wave; CGE: reduction steps of the expand layer (at least cgE)
-template <bool NONNEG, int EPI3, int SL, int NI, int CGE>
-__global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockArgs a) {
+// SL: expanded channels per slice; NI: project items per wave; CGE: reduction steps of the expand layer (at least cgE);
+// WV: waves per workgroup (16 where the registers of a quarter SIMD do, 8 with twice the registers otherwise)
+template <bool NONNEG, int EPI3, int SL, int NI, int CGE, int WV>
+__global__ void __launch_bounds__(64 * WV) conv_block_kernel(const BlockArgs a) {
     extern __shared__ v4i blk_lds[];
     char* const lds = reinterpret_cast<char*>(blk_lds);
     char* const ldsE = lds + a.lds_e;
@@ -71,6 +80,7 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 15, q = lane >> 4;
     const int band = blockIdx.x, n = blockIdx.y;
+    const int s_begin = blockIdx.z * a.spp, s_end = min(s_begin + a.spp, a.slices);
     // bands of nearly equal height (at most RB rows): band b owns rows [b * H / bands, (b + 1) * H / bands)
     const int r0 = band * a.H / a.bands, rows = (band + 1) * a.H / a.bands - r0;
     const int in_row0 = max(r0 - 1, 0), in_row1 = min(r0 + rows, a.H - 1);
@@ -78,10 +88,11 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
     const int out_pixN = rows * a.W;
 
     constexpr int npairsE = SL / 32, noct = SL / 8, kqs = SL / 16, KSS = SL / 64;
-    static_assert(BLK_WAVES % noct == 0, "a wave keeps one octet of the slice");
+    constexpr int OPW = noct > WV ? noct / WV : 1;  // octets of a slice per wave (16 over 8 waves: two)
+    static_assert(noct % WV == 0 || WV % noct == 0, "the octets of a slice divide evenly over the waves");
     // A: pair of the slice and first pixel group of this wave
     const int prE = wave % npairsE, gaE0 = wave / npairsE;
-    constexpr int gaEs = BLK_WAVES / npairsE;
+    constexpr int gaEs = WV / npairsE;
 
     // the expand weights of a slice: this wave's channel pair, every reduction step
     v4i wA[CGE][2];
@@ -102,7 +113,7 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
     // weights and the band's shortcut elements; zero the expanded lines (their borders are never written). Every array's
     // first round of loads is requested before any is waited for: one memory latency for the lot. ----------------------
     {
-        constexpr int T = 64 * BLK_WAVES;
+        constexpr int T = 64 * WV;
         const int nX = a.GA * a.cgE * 64;
         const int8_t* xi = a.x + (size_t)n * a.Cin8 * a.HW * 8;
         auto load_x = [&](int i, v2i& lo, v2i& hi) {
@@ -148,7 +159,7 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
         if (tid < n2) k2v = g2[tid];
         if (tid < n3) k3v = load_c3(tid);
         if (tid < n4) rv = load_res(tid);
-        load_wA(0);
+        load_wA(s_begin);
         const int e16 = noct * a.ER * a.pitch / 16;
         v4i* e = reinterpret_cast<v4i*>(ldsE);
         for (int i = tid; i < e16; i += T) e[i] = v4i{0, 0, 0, 0};
@@ -195,12 +206,12 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
     v4i acc[NI][2];
 #pragma unroll
     for (int i = 0; i < NI; ++i) acc[i][0] = acc[i][1] = v4i{0, 0, 0, 0};
-    constexpr bool PFP = NI == 1;  // the project weights are requested a phase ahead where the registers allow
+    constexpr bool PFP = NI == 1 || (WV == 8 && NI <= 3);  // the project weights are requested a phase ahead where the registers allow
     v4i wP[NI][KSS][2];
     auto load_wP = [&](int s) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int prP = min(wave + BLK_WAVES * i, a.itemsP - 1) % a.npairsP;
+            const int prP = min(wave + WV * i, a.itemsP - 1) % a.npairsP;
 #pragma unroll
             for (int ks = 0; ks < KSS; ++ks) {
                 const int cgp = min(s * KSS + ks, a.cgP - 1);
@@ -211,7 +222,7 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
     };
     blk_barrier();
 
-    for (int s = 0; s < a.slices; ++s) {
+    for (int s = s_begin; s < s_end; ++s) {
         // ================= A: expand =================
         if constexpr (PFP) load_wP(s);
         {
@@ -260,10 +271,12 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
         }
         blk_barrier();
         // ================= B: depthwise =================
-        if (s + 1 < a.slices) load_wA(s + 1);
+        if (s + 1 < s_end) load_wA(s + 1);
         {
             const int nrc = (rows + a.rpi - 1) / a.rpi;
-            const int ol = wave % noct;
+#pragma unroll
+            for (int k = 0; k < OPW; ++k) {
+            const int ol = wave % noct + WV * k;
             const int oct_abs = s * noct + ol;
             if (oct_abs < a.Ce8) {  // wave-uniform
                 const int* const c = ldsC2 + oct_abs * BLK_OCT_DW;
@@ -287,7 +300,7 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
                 }
                 const char* const ei = ldsE + (size_t)(ol * a.ER) * a.pitch + (4 * nx + 2 * q) * 8;
                 char* const dout = ldsD + (size_t)(ol >> 1) * 256 + (ol & 1) * 8;
-                for (int rc = wave / noct; rc < nrc; rc += BLK_WAVES / noct) {
+                for (int rc = WV > noct ? wave / noct : 0; rc < nrc; rc += WV > noct ? WV / noct : 1) {
                     const int orow = rc * a.rpi + row_sub;
                     const int orc = min(orow, a.RB - 1);
                     v4i c0 = zero4, c1 = zero4;
@@ -305,13 +318,14 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
                     }
                 }
             }
+            }
         }
         blk_barrier();
         // ================= C: project =================
         if constexpr (!PFP) load_wP(s);
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int it = wave + BLK_WAVES * i;
+            const int it = wave + WV * i;
             if (it < a.itemsP) {  // wave-uniform
                 const int gd = it / a.npairsP;
 #pragma unroll
@@ -325,10 +339,52 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
             }
         }
     }
+    // ---- several workgroups per band: the last to arrive collects the others' accumulators --------------------------
+    if (a.split > 1) {
+        const int bi = n * a.bands + band;
+        // The accumulators travel through memory at agent scope (sc1): the stores go through to the level all compute
+        // units share and the loads do not hit in a cache that could hold older data, so the hand-over needs no
+        // write-back or invalidation of a whole L2.
+        constexpr int AGENT = 1 << 4;
+        const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(a.partial, 0, a.partial_bytes, 0x00020000);
+        const unsigned mine = ((unsigned)(bi * a.split + (int)blockIdx.z) * (unsigned)a.itemsP) * 2048u + (unsigned)lane * 16u;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int it = wave + WV * i;
+            if (it < a.itemsP) {  // wave-uniform
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_blk, acc[i][0]), rp, (int)(mine + (unsigned)it * 2048u), 0, AGENT);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_blk, acc[i][1]), rp, (int)(mine + (unsigned)it * 2048u + 1024u), 0, AGENT);
+            }
+        }
+        __syncthreads();  // every wave's stores are acknowledged (the barrier's wait covers the memory counter)
+        int* const flag = reinterpret_cast<int*>(ldsD);  // (the depthwise results are not read any more)
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(a.counters + bi, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const bool last = before == (unsigned)(a.split - 1);
+            if (last) __hip_atomic_store(a.counters + bi, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+            *flag = last ? 1 : 0;
+        }
+        __syncthreads();
+        if (*flag == 0) return;  // whole workgroup
+        for (int z = 0; z < a.split; ++z) {
+            if (z == (int)blockIdx.z) continue;
+            const unsigned theirs = ((unsigned)(bi * a.split + z) * (unsigned)a.itemsP) * 2048u + (unsigned)lane * 16u;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int it = wave + WV * i;
+                if (it < a.itemsP) {  // wave-uniform
+                    const v4i t0 = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rp, (int)(theirs + (unsigned)it * 2048u), 0, AGENT));
+                    const v4i t1 = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rp, (int)(theirs + (unsigned)it * 2048u + 1024u), 0, AGENT));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][0][e] += t0[e], acc[i][1][e] += t1[e];
+                }
+            }
+        }
+    }
     // ---- the project layer's epilogue (fp32: its constants and the band's shortcut elements wait in LDS) --------------
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-        const int it = wave + BLK_WAVES * i;
+        const int it = wave + WV * i;
         if (it >= a.itemsP) break;  // wave-uniform
         const int prP = it % a.npairsP, gd = it / a.npairsP;
         const int ch0 = 32 * prP + 8 * q;
@@ -387,9 +443,11 @@ __global__ void __launch_bounds__(64 * BLK_WAVES) conv_block_kernel(const BlockA
 // host side
 // ---------------------------------------------------------------------------------------------------------------------
 
-// plan[0] = rows per band, plan[1] = bands, plan[2] = slice (expanded channels), plan[3] = LDS bytes
-// force_rb / force_sl: 0 = automatic
-bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int force_sl, int plan[4], BlockArgs* out) {
+// plan[0] = rows per band, plan[1] = bands, plan[2] = slice (expanded channels), plan[3] = LDS bytes, plan[4] = workgroups
+// per band (each takes a share of the slices), plan[5] = ints of workspace for their accumulators (0 when plan[4] == 1)
+// force_rb / force_sl / force_split: 0 = automatic
+bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int force_sl, int force_split, int plan[6],
+                     BlockArgs* out) {
     const int W = ge.W, H = ge.H, Ce = ge.K, Cout = gp.K;
     if (W > 64 || W < 1 || H < 1) return false;
     const int cpr = (W + 3) / 4, rpi = 16 / cpr;
@@ -402,7 +460,7 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
     auto fits = [&](int RB, int SL, int* total) {
         const int rows_in = std::min(RB + 2, H);
         const int GA = (rows_in * W + 15) / 16, GD = (RB * W + 15) / 16;
-        if (npairsP * GD > BLK_WAVES * BLK_NI) return false;
+        if (npairsP * GD > 8 * BLK_NI8) return false;
         const int x = GA * cgE * 1024;
         const int e = (SL / 8) * (RB + 2) * pitch;
         const int d = GD * (SL / 16) * 256;
@@ -435,7 +493,20 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
         fits(RB, SL, &tot);
     }
     plan[0] = RB, plan[1] = (H + RB - 1) / RB, plan[2] = SL, plan[3] = tot;
+    // Fewer bands than half the compute units: the slices of a band are dealt to several workgroups
+    const int slices = (Ce + SL - 1) / SL;
+    const long wgs1 = (long)ge.N * plan[1];
+    int split = force_split > 0 ? force_split : (wgs1 < 128 ? (int)std::min<long>(slices, 256 / wgs1) : 1);
+    split = std::max(1, std::min(split, slices));
+    const int spp = (slices + split - 1) / split;
+    split = (slices + spp - 1) / spp;  // no workgroup without a slice
+    const int GDp = (RB * W + 15) / 16;
+    plan[4] = split;
+    const long ws = split > 1 ? wgs1 * split * npairsP * GDp * 512 : 0;
+    if (ws >= (1l << 28) || wgs1 > 65536) return false;
+    plan[5] = (int)ws;
     if (out) {
+        out->split = split, out->spp = spp;
         BlockArgs& a = *out;
         a.Cin8 = ge.C / 8, a.cgE = cgE, a.mtE = igemm_padded_rows(Ce) / 16;
         a.Ce = Ce, a.Ce8 = Ce / 8;
@@ -511,41 +582,76 @@ void block_pack_dw_consts(const int8_t* w, const float* si, const float* bi, con
     }
 }
 
-template <bool NN, int E3, int SL, int NI, int CGE>
+// The arrival counters of the bands whose slices are dealt to several workgroups: a ring in static device memory (every
+// GPU has its own copy; the address is looked up once per device). A launch takes the next N x bands words; the last
+// workgroup of a band leaves its word at zero again, so the ring needs no clearing, and launches that overlap on
+// different streams count in different words.
+constexpr int BLK_COUNTERS = 1 << 17;
+static __device__ unsigned blk_counters[BLK_COUNTERS];
+static std::mutex g_counter_mutex;
+static unsigned* g_counter_ptr[64] = {};
+static unsigned g_counter_next[64] = {};
+
+static hipError_t block_counters(int words, unsigned** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || words > BLK_COUNTERS / 2) return hipErrorInvalidValue;
+    std::lock_guard<std::mutex> lock(g_counter_mutex);
+    if (!g_counter_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(blk_counters));
+        if (e != hipSuccess || !p) return e == hipSuccess ? hipErrorInvalidSymbol : e;
+        g_counter_ptr[dev] = static_cast<unsigned*>(p);
+    }
+    if (g_counter_next[dev] + (unsigned)words > (unsigned)BLK_COUNTERS) g_counter_next[dev] = 0;
+    *out = g_counter_ptr[dev] + g_counter_next[dev];
+    g_counter_next[dev] += (unsigned)words;
+    return hipSuccess;
+}
+
+template <bool NN, int E3, int SL, int NI, int CGE, int WV>
 static hipError_t launch_block(const BlockArgs& a, const dim3& grid, size_t lds, hipStream_t stream) {
     static bool raised = false;  // more than the default 64 KB of dynamic LDS has to be asked for, once per kernel
     if (lds > 64 * 1024 && !raised) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<NN, E3, SL, NI, CGE>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<NN, E3, SL, NI, CGE, WV>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         raised = true;
     }
-    hipLaunchKernelGGL((conv_block_kernel<NN, E3, SL, NI, CGE>), grid, dim3(64 * BLK_WAVES), lds, stream, a);
+    hipLaunchKernelGGL((conv_block_kernel<NN, E3, SL, NI, CGE, WV>), grid, dim3(64 * WV), lds, stream, a);
     return hipGetLastError();
 }
 
 hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int32_t* k1, const int32_t* k2, const int8_t* w_prj, void* out,
                           const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
-                          const Epilogue& e3, int force_rb, int force_sl, hipStream_t stream) {
+                          const Epilogue& e3, int force_rb, int force_sl, int force_split, int* workspace, hipStream_t stream) {
     if (!conv_block_applicable(ge, e1, gd, e2, gp, e3)) return hipErrorInvalidValue;
     BlockArgs a;
-    int plan[4];
-    if (!conv_block_plan(ge, gp, force_rb, force_sl, plan, &a)) return hipErrorInvalidValue;
+    int plan[6];
+    if (!conv_block_plan(ge, gp, force_rb, force_sl, force_split, plan, &a)) return hipErrorInvalidValue;
+    a.partial = workspace, a.partial_bytes = plan[5] * 4, a.counters = nullptr;
+    if (plan[4] > 1) {
+        if (!workspace) return hipErrorInvalidValue;
+        const hipError_t ce = block_counters(ge.N * plan[1], &a.counters);
+        if (ce != hipSuccess) return ce;
+    }
     a.x = x, a.w_exp = w_exp, a.k1 = k1, a.k2 = k2, a.w_prj = w_prj, a.out = out;
     a.e1 = e1, a.e2 = e2, a.e3 = e3;
-    const dim3 grid((unsigned)a.bands, (unsigned)ge.N);
+    const dim3 grid((unsigned)a.bands, (unsigned)ge.N, (unsigned)plan[4]);
     const bool nonneg = pick_epilogue(e1, ge.K) == EPI_I8_P8_NONNEG;
     const bool i8 = pick_epilogue(e3, gp.K) == EPI_I8_P8;
-    const bool wide = plan[2] == 128, few = a.itemsP <= BLK_WAVES;
-#define OHIP_BLK4(NN_, E3_, SL_, NI_) (a.cgE == 1 ? launch_block<NN_, E3_, SL_, NI_, 1>(a, grid, (size_t)plan[3], stream) \
-                                      : a.cgE == 2 ? launch_block<NN_, E3_, SL_, NI_, 2>(a, grid, (size_t)plan[3], stream) \
-                                                   : launch_block<NN_, E3_, SL_, NI_, BLK_CGE>(a, grid, (size_t)plan[3], stream))
-#define OHIP_BLK3(NN_, E3_, SL_) (few ? OHIP_BLK4(NN_, E3_, SL_, 1) : OHIP_BLK4(NN_, E3_, SL_, BLK_NI))
-#define OHIP_BLK2(NN_, E3_) (wide ? OHIP_BLK3(NN_, E3_, 128) : OHIP_BLK3(NN_, E3_, 64))
+    // 16 waves where one reduction step and one project item per wave keep a wave within a quarter of a SIMD's registers;
+    // 8 waves, with twice the registers each, for the shapes that would spill there
+    const bool wide = plan[2] == 128, w16 = a.cgE == 1 && a.itemsP <= 16, few = a.itemsP <= 24;
+#define OHIP_BLK4(NN_, E3_, SL_) \
+    (w16 ? launch_block<NN_, E3_, SL_, 1, 1, 16>(a, grid, (size_t)plan[3], stream) \
+         : few ? launch_block<NN_, E3_, SL_, 3, BLK_CGE, 8>(a, grid, (size_t)plan[3], stream) \
+               : launch_block<NN_, E3_, SL_, BLK_NI8, BLK_CGE, 8>(a, grid, (size_t)plan[3], stream))
+#define OHIP_BLK2(NN_, E3_) (wide ? OHIP_BLK4(NN_, E3_, 128) : OHIP_BLK4(NN_, E3_, 64))
     if (nonneg) return i8 ? OHIP_BLK2(true, EPI_I8_P8) : OHIP_BLK2(true, EPI_F32_P4_FUSED);
     return i8 ? OHIP_BLK2(false, EPI_I8_P8) : OHIP_BLK2(false, EPI_F32_P4_FUSED);
 #undef OHIP_BLK2
-#undef OHIP_BLK3
 #undef OHIP_BLK4
 }
 

@@ -28,7 +28,8 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
 bool conv_block_applicable(const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
                            const Epilogue& e3);
 struct BlockArgs;
-bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int force_sl, int plan[4], BlockArgs* out = nullptr);
+bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int force_sl, int force_split, int plan[6],
+                     BlockArgs* out = nullptr);
 size_t block_expand_const_bytes(int K);
 void block_pack_expand_consts(const float* si, const float* bi, const float* so, int K, bool nonneg, float act_hi,
                               float round_half, int32_t* dst);
@@ -37,7 +38,7 @@ void block_pack_dw_consts(const int8_t* w, const float* si, const float* bi, con
                           float round_half, int32_t* dst);
 hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int32_t* k1, const int32_t* k2, const int8_t* w_prj, void* out,
                           const ConvGeom& ge, const Epilogue& e1, const ConvGeom& gd, const Epilogue& e2, const ConvGeom& gp,
-                          const Epilogue& e3, int force_rb, int force_sl, hipStream_t stream);
+                          const Epilogue& e3, int force_rb, int force_sl, int force_split, int* workspace, hipStream_t stream);
 
 // conv3x3.hip
 bool conv3x3_halo_supported(const ConvGeom& g, const Epilogue& ep);

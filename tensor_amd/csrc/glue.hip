@@ -242,7 +242,8 @@ __global__ void __launch_bounds__(64 * IPM_WAVES) inner_product_mfma_kernel(cons
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream) {
     if (N * OUT == 0) return hipSuccess;
-    if (IN % 16 == 0 && IN >= 64 && N >= 16 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
+    // (the choice must not depend on N: a row's result is then the same bits whatever batch it sits in)
+    if (IN % 16 == 0 && IN >= 64 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
         hipLaunchKernelGGL(inner_product_mfma_kernel, dim3((OUT + 15) / 16, (N + 15) / 16), dim3(64 * IPM_WAVES), 0, stream, x, w, b, y,
                            N, IN, OUT);
         return hipGetLastError();

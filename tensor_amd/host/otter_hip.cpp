@@ -737,10 +737,13 @@ int ConvolutionLayer::forward_block(const ConvolutionLayer* e, const Convolution
         const bool with_q = f32 && q_scale > 0.f;
         Tensor q;
         if (with_q) q = Tensor::empty_device({N, p->out_channels / 8, oh, ow}, ScalarType::Byte8);
+        const size_t ws_bytes = otter_hip_conv_block_workspace_bytes(e->handle_, d->handle_, p->handle_, N, H, W);
+        Tensor ws;
+        if (ws_bytes) ws = Tensor::empty_device({(int64_t)ws_bytes}, ScalarType::Byte);
         const int rc = otter_hip_conv_block_forward(e->handle_, d->handle_, p->handle_, bottom.device_ptr(), N, H, W,
                                                     shortcut ? (const float*)shortcut->device_ptr() : nullptr, top.device_ptr(),
                                                     f32 ? OTTER_HIP_F32_P4 : OTTER_HIP_I8_P8, with_q ? q.device_ptr() : nullptr,
-                                                    q_scale, q_round, nullptr, 0, nullptr);
+                                                    q_scale, q_round, ws_bytes ? ws.device_ptr() : nullptr, ws_bytes, nullptr);
         if (rc) return rc;
         top.mark_device_written();
         if (with_q) {

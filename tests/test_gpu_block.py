@@ -74,6 +74,10 @@ CASES = [
     (40, 136, 24, 2, 11, 13, 0, True, False, False, None),    # no activation (signed blobs), odd sizes, nothing fused behind
     (16, 96, 24, 2, 9, 64, 3, True, False, False, None),      # the widest image the launch takes
     (8, 48, 8, 1, 1, 1, 3, True, True, True, None),           # a single pixel
+    (160, 960, 160, 5, 7, 7, 3, True, True, True, (0, 0, 4)),  # a band's slices dealt to four workgroups
+    (64, 384, 64, 3, 14, 14, 3, True, True, True, (4, 64, 3)),  # six slices over three workgroups per band
+    (160, 960, 320, 3, 7, 7, 3, False, False, False, (0, 128, 8)),  # one slice per workgroup, int8 result
+    (32, 200, 32, 2, 10, 12, 0, True, True, False, (0, 64, 3)),  # four slices over three workgroups: the last takes none... two
 ]
 
 
@@ -125,7 +129,8 @@ def test_default_policy_takes_the_measured_shapes_only(hip):
     hip.conv_block_set_always(0)
     rng = np.random.default_rng(3)
     for (cin, ce, cout, n, hw, want) in [(64, 384, 64, 64, 14, 1), (32, 192, 32, 64, 28, 1), (24, 144, 24, 64, 56, 3),
-                                          (160, 960, 160, 64, 7, 3), (96, 576, 96, 64, 14, 1), (64, 384, 64, 4, 14, 3)]:
+                                          (160, 960, 160, 64, 7, 1), (160, 960, 320, 64, 7, 3), (96, 576, 96, 64, 14, 1), (64, 384, 64, 4, 14, 3),
+                                          (64, 384, 64, 16, 14, 1)]:
         layers = make_block(hip, rng, cin, ce, cout, 3, True)
         e, d, p = (l["conv"] for l in layers)
         assert hip.conv_block_launches(e, d, p, n, hw, hw) == want

@@ -204,13 +204,17 @@ def test_glue_argument_errors(hip):
 @pytest.mark.parametrize("N,IN,OUT,bias", [(64, 1280, 1000, True), (17, 64, 5, True), (100, 96, 33, False),
                                            (16, 1280, 1000, True), (3, 1280, 10, True), (40, 72, 16, True)])
 def test_inner_product_against_float64(hip, N, IN, OUT, bias):
-    """Both kernels behind otter_hip_inner_product (the matrix-core one takes 16 or more rows with IN % 16 == 0, the
-    vector one the rest): y = x w^T + b against a float64 product, to fp32 summation accuracy. The weight is not
-    symmetric and x has a distinct row per image, so a transposed operand or a misplaced row fails."""
+    """Both kernels behind otter_hip_inner_product (the matrix-core one takes IN % 16 == 0 from 64 inputs on, the vector
+    one the rest): y = x w^T + b against a float64 product, to fp32 summation accuracy. The weight is not symmetric and
+    x has a distinct row per image, so a transposed operand or a misplaced row fails. A row's result does not depend
+    on the batch it sits in."""
     rng = np.random.default_rng(N + IN)
     x = rng.normal(0, 1, (N, IN)).astype(np.float32)
     w = rng.normal(0, 0.05, (OUT, IN)).astype(np.float32)
     b = rng.normal(0, 1, OUT).astype(np.float32) if bias else None
     y = hip.inner_product(hip.to_device(x), N, IN, hip.to_device(w), hip.to_device(b) if bias else None, OUT)
     want = x.astype(np.float64) @ w.astype(np.float64).T + (b.astype(np.float64) if bias else 0.0)
-    np.testing.assert_allclose(y.cpu().numpy().reshape(N, OUT), want, rtol=1e-4, atol=1e-4)
+    got = y.cpu().numpy().reshape(N, OUT)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+    alone = hip.inner_product(hip.to_device(x[N - 1:]), 1, IN, hip.to_device(w), hip.to_device(b) if bias else None, OUT)
+    np.testing.assert_array_equal(alone.cpu().numpy().reshape(1, OUT), got[N - 1:])

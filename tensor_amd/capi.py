@@ -261,17 +261,21 @@ class Library:
                                                           C.c_size_t(ws_bytes), self.stream()))
         return out
 
-    def conv_block(self, expand, dw, project, x, n, h, w, residual=None, q_scale=None, q_round_mode=ROUND_SSE):
+    def conv_block(self, expand, dw, project, x, n, h, w, residual=None, q_scale=None, q_round_mode=ROUND_SSE, out=None,
+                   q=None, workspace=None):
         """otter_hip_conv_block_forward: x (int8 Byte8) through expand -> depthwise -> project (+ residual), and with
         q_scale the Byte8 quantization of the result. Returns (out, q or None)."""
         oh, ow = dw.out_hw(*expand.out_hw(h, w))
         oh, ow = project.out_hw(oh, ow)
         f32 = project.out_kind == OUT_F32
         out_layout = F32_P4 if f32 else I8_P8
-        out = self.empty(n * project.K * oh * ow, np.float32 if f32 else np.int8)
-        q = self.empty(n * project.K * oh * ow, np.int8) if q_scale is not None else None
+        if out is None:
+            out = self.empty(n * project.K * oh * ow, np.float32 if f32 else np.int8)
+        if q is None and q_scale is not None:
+            q = self.empty(n * project.K * oh * ow, np.int8)
         ws_bytes = self.lib.otter_hip_conv_block_workspace_bytes(expand.h, dw.h, project.h, n, h, w)
-        workspace = self.empty(ws_bytes, np.int8) if ws_bytes else None
+        if ws_bytes and workspace is None:
+            workspace = self.empty(ws_bytes, np.int8)
         self._check(self.lib.otter_hip_conv_block_forward(
             expand.h, dw.h, project.h, self.ptr(x), n, h, w, self.ptr(residual) if residual is not None else None,
             self.ptr(out), out_layout, self.ptr(q) if q is not None else None, C.c_float(q_scale or 0.0), q_round_mode,

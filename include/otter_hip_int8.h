@@ -224,6 +224,13 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* expand, const otter_hip
                                  const otter_hip_conv_t* project, const void* in, int n, int in_h, int in_w,
                                  const float* residual, void* out, int out_layout, void* out_q, float q_scale,
                                  int q_round_mode, void* workspace, size_t workspace_bytes, void* stream);
+/* Test hook with no counterpart in the reference, host arithmetic only (no GPU needed): the launch plan of the single
+ * launch for a block in_channels -> expanded_channels -> out_channels on n images of in_h x in_w (stride-1 depthwise
+ * layer), with rows_per_band / slice_channels / split forced (0 = automatic). plan = { output rows per band, bands per
+ * image, expanded channels per slice, LDS bytes per workgroup, workgroups per band (each takes a share of the slices),
+ * 32-bit words of workspace for their accumulators }. -1 when the single launch cannot take the shape. */
+int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_channels, int n, int in_h, int in_w,
+                              int rows_per_band, int slice_channels, int split, int plan[6]);
 /* Tuning / test hook with no counterpart in the reference: 1 = every block that qualifies by shape runs as the single
  * launch, 0 = only the shapes measured faster that way (default). Process-wide; returns the previous value; a negative
  * argument only queries. */

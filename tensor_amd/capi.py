@@ -74,7 +74,8 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
-           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always"]
+           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always",
+           "otter_hip_conv_block_plan"]
 
 
 def load_cdll():

@@ -815,6 +815,23 @@ size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const ott
     return (b0 + 255) / 256 * 256 + (b1 + 255) / 256 * 256;
 }
 
+int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_channels, int n, int in_h, int in_w,
+                              int rows_per_band, int slice_channels, int split, int plan[6]) {
+    if (!plan || in_channels < 8 || in_channels % 8 || expanded_channels < 8 || expanded_channels % 8 || out_channels < 8 ||
+        out_channels % 8 || n < 1 || in_h < 1 || in_w < 1 || rows_per_band < 0 || split < 0 ||
+        (slice_channels != 0 && slice_channels != 64 && slice_channels != 128))
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_plan: bad argument");
+    otter_hip_conv_desc d{};
+    d.kernel_h = d.kernel_w = 1, d.stride_h = d.stride_w = 1, d.dilation_h = d.dilation_w = 1, d.groups = 1;
+    d.in_channels = in_channels, d.out_channels = expanded_channels;
+    const ConvGeom ge = make_geom(d, n, in_h, in_w);
+    d.in_channels = expanded_channels, d.out_channels = out_channels;
+    const ConvGeom gp = make_geom(d, n, in_h, in_w);
+    if (!conv_block_plan(ge, gp, rows_per_band, slice_channels, split, plan))
+        return fail(OTTER_HIP_ERR_UNSUPPORTED, "otter_hip_conv_block_plan: the single launch does not take this shape");
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_conv_block_set_always(int on) {
     const int before = g_block_always;
     if (on >= 0) g_block_always = on ? 1 : 0;

@@ -16,6 +16,7 @@
 // Two barriers per slice (A|B, B|C); C of one slice and A of the next run without one.
 // Every intermediate value is the one the three layers would have written: same accumulators, same epilogue code.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -612,12 +613,19 @@ static hipError_t block_counters(int words, unsigned** out) {
 
 template <bool NN, int E3, int SL, int NI, int CGE, int WV>
 static hipError_t launch_block(const BlockArgs& a, const dim3& grid, size_t lds, hipStream_t stream) {
-    static bool raised = false;  // more than the default 64 KB of dynamic LDS has to be asked for, once per kernel
-    if (lds > 64 * 1024 && !raised) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<NN, E3, SL, NI, CGE, WV>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    // more than the default 64 KB of dynamic LDS has to be asked for, once per kernel and device
+    static std::atomic<bool> raised[64] = {};
+    if (lds > 64 * 1024) {
+        int dev = -1;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
-        raised = true;
+        if (dev < 0 || dev >= 64) return hipErrorInvalidValue;
+        if (!raised[dev].load(std::memory_order_acquire)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<NN, E3, SL, NI, CGE, WV>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+            raised[dev].store(true, std::memory_order_release);
+        }
     }
     hipLaunchKernelGGL((conv_block_kernel<NN, E3, SL, NI, CGE, WV>), grid, dim3(64 * WV), lds, stream, a);
     return hipGetLastError();

@@ -28,7 +28,7 @@ def quantize_weights(wf):
     return wq, ws
 
 
-def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1):
+def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1, out_round=capi.ROUND_SSE):
     """The three layers as a MobileNetV2 block has them: expand and depthwise with `act` and int8 results, a linear
     project layer with an fp32 or int8 result."""
     layers = []
@@ -41,7 +41,7 @@ def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1):
         si = (np.float32(1.0) / (in_scale * ws)).astype(np.float32)
         conv = hip.conv(wq=wq, scale_in=si, bias=bias, in_scale=float(in_scale), out_scale=[out_scale] if i8 else None,
                         stride=(s, s), pad=(pad, pad), groups=groups, act=a,
-                        out_kind=capi.OUT_I8 if i8 else capi.OUT_F32, out_round=capi.ROUND_SSE)
+                        out_kind=capi.OUT_I8 if i8 else capi.OUT_F32, out_round=out_round)
         layers.append(dict(conv=conv, wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale), k=k,
                            stride=s, pad=pad, groups=groups, act=a, int8_out=i8))
         in_scale = out_scale
@@ -121,6 +121,72 @@ def test_block_equals_the_three_layers(hip, oracle, cin, ce, cout, N, H, W, act,
             assert (capi.unpack_np(got_q.cpu().numpy(), 8, (N, cout, H, W)) == q).all()
     else:
         assert (out == cur).all()
+    for l in layers:
+        l["conv"].close()
+
+
+@pytest.mark.parametrize("act,f32_out", [(3, True), (0, False)])
+def test_block_with_the_exact_rounding_mode(hip, act, f32_out):
+    """Layers that round with 0.49999997 (the reference's unpacked route) keep that constant inside the single launch,
+    in both requantizations, the int8 result and the quantized twin."""
+    rng = np.random.default_rng(11 + act)
+    layers = make_block(hip, rng, 64, 384, 64, act, f32_out, out_round=capi.ROUND_EXACT)
+    e, d, p = (l["conv"] for l in layers)
+    N, H, W = 3, 14, 14
+    assert hip.conv_block_launches(e, d, p, N, H, W) == 1
+    x = rng.integers(-127, 128, (N, 64, H, W)).astype(np.int8)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    q_scale = 17.25 if f32_out else None
+    got, got_q = hip.conv_block(e, d, p, xd, N, H, W, q_scale=q_scale, q_round_mode=capi.ROUND_EXACT)
+    t = e.forward(xd, capi.I8_P8, N, H, W, capi.I8_P8)
+    t = d.forward(t, capi.I8_P8, N, H, W, capi.I8_P8)
+    if f32_out:
+        want, want_q = p.forward_twin(t, capi.I8_P8, N, H, W, q_scale, capi.ROUND_EXACT)
+    else:
+        want, want_q = p.forward(t, capi.I8_P8, N, H, W), None
+    hip.torch.cuda.synchronize()
+    assert hip.torch.equal(got, want)
+    if f32_out:
+        assert hip.torch.equal(got_q, want_q)
+    for l in layers:
+        l["conv"].close()
+
+
+def test_block_replayed_from_a_captured_graph(hip):
+    """A launch whose bands are dealt to several workgroups, captured into a graph and replayed on new inputs, with eager
+    launches in between: the arrival counters it was captured with are left at zero by every launch, so each replay
+    equals the three layers one by one."""
+    torch = hip.torch
+    rng = np.random.default_rng(23)
+    N, H, W = 5, 7, 7
+    layers = make_block(hip, rng, 160, 960, 160, 3, True)
+    e, d, p = (l["conv"] for l in layers)
+    e.set_block_plan(0, 0, 4)
+    assert hip.conv_block_launches(e, d, p, N, H, W) == 1
+    xs = [hip.to_device(capi.pack_np(rng.integers(-127, 128, (N, 160, H, W)).astype(np.int8), 8)) for _ in range(3)]
+    res = hip.to_device(capi.pack_np(rng.normal(0, 1, (N, 160, H, W)).astype(np.float32), 4))
+    wants = [tuple(t.clone() for t in one_by_one(hip, layers, x, N, H, W, res, 21.5)) for x in xs]
+    x_static = xs[0].clone()
+    out = hip.empty(N * 160 * H * W, np.float32)
+    q = hip.empty(N * 160 * H * W, np.int8)
+    ws = hip.empty(hip.lib.otter_hip_conv_block_workspace_bytes(e.h, d.h, p.h, N, H, W), np.int8)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):  # (the first launch of a kernel raises its LDS limit: not inside a capture)
+        hip.conv_block(e, d, p, x_static, N, H, W, residual=res, q_scale=21.5, out=out, q=q, workspace=ws)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        hip.conv_block(e, d, p, x_static, N, H, W, residual=res, q_scale=21.5, out=out, q=q, workspace=ws)
+    for rep in range(2):
+        for x, (want, want_q) in zip(xs, wants):
+            x_static.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want.view(-1)) and torch.equal(q, want_q.view(-1))
+            with torch.cuda.stream(side):
+                eager, eager_q = hip.conv_block(e, d, p, x, N, H, W, residual=res, q_scale=21.5)
+            side.synchronize()
+            assert torch.equal(eager, want) and torch.equal(eager_q, want_q)
     for l in layers:
         l["conv"].close()
 

@@ -8,7 +8,8 @@ Prints ONE JSON line. The headline workload is the fourth benchmark configuratio
 56x56, batch 64, fused requantize+ReLU. One step = the four layers back to back on device-resident int8
 activations. The other single-GPU configurations (depthwise c1 at stride 1 and 2 with its HBM roofline, the
 1x1 GEMM c2 and its int8-output variant, the single-image c0 and the same layer at batch 64) are measured the same
-way and reported under "also". A bandwidth-bound kernel's roofline figure comes from a loop that rotates over enough
+way and reported under "also", followed by a plain device-to-device copy of 256 MiB ("copy": what a copy reaches on
+the box the line was measured on). A bandwidth-bound kernel's roofline figure comes from a loop that rotates over enough
 buffer sets to exceed the 256 MB last-level cache; the figure of the loop over one (cache-resident) set is reported
 beside it as "roofline_resident".
 
@@ -418,7 +419,7 @@ def build_copy(hip, capi, rng):
     src = torch.zeros(n, dtype=torch.int8, device=hip.device)
     dst = torch.empty_like(src)
     return dict(name="copy", step=lambda: dst.copy_(src), ops=0.0, launches=1, bytes=2 * n, dom_ops=0.0, dom_bytes=2 * n,
-                bound="hbm", workload="device-to-device copy of 256 MiB (counter calibration)", dom_kernel="copy",
+                bound="hbm", workload="device-to-device copy of 256 MiB (counter calibration; what a plain copy reaches on this box)", dom_kernel="copy",
                 dom_fn=None, x=None, params=[], shape=(n,))
 
 
@@ -818,7 +819,7 @@ def main():
             line["cpu_baseline"] = {"error": str(e)[:200]}
     if not a.no_also:
         also = []
-        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det", "blk14") + tuple(LAYER_SHAPES):
+        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det", "blk14") + tuple(LAYER_SHAPES) + ("copy",):
             if name == a.workload or name not in builders:
                 continue
             w2 = builders[name](np.random.default_rng(0))

@@ -529,6 +529,10 @@ def test_grouped_and_odd_depthwise_routes(hip, oracle, C, K, k, s, p, g, N, H, W
     (4, 40, 1, 1, 2, 12, 17, True, 1, True),     # int8 planar input, 2.5 tiles
     (5, 64, 2, 0, 1, 15, 16, True, 0, False),    # the widest reduction (45 of 64 bytes), 4 tiles
     (3, 8, 1, 1, 5, 8, 8, False, 1, False),      # half a tile
+    (3, 16, 2, 1, 1, 10, 420, False, 1, True),   # a wide image: the strip's rows are loaded in two rounds of 16-byte loads
+    (3, 16, 1, 1, 2, 9, 16, True, 0, True),      # int8 planar rows of whole 4-byte units, signed result
+    (2, 8, 2, 0, 1, 11, 23, False, 3, True),     # two channels, no padding, odd width: scalar loads, clip at six
+    (4, 32, 2, 1, 2, 3, 4, True, 2, True),       # fewer output rows than a strip, one 4-pixel unit per row
 ])
 def test_few_channel_3x3_stem_kernel(hip, oracle, C, K, s, p, N, H, W, in_i8, act, int8_out):
     """3x3 on a blob with at most 5 channels goes straight from the unpacked blob (quantized on the way) to the

@@ -50,9 +50,8 @@ void stem_pack_weights(const int8_t* w, int K, int C, int8_t* dst) {
         }
 }
 
-// CT: the channel count when known at compile time (3: an RGB image), 0: g.C at run time (up to STEM_MAX_C, absent
-// channels loaded from a clamped address and dropped)
-template <int MT, bool F32_OUT, bool IN_F32, int CT>
+// (absent channels are loaded from a clamped address and dropped)
+template <int MT, bool F32_OUT, bool IN_F32>
 __global__ void __launch_bounds__(256) conv_stem3x3_kernel(const void* __restrict__ x_, const int8_t* __restrict__ wpk,
                                                            void* __restrict__ out, ConvGeom g, Epilogue ep,
                                                            const float* __restrict__ in_scale, int in_round,
@@ -91,8 +90,8 @@ __global__ void __launch_bounds__(256) conv_stem3x3_kernel(const void* __restric
     const int OHW = g.OH * g.OW;
     const int oy_end = min((strip + 1) * STEM_ROWS_PER_WAVE, g.OH);
 
-    constexpr int NC = CT ? CT : STEM_MAX_C;
-    const int C = CT ? CT : g.C;
+    constexpr int NC = STEM_MAX_C;
+    const int C = g.C;
     const unsigned plane_u = (unsigned)plane;
     for (int oy = strip * STEM_ROWS_PER_WAVE; oy < oy_end; ++oy) {
         // ---- this lane's 16 reduction bytes: kernel row kg, byte 3*c + v. Every lane loads all of its 3*NC values
@@ -453,7 +452,7 @@ hipError_t run_conv_stem(const void* x, bool in_f32, const int8_t* wpk, void* ou
     const dim3 grid((unsigned)((total + 3) / 4)), block(256);
     const bool f32_out = ep.out_kind == OTTER_HIP_OUT_F32;
 #define OHIP_STEM(MT_, FO_, FI_)                                                                                   \
-    hipLaunchKernelGGL((conv_stem3x3_kernel<MT_, FO_, FI_, 0>), grid, block, 0, stream, x, wpk, out, g, ep, in_scale, \
+    hipLaunchKernelGGL((conv_stem3x3_kernel<MT_, FO_, FI_>), grid, block, 0, stream, x, wpk, out, g, ep, in_scale,    \
                        in_round, col_groups, strips, (int)total)
 #define OHIP_STEM_IO(MT_)                                  \
     do {                                                   \

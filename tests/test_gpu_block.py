@@ -221,3 +221,37 @@ def test_block_falls_back_to_three_launches(hip):
     assert hip.torch.equal(got, want) and hip.torch.equal(got_q, want_q)
     for l in layers:
         l["conv"].close()
+
+
+def test_block_random_shapes(hip):
+    """Seeded random blocks (channel counts, image sizes, activations, result kinds, plans): wherever the single launch
+    takes the shape it equals the three layers one by one, bit for bit."""
+    rng = np.random.default_rng(2024)
+    taken = 0
+    for case in range(40):
+        cin = 8 * int(rng.integers(1, 25))
+        ce = 8 * int(rng.integers(1, min(6 * cin // 8, 144) + 1))
+        cout = 8 * int(rng.integers(1, 21))
+        N, H, W = int(rng.integers(1, 4)), int(rng.integers(1, 21)), int(rng.integers(1, 31))
+        act = int(rng.choice([0, 1, 3]))
+        f32_out = bool(rng.integers(0, 2))
+        with_res = f32_out and cin == cout and bool(rng.integers(0, 2))
+        with_twin = f32_out and bool(rng.integers(0, 2))
+        layers = make_block(hip, rng, cin, ce, cout, act, f32_out)
+        e, d, p = (l["conv"] for l in layers)
+        if rng.integers(0, 2):
+            e.set_block_plan(int(rng.integers(0, H + 1)), int(rng.choice([0, 64, 128])), int(rng.integers(0, 5)))
+        if hip.conv_block_launches(e, d, p, N, H, W) == 1:
+            taken += 1
+            xd = hip.to_device(capi.pack_np(rng.integers(-127, 128, (N, cin, H, W)).astype(np.int8), 8))
+            resd = hip.to_device(capi.pack_np(rng.normal(0, 1, (N, cout, H, W)).astype(np.float32), 4)) if with_res else None
+            q_scale = 19.0 if with_twin else None
+            got, got_q = hip.conv_block(e, d, p, xd, N, H, W, residual=resd, q_scale=q_scale)
+            want, want_q = one_by_one(hip, layers, xd, N, H, W, resd, q_scale)
+            hip.torch.cuda.synchronize()
+            assert hip.torch.equal(got, want), (case, cin, ce, cout, N, H, W, act, f32_out)
+            if with_twin:
+                assert hip.torch.equal(got_q, want_q), (case, cin, ce, cout, N, H, W)
+        for l in layers:
+            l["conv"].close()
+    assert taken >= 20

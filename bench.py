@@ -236,7 +236,9 @@ def build_c2(hip, capi, rng, int8_out=False):
                 dom_bytes=dom_bytes, bound="hbm",
                 workload="int8 1x1 conv 256->512 @28x28 batch 32 (GEMM 512x25088x256), fp32 in -> quantize -> conv + "
                          "bias + " + tail,
-                dom_kernel="conv 1x1 256->512 (MFMA implicit GEMM, %s out)" % ("int8" if int8_out else "fp32"),
+                dom_kernel="conv 1x1 256->512 (MFMA %s, %s out)" % (
+                    "streamed 1x1" if conv.kernel_kind(capi.I8_P8, N, H, W, out_layout) == 5 else "implicit GEMM",
+                    "int8" if int8_out else "fp32"),
                 dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, out_layout, out=out),
                 x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
                 shape=(N, C, H, W), int8_out=int8_out)

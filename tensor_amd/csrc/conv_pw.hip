@@ -1,11 +1,12 @@
-// Pointwise (1x1, stride 1) int8 -> int8 convolution over at most 64 input channels, as a streaming kernel.
+// Pointwise (1x1, stride 1) int8 -> int8 convolution over at most 256 input channels, as a streaming kernel.
 //
-// With one MFMA reduction step per output the layer is an elementwise pass: read C bytes per pixel, write K bytes,
-// and the time goes into the requantization of the K results, not into the product. The implicit-GEMM kernel pays
+// With one to four MFMA reduction steps per output the layer is an elementwise pass: read C bytes per pixel, write K
+// bytes, and the time goes into the requantization of the K results, not into the product. The implicit-GEMM kernel pays
 // for its generality here (output rows padded to its row tile, the pixels' round trip through LDS and two barriers
 // per workgroup for one MFMA step, a workgroup prologue per tile). This kernel has no tile grid and one barrier:
 //   - a wave owns G groups of 16 consecutive pixels of one image and loads their bytes straight into the MFMA's
-//     B operand (lane (q, p): channels 16q..16q+15 of pixel p = two 8-byte elements of the Byte8 blob);
+//     B operands (reduction step cg, lane (q, p): channels 64cg+16q..+15 of pixel p = two 8-byte elements of the
+//     Byte8 blob);
 //   - it walks the output channels in pairs of 16-row tiles (32 channels); the A operands (the implicit-GEMM weight
 //     packing as it lies in memory, 16 bytes per lane and tile) and the per-channel constants of the workgroup's
 //     pairs sit in LDS, copied there once per workgroup, and are read once per pair for all G groups;
@@ -26,10 +27,11 @@ typedef unsigned v2u_store __attribute__((__vector_size__(2 * sizeof(unsigned)))
 
 constexpr unsigned PW_OOB = 0x80000000u;  // past any buffer: the load returns zero, the store is dropped
 
-// LDS image of one pair of row tiles: the two A operands in lane order, then scale_in, bias, scale_out (32 floats
-// each) and the clamps (16 dwords) of the pair's 32 channels
-constexpr int PW_PAIR_V4 = 128 + 8 + 8 + 8 + 4;  // 16-byte units
-constexpr int PW_MAX_PAIRS = 24;
+// LDS image of one pair of row tiles: per reduction step the two A operands in lane order, then scale_in, bias,
+// scale_out (32 floats each) and the clamps (16 dwords) of the pair's 32 channels
+constexpr int pw_pair_v4(int cg) { return 128 * cg + 8 + 8 + 8 + 4; }  // 16-byte units
+constexpr int pw_max_pairs(int cg) { return (64 * 1024) / (pw_pair_v4(cg) * 16); }  // a slice's image stays under 64 KB
+constexpr int PW_MAX_CG = 4;
 
 // grid: x = chunks of 4 waves x G groups x 16 pixels of an image, y = image, z = slice of the channel pairs
 // qh (EPI_I8_P8_NONNEG): the upper clamps of the rounded results, one 16-bit value per padded channel
@@ -37,11 +39,13 @@ constexpr int PW_MAX_PAIRS = 24;
 // The four waves of a workgroup share one copy of their slice's weights and constants in LDS: read from there a
 // lane group's constants are one broadcast each, where 64 lanes loading them from memory keep the texture
 // addresser busy for longer than the requantization of two pixel groups takes.
-template <int EPI, int G>
+// CG: reduction steps (64 input channels each); mt: 16-row tiles of the packed weights per reduction step
+template <int EPI, int G, int CG>
 __global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                              int8_t* __restrict__ out, Epilogue ep,
                                                              const unsigned* __restrict__ qh, int C8, int K, int HW,
-                                                             int pairs_per_slice) {
+                                                             int pairs_per_slice, int mt) {
+    constexpr int PW_PAIR_V4 = pw_pair_v4(CG);
     extern __shared__ v4i pw_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q = lane >> 4, p = lane & 15;
@@ -54,17 +58,20 @@ __global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __res
     const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(out + (size_t)n * out_img, 0, (int)out_img, 0x00020000);
 
     // B operands of the G groups (all out of range for a wave past the image: zeros, and nothing is stored)
-    v4i b[G];
-    const bool plane0 = 2 * q < C8, plane1 = 2 * q + 1 < C8;
+    v4i b[G][CG];
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) {
         const int pix = pix0 + 16 * gi + p;
-        const unsigned o0 = ((unsigned)(2 * q) * HW + pix) * 8u;
         const bool in = pix < HW;
-        const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && plane0 ? o0 : PW_OOB), 0, 0));
-        const v2i hi = __builtin_bit_cast(
-            v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && plane1 ? o0 + (unsigned)HW * 8u : PW_OOB), 0, 0));
-        b[gi] = v4i{lo[0], lo[1], hi[0], hi[1]};
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {
+            const int oct = 8 * cg + 2 * q;
+            const unsigned o0 = ((unsigned)oct * HW + pix) * 8u;
+            const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && oct < C8 ? o0 : PW_OOB), 0, 0));
+            const v2i hi = __builtin_bit_cast(
+                v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(in && oct + 1 < C8 ? o0 + (unsigned)HW * 8u : PW_OOB), 0, 0));
+            b[gi][cg] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        }
     }
 
     const int pairs = (K + 31) / 32;
@@ -80,12 +87,13 @@ __global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __res
         const int total = (pr1 - pr0) * PW_PAIR_V4;
         for (int i = threadIdx.x; i < total; i += 256) {
             const int pr = pr0 + i / PW_PAIR_V4, r = i % PW_PAIR_V4;
+            constexpr int W4 = 128 * CG;
             v4i v;
-            if (r < 128) v = wg[pr * 128 + r];
-            else if (r < 136) v = sg[pr * 8 + r - 128];
-            else if (r < 144) v = bg[pr * 8 + r - 136];
-            else if (r < 152) v = og[pr * 8 + r - 144];
-            else if constexpr (EPI == EPI_I8_P8_NONNEG) v = cg[pr * 4 + r - 152];
+            if (r < W4) v = wg[((size_t)(r / 128) * mt + 2 * pr) * 64 + r % 128];  // (step, the pair's two tiles, lane)
+            else if (r < W4 + 8) v = sg[pr * 8 + r - W4];
+            else if (r < W4 + 16) v = bg[pr * 8 + r - W4 - 8];
+            else if (r < W4 + 24) v = og[pr * 8 + r - W4 - 16];
+            else if constexpr (EPI == EPI_I8_P8_NONNEG) v = cg[pr * 4 + r - W4 - 24];
             else v = v4i{0, 0, 0, 0};
             pw_lds[i] = v;
         }
@@ -95,11 +103,14 @@ __global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __res
 
     for (int pr = pr0; pr < pr1; ++pr) {
         const v4i* l = pw_lds + (pr - pr0) * PW_PAIR_V4;
-        const v4i a0 = l[lane], a1 = l[64 + lane];
+        v4i a0[CG], a1[CG];
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) a0[cg] = l[128 * cg + lane], a1[cg] = l[128 * cg + 64 + lane];
         Epi8 prm;
         {
-            const v4i s0 = l[128 + 2 * q], s1 = l[129 + 2 * q], b0 = l[136 + 2 * q], b1 = l[137 + 2 * q];
-            const v4i o0 = l[144 + 2 * q], o1 = l[145 + 2 * q], c = l[152 + q];
+            constexpr int W4 = 128 * CG;
+            const v4i s0 = l[W4 + 2 * q], s1 = l[W4 + 1 + 2 * q], b0 = l[W4 + 8 + 2 * q], b1 = l[W4 + 9 + 2 * q];
+            const v4i o0 = l[W4 + 16 + 2 * q], o1 = l[W4 + 17 + 2 * q], c = l[W4 + 24 + q];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
@@ -113,8 +124,13 @@ __global__ void __launch_bounds__(256) conv_pw_stream_kernel(const int8_t* __res
         const unsigned orow = (unsigned)(ch0 >> 3) * HW;
 #pragma unroll
         for (int gi = 0; gi < G; ++gi) {
-            const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b[gi], v4i{0, 0, 0, 0}, 0, 0, 0);
-            const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b[gi], v4i{0, 0, 0, 0}, 0, 0, 0);
+            v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b[gi][0], v4i{0, 0, 0, 0}, 0, 0, 0);
+            v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b[gi][0], v4i{0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+            for (int cg = 1; cg < CG; ++cg) {
+                c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[cg], b[gi][cg], c0, 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[cg], b[gi][cg], c1, 0, 0, 0);
+            }
             const int a8[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
             const v2i r = epi8_quant_i8p8<EPI == EPI_I8_P8_NONNEG>(ep, prm, a8);
             const int pix = pix0 + 16 * gi + p;
@@ -138,8 +154,13 @@ void conv_pw_stream_clamps(float act_hi, float round_half, const float* scale_ou
 
 bool conv_pw_stream_applicable(const ConvGeom& g, const Epilogue& ep) {
     if (g.groups != 1 || g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph != 0 || g.pw != 0) return false;
-    if (g.Cs || g.Ks || g.C % 8 || g.C > 64 || g.K % 8 || g.N < 1 || g.N > 65535) return false;
+    if (g.Cs || g.Ks || g.C % 8 || g.C > 64 * PW_MAX_CG || g.K % 8 || g.N < 1 || g.N > 65535) return false;
     if ((size_t)std::max(g.C, g.K) * g.H * g.W >= (1ull << 31)) return false;  // 32-bit offsets inside an image
+    // Several reduction steps: a workgroup copies 2 KB of weights per step and channel pair into LDS for its 128 or 256
+    // pixels, which pays from about 12 000 pixels on. Measured against the implicit-GEMM kernel (kernel trace, us):
+    // 256 -> 512 @28x28 b32 12.8 / 14.0, 128 -> 128 @28x28 b64 7.0 / 8.4, 256 -> 64 @56x56 b16 6.1 / 7.3, 96 -> 576
+    // @14x14 b64 7.6 / 8.0, 88 -> 88 @52x52 b16 6.8 / 7.0; 176 -> 176 @26x26 b16 (10 816 pixels) 5.9 / 5.0.
+    if (g.C > 64 && (long)g.N * g.H * g.W < 12000) return false;
     const int epi = pick_epilogue(ep, g.K);
     return epi == EPI_I8_P8 || epi == EPI_I8_P8_NONNEG;
 }
@@ -155,19 +176,19 @@ void conv_pw_stream_plan(const ConvGeom& g, int* groups, int* slices) {
     int s = 1;
     const int smax = std::max(1, pairs / 2);
     while (s < smax && waves(G, s) < 8192) ++s;
-    while ((pairs + s - 1) / s > PW_MAX_PAIRS) ++s;  // a slice's LDS image stays under 64 KB
+    while ((pairs + s - 1) / s > pw_max_pairs((g.C + 63) / 64)) ++s;  // a slice's LDS image stays under 64 KB
     const int per = (pairs + s - 1) / s;
     *groups = G, *slices = (pairs + per - 1) / per;
 }
 
-template <int EPI, int G>
+template <int EPI, int G, int CG>
 static hipError_t launch_pw(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
                             const unsigned* qh, int slices, hipStream_t stream) {
     const int HW = g.H * g.W, pairs = (g.K + 31) / 32;
     const int per = (pairs + slices - 1) / slices;
     const dim3 grid((HW + 64 * G - 1) / (64 * G), g.N, (pairs + per - 1) / per);
-    hipLaunchKernelGGL((conv_pw_stream_kernel<EPI, G>), grid, dim3(256), (size_t)per * PW_PAIR_V4 * 16, stream, x, wpk,
-                       (int8_t*)out, ep, qh, g.C / 8, g.K, HW, per);
+    hipLaunchKernelGGL((conv_pw_stream_kernel<EPI, G, CG>), grid, dim3(256), (size_t)per * pw_pair_v4(CG) * 16, stream, x, wpk,
+                       (int8_t*)out, ep, qh, g.C / 8, g.K, HW, per, igemm_padded_rows(g.K) / 16);
     return hipGetLastError();
 }
 
@@ -180,17 +201,22 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
     conv_pw_stream_plan(g, &G, &s);
     if (force_groups) G = force_groups;
     if (force_slices) s = force_slices;
-    const int pairs = (g.K + 31) / 32;
+    const int pairs = (g.K + 31) / 32, cgs = (g.C + 63) / 64;
     if ((G != 2 && G != 4) || s < 1 || s > pairs) return hipErrorInvalidValue;
-    while ((pairs + s - 1) / s > PW_MAX_PAIRS) ++s;  // a slice's LDS image stays under 64 KB
+    if (cgs > 2) G = 2;  // (four groups of three or four reduction steps are more operand registers than pay)
+    while ((pairs + s - 1) / s > pw_max_pairs(cgs)) ++s;  // a slice's LDS image stays under 64 KB
     const bool nonneg = pick_epilogue(ep, g.K) == EPI_I8_P8_NONNEG;
     if (nonneg && !qh) return hipErrorInvalidValue;
-#define OHIP_PW(G_) \
-    if (G == G_) \
-        return nonneg ? launch_pw<EPI_I8_P8_NONNEG, G_>(x, wpk, out, g, ep, qh, s, stream) \
-                      : launch_pw<EPI_I8_P8, G_>(x, wpk, out, g, ep, qh, s, stream);
-    OHIP_PW(4)
-    OHIP_PW(2)
+#define OHIP_PW(G_, CG_) \
+    if (G == G_ && cgs == CG_) \
+        return nonneg ? launch_pw<EPI_I8_P8_NONNEG, G_, CG_>(x, wpk, out, g, ep, qh, s, stream) \
+                      : launch_pw<EPI_I8_P8, G_, CG_>(x, wpk, out, g, ep, qh, s, stream);
+    OHIP_PW(4, 1)
+    OHIP_PW(2, 1)
+    OHIP_PW(4, 2)
+    OHIP_PW(2, 2)
+    OHIP_PW(2, 3)
+    OHIP_PW(2, 4)
 #undef OHIP_PW
     return hipErrorInvalidValue;
 }

@@ -281,7 +281,8 @@ def build_c0(hip, capi, rng, batch=1):
     return dict(name="c0", step=step, ops=ops, launches=2, dom_ops=ops,
                 dom_bytes=N * C * H * W + K * C * 9 + 4 * N * K * H * W, bound="mfma",
                 workload="single int8 3x3 conv 64->64 s1 p1, 1x64x56x56 fp32 in -> fp32 out (latency-bound)",
-                dom_kernel="conv 3x3 64->64 (MFMA implicit GEMM, fp32 out)",
+                dom_kernel="conv 3x3 64->64 (MFMA, %s, fp32 out)" % (
+                    "LDS halo" if conv.kernel_kind(capi.I8_P8, N, H, W, capi.F32_P4) == 3 else "implicit GEMM"),
                 dom_fn=None, x=x, params=[dict(wq=wq, ws=ws, bias=None, in_scale=float(in_scale))],
                 shape=(N, C, H, W))
 

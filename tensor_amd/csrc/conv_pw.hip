@@ -1,6 +1,7 @@
-// Pointwise (1x1, stride 1) int8 -> int8 convolution over at most 256 input channels, as a streaming kernel.
+// Pointwise (1x1, stride 1) int8 -> int8 convolution over at most 64 input channels, or 200 .. 256 on large blobs, as a
+// streaming kernel.
 //
-// With one to four MFMA reduction steps per output the layer is an elementwise pass: read C bytes per pixel, write K
+// With one (or, on large blobs, four) MFMA reduction steps per output the layer is an elementwise pass: read C bytes per pixel, write K
 // bytes, and the time goes into the requantization of the K results, not into the product. The implicit-GEMM kernel pays
 // for its generality here (output rows padded to its row tile, the pixels' round trip through LDS and two barriers
 // per workgroup for one MFMA step, a workgroup prologue per tile). This kernel has no tile grid and one barrier:
@@ -156,11 +157,13 @@ bool conv_pw_stream_applicable(const ConvGeom& g, const Epilogue& ep) {
     if (g.groups != 1 || g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph != 0 || g.pw != 0) return false;
     if (g.Cs || g.Ks || g.C % 8 || g.C > 64 * PW_MAX_CG || g.K % 8 || g.N < 1 || g.N > 65535) return false;
     if ((size_t)std::max(g.C, g.K) * g.H * g.W >= (1ull << 31)) return false;  // 32-bit offsets inside an image
-    // Several reduction steps: a workgroup copies 2 KB of weights per step and channel pair into LDS for its 128 or 256
-    // pixels, which pays from about 12 000 pixels on. Measured against the implicit-GEMM kernel (kernel trace, us):
-    // 256 -> 512 @28x28 b32 12.8 / 14.0, 128 -> 128 @28x28 b64 7.0 / 8.4, 256 -> 64 @56x56 b16 6.1 / 7.3, 96 -> 576
-    // @14x14 b64 7.6 / 8.0, 88 -> 88 @52x52 b16 6.8 / 7.0; 176 -> 176 @26x26 b16 (10 816 pixels) 5.9 / 5.0.
-    if (g.C > 64 && (long)g.N * g.H * g.W < 12000) return false;
+    // More than one reduction step: a workgroup copies 2 KB of weights per step and channel pair into LDS for its 128
+    // pixels, which pays on large blobs with four steps. Measured against the implicit-GEMM kernel (kernel trace of the
+    // layer alone, us): 256 -> 512 @28x28 b32 12.8 / 14.0, 256 -> 64 @56x56 b16 6.1 / 7.3. With two or three steps the
+    // kernel also ran 128 -> 128 @28x28 b64 at 7.0 / 8.4, but 176 -> 176 @26x26 b16 at 5.9 / 5.0, and the pointwise
+    // layers of the two benchmark networks that would take it (88 .. 176 channels) made their passes 0.3 - 1 % slower on
+    // the same box (cold inputs): those stay on the implicit-GEMM kernel.
+    if (g.C > 64 && (g.C <= 192 || (long)g.N * g.H * g.W < 20000)) return false;
     const int epi = pick_epilogue(ep, g.K);
     return epi == EPI_I8_P8 || epi == EPI_I8_P8_NONNEG;
 }
@@ -203,7 +206,7 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
     if (force_slices) s = force_slices;
     const int pairs = (g.K + 31) / 32, cgs = (g.C + 63) / 64;
     if ((G != 2 && G != 4) || s < 1 || s > pairs) return hipErrorInvalidValue;
-    if (cgs > 2) G = 2;  // (four groups of three or four reduction steps are more operand registers than pay)
+    if (cgs > 1) G = 2;  // (four groups of four reduction steps are more operand registers than pay)
     while ((pairs + s - 1) / s > pw_max_pairs(cgs)) ++s;  // a slice's LDS image stays under 64 KB
     const bool nonneg = pick_epilogue(ep, g.K) == EPI_I8_P8_NONNEG;
     if (nonneg && !qh) return hipErrorInvalidValue;
@@ -213,9 +216,6 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
                       : launch_pw<EPI_I8_P8, G_, CG_>(x, wpk, out, g, ep, qh, s, stream);
     OHIP_PW(4, 1)
     OHIP_PW(2, 1)
-    OHIP_PW(4, 2)
-    OHIP_PW(2, 2)
-    OHIP_PW(2, 3)
     OHIP_PW(2, 4)
 #undef OHIP_PW
     return hipErrorInvalidValue;

@@ -350,16 +350,16 @@ def test_random_shapes_against_oracle(hip, oracle, C, K, k, s, p, d, g, N, H, W)
                          ids=["auto", "g4s1", "g2s2", "g2s3", "g2s1", "g4s5"])
 def test_streamed_pointwise_kernel(hip, oracle, groups_slices):
     """The streamed 1x1 int8 -> int8 kernel (at most 256 input channels): 1 to 8 input octets (a half-used operand
-    register, a full one), two to four reduction steps (72..256 channels, the last step partly filled) on blobs of at
-    least 12 000 pixels, output channel counts that end inside a pair of row tiles (8, 24, 40, 144) and on one, pixel
+    register, a full one), four reduction steps (200..256 channels, the last step partly filled) on blobs of at least
+    20 000 pixels, output channel counts that end inside a pair of row tiles (8, 24, 40, 144) and on one, pixel
     counts that are not whole groups of 16 (and images smaller than one group), every epilogue the fast int8 path has
     (none, ReLU, clip, LeakyReLU), with and without bias, forced pixel groups per wave and channel slices. fp32
-    output, and several reduction steps over few pixels, stay on the implicit-GEMM kernel."""
+    output, 72..192 input channels, and four reduction steps over few pixels, stay on the implicit-GEMM kernel."""
     G, S = groups_slices
     rng = np.random.default_rng(100 + 8 * G + S)
     for (C, K, N, H, W) in [(16, 96, 2, 19, 23), (24, 144, 1, 28, 28), (32, 16, 3, 9, 11), (8, 8, 2, 3, 3),
                             (64, 384, 1, 14, 14), (40, 24, 2, 16, 16), (56, 40, 1, 5, 41), (32, 192, 2, 1, 70),
-                            (96, 40, 2, 80, 80), (136, 64, 1, 110, 111), (256, 24, 4, 56, 56), (200, 72, 13, 31, 31)]:
+                            (256, 24, 7, 56, 56), (200, 72, 21, 31, 31), (232, 40, 2, 100, 101)]:
         pairs = (K + 31) // 32
         tile = (-5, G | min(S, pairs) << 3) if G else None
         x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W)

@@ -780,7 +780,7 @@ static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_
     // rows of one image each, or a share of a band's expanded channels) about fill the 256 compute units once.
     // Measured at batch 64 against the three launches (kernel trace; in brackets the three launches inside a network,
     // where each starts on cold inputs): 14x14 64 -> 384 -> 64 13.2 us against 17.8, 14x14 96 -> 576 -> 96 21.8 against
-    // 23.5 (29.8), 28x28 32 -> 192 -> 32 16.8 against 21.8, 7x7 160 -> 960 -> 160 with the slices of an image dealt to
+    // 23.5 (29.8), 28x28 32 -> 192 -> 32 15.2 against 21.8, 7x7 160 -> 960 -> 160 with the slices of an image dealt to
     // four workgroups 18.5 against 20 (23.4). Not taken: 56x56 24 -> 144 -> 24 (896 workgroups of 13 us each on 256
     // compute units) 56 against 45, 7x7 160 -> 960 -> 320 (more project items per wave than registers for their
     // weights) 23.9 against 24.4.

@@ -58,7 +58,7 @@ def test_automatic_plans_of_the_tuned_shapes():
     assert (p["rb"], p["bands"], p["sl"], p["split"]) == (4, 4, 128, 1)
     # 28x28: four bands of 7 rows
     p = block_plan(lib, 32, 192, 32, 64, 28, 28)
-    assert (p["bands"], p["split"]) == (4, 1) and p["rb"] in (7, 8)
+    assert (p["rb"], p["bands"], p["sl"], p["split"]) == (7, 4, 64, 1)  # (192 channels: three slices of 64, not 128 + 64)
     # 7x7: one band per image, the eight slices of 960 channels dealt to four workgroups
     p = block_plan(lib, 160, 960, 160, 64, 7, 7)
     assert (p["rb"], p["bands"], p["sl"], p["split"]) == (7, 1, 128, 4)

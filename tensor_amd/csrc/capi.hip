@@ -781,9 +781,9 @@ static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_
     // Measured at batch 64 against the three launches (kernel trace; in brackets the three launches inside a network,
     // where each starts on cold inputs): 14x14 64 -> 384 -> 64 13.2 us against 17.8, 14x14 96 -> 576 -> 96 21.8 against
     // 23.5 (29.8), 28x28 32 -> 192 -> 32 15.2 against 21.8, 7x7 160 -> 960 -> 160 with the slices of an image dealt to
-    // four workgroups 18.5 against 20 (23.4). Not taken: 56x56 24 -> 144 -> 24 (896 workgroups of 13 us each on 256
-    // compute units) 56 against 45, 7x7 160 -> 960 -> 320 (more project items per wave than registers for their
-    // weights) 23.9 against 24.4.
+    // four workgroups 18.5 against 20 (23.4), 7x7 160 -> 960 -> 320 as two bands of 20 project tiles, each dealt to two
+    // workgroups, 20.8 against 20.3 (24.4). Not taken: 56x56 24 -> 144 -> 24 (896 workgroups of 13 us each on 256
+    // compute units) 53 against 45.
     const long wgs = (long)g[0].N * plan[1] * plan[4];
     const int items = ((g[2].K + 31) / 32) * ((plan[0] * g[0].W + 15) / 16);
     return g[0].C <= 192 && g[0].W <= 28 && wgs >= 128 && wgs <= 512 && items <= 24;

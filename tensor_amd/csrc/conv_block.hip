@@ -472,6 +472,7 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
         return *total <= kLdsMax;
     };
     int RB = 0, SL = 0, tot = 0;
+    bool fill = false;  // bands lowered for the project layer's sake: deal their slices out until the compute units have work
     if (force_rb > 0 || force_sl > 0) {
         RB = force_rb > 0 ? std::min(force_rb, H) : std::min(H, std::max(rpi, 4));
         SL = force_sl == 64 || force_sl == 128 ? force_sl : 64;
@@ -497,13 +498,26 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
         // are bands of 7, not of 8: one pixel group less in every phase, 17.5 -> 16.4 us)
         const int nb = (H + RB - 1) / RB;
         RB = (H + nb - 1) / nb;
+        // More than 24 (channel pair, pixel group) tiles of the project layer per band take the kernel variant with six
+        // of them per wave, which is slow (7x7 160 -> 960 -> 320 b64: 28 us as one band of 40 tiles dealt to four
+        // workgroups, 20.8 us as two bands of 20 dealt to two each): lower bands where that brings the count to 24.
+        if (npairsP * ((RB * W + 15) / 16) > 24) {
+            for (int rb = RB - 1; rb >= 1; --rb) {
+                const int nb2 = (H + rb - 1) / rb, rbt = (H + nb2 - 1) / nb2;
+                int t2 = 0;
+                if (npairsP * ((rbt * W + 15) / 16) <= 24 && fits(rbt, SL, &t2)) {
+                    RB = rbt, fill = true;
+                    break;
+                }
+            }
+        }
         fits(RB, SL, &tot);
     }
     plan[0] = RB, plan[1] = (H + RB - 1) / RB, plan[2] = SL, plan[3] = tot;
     // Fewer bands than half the compute units: the slices of a band are dealt to several workgroups
     const int slices = (Ce + SL - 1) / SL;
     const long wgs1 = (long)ge.N * plan[1];
-    int split = force_split > 0 ? force_split : (wgs1 < 128 ? (int)std::min<long>(slices, 256 / wgs1) : 1);
+    int split = force_split > 0 ? force_split : (wgs1 < 128 || (fill && wgs1 < 256) ? (int)std::min<long>(slices, 256 / wgs1) : 1);
     split = std::max(1, std::min(split, slices));
     const int spp = (slices + split - 1) / split;
     split = (slices + spp - 1) / spp;  // no workgroup without a slice

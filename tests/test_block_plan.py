@@ -62,6 +62,9 @@ def test_automatic_plans_of_the_tuned_shapes():
     # 7x7: one band per image, the eight slices of 960 channels dealt to four workgroups
     p = block_plan(lib, 160, 960, 160, 64, 7, 7)
     assert (p["rb"], p["bands"], p["sl"], p["split"]) == (7, 1, 128, 4)
+    # 7x7 with 320 output channels: one band would hold 40 project tiles; two bands of 20, each dealt to two workgroups
+    p = block_plan(lib, 160, 960, 320, 64, 7, 7)
+    assert (p["rb"], p["bands"], p["sl"], p["split"]) == (4, 2, 128, 2)
     # a small batch: the slices split as far as they go
     p = block_plan(lib, 64, 384, 64, 4, 14, 14)
     assert p["split"] == 3

@@ -195,7 +195,7 @@ def test_default_policy_takes_the_measured_shapes_only(hip):
     hip.conv_block_set_always(0)
     rng = np.random.default_rng(3)
     for (cin, ce, cout, n, hw, want) in [(64, 384, 64, 64, 14, 1), (32, 192, 32, 64, 28, 1), (24, 144, 24, 64, 56, 3),
-                                          (160, 960, 160, 64, 7, 1), (160, 960, 320, 64, 7, 3), (96, 576, 96, 64, 14, 1), (64, 384, 64, 4, 14, 3),
+                                          (160, 960, 160, 64, 7, 1), (160, 960, 320, 64, 7, 1), (96, 576, 96, 64, 14, 1), (64, 384, 64, 4, 14, 3),
                                           (64, 384, 64, 16, 14, 1)]:
         layers = make_block(hip, rng, cin, ce, cout, 3, True)
         e, d, p = (l["conv"] for l in layers)

@@ -517,7 +517,10 @@ bool conv_block_plan(const ConvGeom& ge, const ConvGeom& gp, int force_rb, int f
     // Fewer bands than half the compute units: the slices of a band are dealt to several workgroups
     const int slices = (Ce + SL - 1) / SL;
     const long wgs1 = (long)ge.N * plan[1];
-    int split = force_split > 0 ? force_split : (wgs1 < 128 || (fill && wgs1 < 256) ? (int)std::min<long>(slices, 256 / wgs1) : 1);
+    int split = 1;
+    if (force_split > 0) split = force_split;
+    else if (wgs1 < 128) split = (int)std::min<long>(slices, 256 / wgs1);
+    else if (fill && wgs1 < 256) split = (int)std::min<long>(slices, (256 + wgs1 - 1) / wgs1);  // (at least two per band)
     split = std::max(1, std::min(split, slices));
     const int spp = (slices + split - 1) / split;
     split = (slices + spp - 1) / spp;  // no workgroup without a slice

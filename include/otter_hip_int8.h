@@ -180,15 +180,22 @@ int otter_hip_conv_forward_residual(const otter_hip_conv_t* handle, const void* 
  * starts as soon as the tiles of the previous layer it reads are done; otherwise as n launches. The single launch
  * waits on flags between workgroups; every wait is bounded, and otter_hip_conv_chain_status reports (after
  * synchronizing the device) whether one ever gave up, in which case the outputs of the chain calls since the last
- * status call are not valid. The flags live in static device memory, one set per stream for the first four streams
- * that call this on a GPU (calls on different streams may overlap); further streams run their chains as n launches.
- * Like every entry point here it allocates nothing, and after one eager call on a stream it may be captured into a
- * HIP graph on that stream and replayed (a launch takes its sequence number from device memory, not from the kernel
- * arguments). */
+ * status call are not valid. The flags live in static device memory, four sets per GPU. A set belongs to the stream
+ * that launched on it last (calls on different streams may overlap); a stream without one takes a free set or the
+ * least recently used set whose last launch has completed, and only when all four are busy does a call run its chain
+ * as n launches (otter_hip_conv_chain_last_launches tells). Like every entry point here it allocates nothing, and
+ * after one eager call on a stream it may be captured into a HIP graph on that stream and replayed (a launch takes
+ * its sequence number from device memory, not from the kernel arguments); the set a captured call was given stays
+ * with the capturing stream for the life of the process, so do not replay such a graph on another stream while that
+ * stream runs chains of its own. */
 size_t otter_hip_conv_chain_workspace_bytes(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);
 int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_layers, const void* in, int n, int in_h,
                                  int in_w, void* out, void* workspace, size_t workspace_bytes, void* stream);
 int otter_hip_conv_chain_status(int* gave_up);
+/* The number of convolution launches the last otter_hip_conv_chain_forward on the calling host thread actually made
+ * (1: the single persistent launch; n_layers: layer by layer, also when every flag set was busy; 0: none yet). The
+ * reference has no counterpart (its Net runs a layer per call, Tensor/Net.cpp:413-505). */
+int otter_hip_conv_chain_last_launches(void);
 /* For tests and profiling: the number of convolution launches otter_hip_conv_chain_forward makes for this chain and
  * input (1: the single persistent launch; n_layers: layer by layer), or a negative status. */
 int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);

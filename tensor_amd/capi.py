@@ -73,6 +73,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
+           "otter_hip_conv_chain_last_launches",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
            "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always",
            "otter_hip_conv_block_plan"]
@@ -301,6 +302,10 @@ class Library:
     def conv_chain_set_min_tiles(self, tiles):
         """otter_hip_conv_chain_set_min_tiles: returns the previous threshold."""
         return self.lib.otter_hip_conv_chain_set_min_tiles(int(tiles))
+
+    def conv_chain_last_launches(self):
+        """otter_hip_conv_chain_last_launches: the launches the last chain call of this thread actually made."""
+        return self.lib.otter_hip_conv_chain_last_launches()
 
     def conv_chain_gave_up(self):
         """otter_hip_conv_chain_status: synchronizes; True if a chain launch since the last call gave up a wait."""

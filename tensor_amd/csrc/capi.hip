@@ -637,6 +637,8 @@ int otter_hip_conv_chain_set_min_tiles(int tiles) {
     return before;
 }
 
+static thread_local int t_chain_last_launches = 0;  // kernels the last otter_hip_conv_chain_forward of this thread enqueued
+
 int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w) {
     int rc = chain_check(handles, n_layers, n, in_h, in_w, "otter_hip_conv_chain_launches");
     if (rc) return rc;
@@ -692,9 +694,12 @@ int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_l
         }
         const hipError_t ce = run_conv3x3_chain(g, eps.data(), wpk.data(), act.data(), n_layers, nullptr, stream,
                                                  handles[0]->force_tm == -1 ? handles[0]->force_tn : 0);
-        if (ce == hipSuccess) return OTTER_HIP_OK;
+        if (ce == hipSuccess) {
+            t_chain_last_launches = 1;
+            return OTTER_HIP_OK;
+        }
         if (ce != hipErrorNotReady) OHIP_CHECK(ce);
-        // (every flag set of this GPU belongs to another stream: this stream takes the layers one by one)
+        // (every flag set of this GPU is busy on another stream: this stream takes the layers one by one)
     }
     // anything else: the layers one after the other, the same blobs
     for (int l = 0; l < n_layers; ++l) {
@@ -702,13 +707,15 @@ int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_l
                           stream_, nullptr, 0.f, 0);
         if (rc) return rc;
     }
+    t_chain_last_launches = n_layers;
     return OTTER_HIP_OK;
 }
 
+int otter_hip_conv_chain_last_launches(void) { return t_chain_last_launches; }
+
 int otter_hip_conv_chain_status(int* gave_up) {
     if (!gave_up) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_status: null");
-    OHIP_CHECK(hipDeviceSynchronize());
-    OHIP_CHECK(conv3x3_chain_error(gave_up));
+    OHIP_CHECK(conv3x3_chain_error(gave_up));  // (synchronizes with the device)
     return OTTER_HIP_OK;
 }
 

@@ -24,6 +24,7 @@
 //     passed s_waitcnt vmcnt(0) by then, so all of the tile's stores have been acknowledged by L2.
 //   * Each layer writes a buffer nobody has read before in this launch (the caller provides layers - 1 intermediate
 //     buffers), so a compute unit's vector L1 cannot hold a stale line of what it is about to read.
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -436,12 +437,19 @@ struct ChainDevice {
     int* flags = nullptr;
     int* ctl = nullptr;
     int xcds = 0;
-    // slot -> the stream that owns it (first come, for the life of the process)
+    // A flag set (slot) belongs to the stream that launched on it last. A stream that has none takes a free slot, or the
+    // least recently used one whose last launch has completed (its event says so): a caller that rotates through more
+    // streams than there are slots keeps the single launch as long as at most CHAIN_SLOTS of them are busy at a time.
+    // A slot handed to a stream under graph capture is baked into the graph and stays with that stream for good.
     hipStream_t stream[CHAIN_SLOTS] = {};
     bool used[CHAIN_SLOTS] = {};
+    bool pinned[CHAIN_SLOTS] = {};
+    hipEvent_t done[CHAIN_SLOTS] = {};
+    unsigned long stamp[CHAIN_SLOTS] = {};
+    unsigned long clock = 0;
 };
 ChainDevice g_chain_dev[16];
-std::mutex g_chain_mutex;
+std::mutex g_chain_mutex;  // slot table, launches and the status read-and-rewind
 
 }  // namespace
 
@@ -472,9 +480,14 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 16) return hipErrorInvalidDevice;
     ChainDevice& cd = g_chain_dev[dev];
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if ((e = hipStreamIsCapturing(stream, &cs)) != hipSuccess) return e;
+    const bool capturing = cs != hipStreamCaptureStatusNone;
+    // the launch itself is made under the lock as well: conv3x3_chain_error rewinds the queues of every slot from the
+    // host and must not meet a launch that another thread enqueues in between
+    std::lock_guard<std::mutex> lock(g_chain_mutex);
     int slot = -1;
     {
-        std::lock_guard<std::mutex> lock(g_chain_mutex);
         if (!cd.flags) {
             void *pf = nullptr, *pc = nullptr;
             if ((e = hipGetSymbolAddress(&pf, HIP_SYMBOL(g_chain_flags))) != hipSuccess) return e;
@@ -487,8 +500,25 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
         for (int i = 0; i < CHAIN_SLOTS && slot < 0; ++i)
             if (cd.used[i] && cd.stream[i] == stream) slot = i;
         for (int i = 0; i < CHAIN_SLOTS && slot < 0; ++i)
-            if (!cd.used[i]) cd.used[i] = true, cd.stream[i] = stream, slot = i;
-        if (slot < 0) return hipErrorNotReady;  // more streams than slots: the caller runs the layers one by one
+            if (!cd.used[i]) slot = i;
+        if (slot < 0) {
+            // every slot has an owner: the one that has been idle longest, if its last launch has completed
+            int lru = -1;
+            for (int i = 0; i < CHAIN_SLOTS; ++i)
+                if (!cd.pinned[i] && (lru < 0 || cd.stamp[i] < cd.stamp[lru])) lru = i;
+            for (int k = 0; k < CHAIN_SLOTS && slot < 0 && lru >= 0; ++k) {
+                const int i = (lru + k) % CHAIN_SLOTS;
+                if (cd.pinned[i] || !cd.done[i]) continue;
+                const hipError_t q = hipEventQuery(cd.done[i]);
+                if (q == hipSuccess) slot = i;
+                else if (q != hipErrorNotReady) return q;
+            }
+            if (slot < 0) return hipErrorNotReady;  // all busy: the caller runs the layers one by one
+        }
+        if (!cd.done[slot] && (e = hipEventCreateWithFlags(&cd.done[slot], hipEventDisableTiming)) != hipSuccess) return e;
+        cd.used[slot] = true, cd.stream[slot] = stream;
+        cd.pinned[slot] = cd.pinned[slot] || capturing;
+        cd.stamp[slot] = ++cd.clock;
     }
     ChainArgs ca;
     for (int l = 0; l < layers; ++l) {
@@ -509,12 +539,12 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
 #define OHIP_CHAIN_W(FN_, E_, P_, W_)                                                                                  \
     do {                                                                                                               \
         auto kern = conv3x3_chain_kernel<FN_, E_, P_, W_>;                                                             \
-        static bool attr_set = false;                                                                                  \
-        if (!attr_set) {                                                                                               \
+        static std::atomic<bool> attr_set[16] = {};                                                                    \
+        if (!attr_set[dev].load(std::memory_order_acquire)) {                                                          \
             hipError_t e2 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,        \
                                                 kChainLdsBytes + kChainPrmBytes);                                      \
             if (e2 != hipSuccess) return e2;                                                                           \
-            attr_set = true;                                                                                           \
+            attr_set[dev].store(true, std::memory_order_release);                                                      \
         }                                                                                                              \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_bytes, stream, g, eps[0], ca, igemm_padded_rows(g.K) / 16, \
                            igemm_channel_groups(g.C), r_max, tpi, act_bytes);                                          \
@@ -545,16 +575,21 @@ hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_
 #undef OHIP_CHAIN
 #undef OHIP_CHAIN_W
     if (error_word_out) *error_word_out = 0;
-    return hipGetLastError();
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    // (no event inside a capture: the slot is pinned to the stream then and never asked for its state)
+    return capturing ? hipSuccess : hipEventRecord(cd.done[slot], stream);
 }
 
 // the error word of the last chain launches on this device (1: a workgroup gave up waiting for a producer tile);
-// synchronizes with the device and clears it
+// synchronizes with the device and clears it. Launches on other host threads wait at the lock meanwhile, so the rewind
+// cannot meet a launch in flight.
 hipError_t conv3x3_chain_error(int* error_word) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     *error_word = 0;
+    std::lock_guard<std::mutex> lock(g_chain_mutex);
+    if ((e = hipDeviceSynchronize()) != hipSuccess) return e;
     if (dev < 0 || dev >= 16 || !g_chain_dev[dev].ctl) return hipSuccess;
     int ctl[CHAIN_SLOTS * 16];
     if ((e = hipMemcpy(ctl, g_chain_dev[dev].ctl, sizeof(ctl), hipMemcpyDeviceToHost)) != hipSuccess) return e;

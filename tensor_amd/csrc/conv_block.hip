@@ -357,7 +357,12 @@ __global__ void __launch_bounds__(64 * WV) conv_block_kernel(const BlockArgs a) 
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_blk, acc[i][1]), rp, (int)(mine + (unsigned)it * 2048u + 1024u), 0, AGENT);
             }
         }
-        __syncthreads();  // every wave's stores are acknowledged (the barrier's wait covers the memory counter)
+        // A barrier does not wait for the memory counter: every wave first waits until its own stores have been
+        // acknowledged (vmcnt(0)), and only then does the barrier say that the whole workgroup's partial sums are
+        // visible at agent scope. Without the wait the arrival below could be counted while a store is still in flight,
+        // and the last workgroup would add whatever the slot held before.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
         int* const flag = reinterpret_cast<int*>(ldsD);  // (the depthwise results are not read any more)
         if (tid == 0) {
             const unsigned before = __hip_atomic_fetch_add(a.counters + bi, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -606,31 +611,53 @@ void block_pack_dw_consts(const int8_t* w, const float* si, const float* bi, con
     }
 }
 
-// The arrival counters of the bands whose slices are dealt to several workgroups: a ring in static device memory (every
-// GPU has its own copy; the address is looked up once per device). A launch takes the next N x bands words; the last
-// workgroup of a band leaves its word at zero again, so the ring needs no clearing, and launches that overlap on
-// different streams count in different words.
+// The arrival counters of the bands whose slices are dealt to several workgroups live in static device memory (every
+// GPU has its own copy; the address is looked up once per device), in two halves:
+//  * launches that run now take the next N x bands words of a ring (the lower half). The last workgroup of a band leaves
+//    its word at zero again, so the ring needs no clearing, and launches that overlap on different streams count in
+//    different words as long as fewer than BLK_COUNTERS / 2 words are handed out between them;
+//  * launches recorded into a HIP graph keep the words they were given for as long as the graph is replayed, so they must
+//    never meet the ring: they take theirs from the upper half, which is only handed to captured launches, and a small
+//    fill kernel recorded in front of the launch zeroes them on every replay (a replay that was cut short cannot poison
+//    the next one). When the upper half has been handed out once it is dealt again from its start: two graphs whose
+//    launches share words must then not be replayed at the same time.
 constexpr int BLK_COUNTERS = 1 << 17;
 static __device__ unsigned blk_counters[BLK_COUNTERS];
 static std::mutex g_counter_mutex;
 static unsigned* g_counter_ptr[64] = {};
-static unsigned g_counter_next[64] = {};
+static unsigned g_counter_next[64][2] = {};
 
-static hipError_t block_counters(int words, unsigned** out) {
+__global__ void blk_zero_counters_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+static hipError_t block_counters(int words, hipStream_t stream, unsigned** out) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64 || words > BLK_COUNTERS / 2) return hipErrorInvalidValue;
-    std::lock_guard<std::mutex> lock(g_counter_mutex);
-    if (!g_counter_ptr[dev]) {
-        void* p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(blk_counters));
-        if (e != hipSuccess || !p) return e == hipSuccess ? hipErrorInvalidSymbol : e;
-        g_counter_ptr[dev] = static_cast<unsigned*>(p);
+    constexpr unsigned HALF = BLK_COUNTERS / 2;
+    if (dev < 0 || dev >= 64 || words < 1 || (unsigned)words > HALF) return hipErrorInvalidValue;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if ((e = hipStreamIsCapturing(stream, &cs)) != hipSuccess) return e;
+    const int half = cs == hipStreamCaptureStatusNone ? 0 : 1;
+    {
+        std::lock_guard<std::mutex> lock(g_counter_mutex);
+        if (!g_counter_ptr[dev]) {
+            void* p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(blk_counters));
+            if (e != hipSuccess || !p) return e == hipSuccess ? hipErrorInvalidSymbol : e;
+            g_counter_ptr[dev] = static_cast<unsigned*>(p);
+        }
+        unsigned& next = g_counter_next[dev][half];
+        if (next + (unsigned)words > HALF) next = 0;
+        *out = g_counter_ptr[dev] + half * HALF + next;
+        next += (unsigned)words;
     }
-    if (g_counter_next[dev] + (unsigned)words > (unsigned)BLK_COUNTERS) g_counter_next[dev] = 0;
-    *out = g_counter_ptr[dev] + g_counter_next[dev];
-    g_counter_next[dev] += (unsigned)words;
+    if (half) {
+        hipLaunchKernelGGL(blk_zero_counters_kernel, dim3((words + 255) / 256), dim3(256), 0, stream, *out, words);
+        return hipGetLastError();
+    }
     return hipSuccess;
 }
 
@@ -664,7 +691,7 @@ hipError_t run_conv_block(const int8_t* x, const int8_t* w_exp, const int32_t* k
     a.partial = workspace, a.partial_bytes = plan[5] * 4, a.counters = nullptr;
     if (plan[4] > 1) {
         if (!workspace) return hipErrorInvalidValue;
-        const hipError_t ce = block_counters(ge.N * plan[1], &a.counters);
+        const hipError_t ce = block_counters(ge.N * plan[1], stream, &a.counters);
         if (ce != hipSuccess) return ce;
     }
     a.x = x, a.w_exp = w_exp, a.k1 = k1, a.k2 = k2, a.w_prj = w_prj, a.out = out;

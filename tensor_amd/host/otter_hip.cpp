@@ -15,6 +15,9 @@
 
 namespace otter {
 
+// set by ConvolutionLayer::forward_chain, cleared by the download that asks otter_hip_conv_chain_status
+static std::atomic<bool> g_chain_unchecked{false};
+
 namespace {
 
 void hip_check(int rc, const char* what) {
@@ -210,6 +213,13 @@ const void* Tensor::data_ptr() const {
         OTTER_CHECK(s.dev_valid, "tensor has no valid copy");
         hip_check(otter_hip_memcpy_d2h(s.host, s.dev, s.bytes, nullptr), "download");
         hip_check(otter_hip_stream_synchronize(nullptr), "download");
+        // Blobs computed behind a chain launch are only good if none of its bounded waits gave up: asked once per
+        // download that follows such a launch (the device is idle here anyway).
+        if (g_chain_unchecked.exchange(false)) {
+            int gave_up = 0;
+            hip_check(otter_hip_conv_chain_status(&gave_up), "chain status");
+            if (gave_up) throw Error("a chain launch gave up waiting for a producer tile: the blobs computed since are not valid");
+        }
         s.host_valid = true;
     }
     return s.host;
@@ -700,6 +710,7 @@ int ConvolutionLayer::forward_chain(const std::vector<const ConvolutionLayer*>& 
         if (rc) return rc;
         top.mark_device_written();
         ++g_chain_forwards;
+        g_chain_unchecked.store(true);
     } catch (const Error&) {
         return -100;
     }

@@ -152,6 +152,40 @@ def test_block_with_the_exact_rounding_mode(hip, act, f32_out):
         l["conv"].close()
 
 
+@pytest.mark.parametrize("cin,ce,cout,H,split,f32_out", [(160, 960, 160, 7, 4, True), (160, 960, 320, 7, 8, False),
+                                                         (64, 384, 64, 14, 3, True)])
+def test_split_bands_on_changing_inputs_sharing_one_workspace(hip, cin, ce, cout, H, split, f32_out):
+    """Bands whose slices are dealt to several workgroups hand their partial sums over through the workspace. Launches
+    on DIFFERENT inputs, back to back on one stream and one workspace with no synchronisation in between: a partial sum
+    that the last workgroup of a band picked up before its store had landed would be the previous launch's (a different
+    number here), so every result must equal the three layers one by one bit for bit."""
+    torch = hip.torch
+    rng = np.random.default_rng(77 + H + split)
+    N, W = 6, H
+    layers = make_block(hip, rng, cin, ce, cout, 3, f32_out)
+    e, d, p = (l["conv"] for l in layers)
+    e.set_block_plan(0, 0, split)
+    assert hip.conv_block_launches(e, d, p, N, H, W) == 1
+    import ctypes
+    plan = (ctypes.c_int * 6)()
+    assert hip.lib.otter_hip_conv_block_plan(cin, ce, cout, N, H, W, 0, 0, split, plan) == 0
+    assert plan[4] > 1 and plan[5] > 0  # several workgroups per band, partial sums in the workspace
+    xs = [hip.to_device(capi.pack_np(rng.integers(-127, 128, (N, cin, H, W)).astype(np.int8), 8)) for _ in range(8)]
+    wants = [one_by_one(hip, layers, x, N, H, W, None, None)[0].clone() for x in xs]
+    ws = hip.empty(hip.lib.otter_hip_conv_block_workspace_bytes(e.h, d.h, p.h, N, H, W), np.int8)
+    outs = [hip.empty(N * cout * H * W, np.float32 if f32_out else np.int8) for _ in xs]
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for x, out in zip(xs, outs):
+            hip.conv_block(e, d, p, x, N, H, W, out=out, workspace=ws)
+        torch.cuda.synchronize()
+        for out, want in zip(outs, wants):
+            assert torch.equal(out, want.view(-1))
+            out.zero_()
+    for l in layers:
+        l["conv"].close()
+
+
 def test_block_replayed_from_a_captured_graph(hip):
     """A launch whose bands are dealt to several workgroups, captured into a graph and replayed on new inputs, with eager
     launches in between: the arrival counters it was captured with are left at zero by every launch, so each replay

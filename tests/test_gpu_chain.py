@@ -112,10 +112,11 @@ def test_same_shape_chain_that_needs_two_lds_stages_runs_layer_by_layer(hip):
 
 
 def test_chains_on_several_streams_at_once(hip):
-    """Every stream that uses the entry point gets a flag set of its own (four per GPU); launches on different streams
-    may overlap. Six streams each run their own chain, enqueued back to back without a synchronisation in between: the
-    first four as one launch each, the last two layer by layer (no flag set left) - every result equals the layers one
-    by one."""
+    """A GPU has four flag sets; a stream without one takes a free set or an idle one (least recently used, last launch
+    completed), so launches on different streams may overlap. Six streams each run their own chain, enqueued back to
+    back without a synchronisation in between: the first four are one launch each (the device is idle when they start,
+    whoever owned the sets before), the last two are one launch if a set has come free by then and layer by layer if
+    not - every result equals the layers one by one."""
     torch = hip.torch
     rng = np.random.default_rng(21)
     N, C, H, W, L = 8, 128, 28, 28, 4
@@ -130,9 +131,14 @@ def test_chains_on_several_streams_at_once(hip):
     outs = []
     for rep in range(3):
         outs = []
-        for convs, xd, want, st in jobs:
+        for j, (convs, xd, want, st) in enumerate(jobs):
             with torch.cuda.stream(st):
                 outs.append(hip.conv_chain(convs, xd, N, H, W))
+            made = hip.conv_chain_last_launches()
+            assert made in (1, L)
+            if rep == 0 and j < 4:
+                assert made == 1
+        torch.cuda.synchronize()
     assert not hip.conv_chain_gave_up()  # (synchronizes the device)
     for (convs, xd, want, st), got in zip(jobs, outs):
         np.testing.assert_array_equal(got.cpu().numpy(), want)
@@ -167,11 +173,13 @@ def test_chain_replayed_from_a_captured_graph(hip):
     assert hip.conv_chain_launches(convs, N, H, W) == 1
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
-        hip.conv_chain(convs, x_static, N, H, W, out=out, workspace=ws)  # (first call on this stream: takes its flag set)
+        hip.conv_chain(convs, x_static, N, H, W, out=out, workspace=ws)  # (first call on this stream: takes a flag set)
+    assert hip.conv_chain_last_launches() == 1  # the persistent kernel, not the layers one by one
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         hip.conv_chain(convs, x_static, N, H, W, out=out, workspace=ws)
+        assert hip.conv_chain_last_launches() == 1
     for rep in range(2):
         for x, want in zip(xs, wants):
             x_static.copy_(x)
@@ -181,6 +189,7 @@ def test_chain_replayed_from_a_captured_graph(hip):
             # eager work on the same flag set between replays
             with torch.cuda.stream(side):
                 eager = hip.conv_chain(convs, x, N, H, W)
+            assert hip.conv_chain_last_launches() == 1
             side.synchronize()
             assert bool((eager == want.view(-1)).all().item())
     assert not hip.conv_chain_gave_up()

@@ -23,6 +23,7 @@
 #include "Quantize.hpp"
 #include "Convolution.hpp"
 #include "ConvolutionLayer.hpp"
+#include "LayerRegistry.hpp"
 #include "NetOption.hpp"
 #include "Net.hpp"
 #include "ParamDict.hpp"
@@ -224,7 +225,9 @@ __attribute__((visibility("default"))) otter_ref_conv_layer* otter_ref_conv_laye
             if (eq != std::string::npos) lo[kv.substr(0, eq)] = kv.substr(eq + 1);
             pos = e + 1;
         }
-        auto* L = new otter::ConvolutionLayer();
+        // through the registry, as Net::compile does (Tensor/Net.cpp:196): whatever creator is registered under
+        // "Convolution" makes the layer -- the stock one, or the GPU layer of ref_hip_layer.cpp while that is switched on
+        auto* L = static_cast<otter::ConvolutionLayer*>(otter::LayerRegistry::CreateLayer("Convolution"));
         L->bottom_shapes.push_back(otter::tensor({in_n, in_c, in_h, in_w}, ScalarType::Int).view({1, -1}));
         otter::ParamDict pd;
         L->parse_param(lo, pd);

@@ -1525,6 +1525,14 @@ void Net::compile(CompileMode mode) {
         OTTER_CHECK(layer->parse_param(lo, pd) == 0, "layer " + layer->name + ": parse_param failed");
         OTTER_CHECK(layer->compute_output_shape(pd) == 0, "layer " + layer->name + ": compute_output_shape failed");
         OTTER_CHECK(layer->load_param(pd) == 0, "layer " + layer->name + ": load_param failed");
+        // The description already says which convolutions are fp32 (int8_scale_term 0, e.g. conv_1 of the reference's
+        // benchmark/nanodet-plus-m-1.5x_416_int8_mixed.otter): refuse the graph here, by name, rather than return a bare
+        // -1 from that layer's forward later.
+        if (const auto* conv = dynamic_cast<const ConvolutionLayer*>(layer))
+            OTTER_CHECK(conv->int8_scale_term != 0,
+                        "layer " + layer->name + ": an fp32 convolution (int8_scale_term 0) is outside the int8 path this "
+                        "library accelerates; keep such a graph on the reference's Net with the GPU layer registered for "
+                        "its int8 convolutions, which leaves this layer to the stock ConvolutionLayer");
         if (mode == CompileMode::Initial) {
             layer->init_model();
             layer->create_pipeline(option);

@@ -49,7 +49,7 @@ def conv_record(wq, bias, weight_scales, bottom_scale, top_scale, int8_scale_ter
 
 
 def synthetic_int8_weights(layers, rng, bottom_scale=24.0):
-    """A `.bin` for every Convolution of `layers` (hostnet.Net.describe()): int8 weights uniform in [-127, 127] whose
+    """A `.bin` for every Convolution of `layers` (hostnet.Net.describe()): for the int8 ones, int8 weights uniform in [-127, 127] whose
     per-channel scale makes the dequantised weights He-like (so that activations stay O(1) through the network), a
     small bias, and one activation scale for every blob. Returns (bytes, {layer name: dict of what was written})."""
     blob = b""
@@ -57,10 +57,16 @@ def synthetic_int8_weights(layers, rng, bottom_scale=24.0):
     for typ, name, _bottoms, _tops, c, _shape in layers:
         if typ != "Convolution":
             continue
-        if not c["int8_scale_term"]:
-            raise ValueError("%s is not an int8 convolution" % name)
         K, cin, g = c["K"], c["C"], c["groups"]
         fan_in = cin // g * c["kh"] * c["kw"]
+        if not c["int8_scale_term"]:
+            # an fp32 convolution inside an int8 model (conv_1 of the reference's ..._int8_mixed.otter): untagged fp32
+            # weights, He-like so that its result is O(1) like every other blob, then the bias
+            w = rng.normal(0, np.sqrt(2.0 / fan_in), (K, cin // g, c["kh"], c["kw"])).astype(np.float32)
+            bias = rng.normal(0, 0.05, K).astype(np.float32) if c["bias_term"] else None
+            blob += weight_fp32(w) + (vector(bias) if bias is not None else b"")
+            written[name] = dict(w=w, bias=bias, int8_scale_term=0)
+            continue
         wq = rng.integers(-127, 128, size=(K, cin // g, c["kh"], c["kw"])).astype(np.int8)
         dw = cin == g and g == K
         n_ws = 1 if (dw and c["int8_scale_term"] in (2, 102)) else K

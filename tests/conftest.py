@@ -26,6 +26,14 @@ def golden():
 
 
 @pytest.fixture(scope="session")
+def tie_golden():
+    """Layer results on the one value where the reference's two rounding primitives differ (cases.TIE_ROUTE_CASES),
+    written by the compiled reference through tests/golden/make_tie_route_golden.py."""
+    path = os.path.join(ROOT, "tests", "golden", "tie_route_golden.npz")
+    return dict(np.load(path, allow_pickle=False))
+
+
+@pytest.fixture(scope="session")
 def ref():
     """The compiled reference, where oracle/_ref/libotter_ref.so exists; otherwise the test is skipped."""
     from oracle.binding import Ref, ref_available

@@ -74,3 +74,67 @@ def make_inputs(case, seed):
     b = rng.normal(0, 0.5, K).astype(np.float32) if bias else None
     top_scale = np.float32(127.0 / 6.0) if act == "Relu6" else np.float32(rng.uniform(8.0, 30.0))
     return dict(x=x, wq=wq, w_scales=w_scales, in_scale=np.float32(in_scale), bias=b, top_scale=top_scale)
+
+
+# Layers whose results sit on the ONE value where the reference's two rounding primitives part ways:
+# float2int8_sse (Tensor/VecIntrinsic.hpp:71-95, the packed SIMD loops) rounds 0.49999997f (the largest float below one
+# half) to 1 because fl(0.49999997f + 0.5f) = 1.0f, float2int8 = (int)round(v) (the scalar loops) rounds it to 0; for
+# every other float the two agree. Which primitive a LAYER ends in is decided by the reference's routing over
+# (C, K, groups, packing) -- Tensor/QuantizeX86.cpp:402,492-545,617-641 (quantize), :1177-1179,1723-1870,2075-2120
+# (requantize) -- and random tensors never meet that value, so these cases are the only vectors that pin the routing.
+# Same columns as LAYER_CASES plus use_packing_layout. int8-input cases put the tie into the requantize step, fp32-input
+# cases into the quantize step (make_tie_inputs).
+TIE_ROUTE_CASES = [
+    ("tie_requant_k8_packed_1x1",      8,  8, 1, 1, 0, 1,  1, 6, 6, 2, True,  True, True, "",     None, True),
+    ("tie_requant_k8_packed_3x3_relu", 8,  8, 3, 1, 1, 1,  1, 6, 6, 1, True,  True, True, "Relu", None, True),
+    ("tie_requant_k12_packed_byte",   16, 12, 1, 1, 0, 1,  1, 6, 6, 1, True,  True, True, "",     None, True),
+    ("tie_requant_k6_packed_8to1",     8,  6, 3, 1, 1, 1,  1, 6, 6, 1, True,  True, True, "",     None, True),
+    ("tie_requant_dw16_packed",       16, 16, 3, 1, 1, 1, 16, 6, 6, 1, True,  True, True, "",     None, True),
+    ("tie_requant_dw16s2_packed",     16, 16, 3, 2, 1, 1, 16, 7, 7, 1, True,  True, True, "",     None, True),
+    ("tie_requant_k8_unpacked",        8,  8, 3, 1, 1, 1,  1, 6, 6, 1, True,  True, True, "",     None, False),
+    ("tie_requant_k12_unpacked",      16, 12, 1, 1, 0, 1,  1, 6, 6, 1, True,  True, True, "",     None, False),
+    ("tie_quant_c8_packed",            8,  8, 1, 1, 0, 1,  1, 6, 6, 1, False, True, True, "",     None, True),
+    ("tie_quant_c16_packed_dw",       16, 16, 3, 1, 1, 1, 16, 6, 6, 1, False, True, True, "",     None, True),
+    ("tie_quant_c4_packed",            4,  8, 3, 1, 1, 1,  1, 6, 6, 1, False, True, True, "",     None, True),
+    ("tie_quant_c3_packed_stem",       3,  8, 3, 2, 1, 1,  1, 9, 9, 1, False, True, True, "",     None, True),
+    ("tie_quant_c8_unpacked",          8,  8, 1, 1, 0, 1,  1, 6, 6, 1, False, True, True, "",     None, False),
+]
+
+
+def make_tie_inputs(case):
+    """Inputs that put layer results exactly on +-0.49999997f (and on neighbours where both primitives agree).
+
+    Weights: the centre tap of input channel 0 (depthwise: of the channel itself) is +1 for even and -1 for odd output
+    channels, every other weight is 0, so an accumulator is +-x[channel 0].
+    int8 input (requantize side): in_scale = w_scale = 16, hence scale_in = 1/256 exactly; x takes values in
+    {64, -64, 32, 96, 0, 17}; bias = +-(0.25f - 2^-25); top_scale = 1. acc = 64 with the positive bias gives
+    fma(64, 2^-8, 0.25 - 2^-25) = 0.49999997f with no rounding on the way, acc = -64 with the negative bias its negative.
+    fp32 input (quantize side): in_scale = 1, x takes values in {+-0.49999997f, 0.5, 0.25, 1.4999999f, -2.5, 0};
+    w_scale = 0.125 (scale_in = 8), bias = 0.25, top_scale = 1, so the int8 result is 8 x the quantized input and never
+    itself near a tie."""
+    import numpy as np
+    name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params, packing = case
+    rng = np.random.default_rng(sum(map(ord, name)))
+    wq = np.zeros((K, C // g, k, k), np.int8)
+    for o in range(K):
+        wq[o, 0, k // 2, k // 2] = 1 if o % 2 == 0 else -1
+    just_below_half = np.nextafter(np.float32(0.5), np.float32(0))
+    if in_i8:
+        x = np.zeros((N, C, H, W), np.int8)
+        vals = np.array([64, -64, 32, 96, 0, 17, -96], np.int8)
+        chans = range(C) if g == C else [0]
+        for c in chans:
+            x[:, c] = rng.choice(vals, size=(N, H, W), p=[0.3, 0.3, 0.1, 0.1, 0.1, 0.05, 0.05])
+        in_scale, w_scale = np.float32(16), np.float32(16)
+        t = np.float32(0.25) - np.float32(2.0 ** -25)
+        b = np.array([t if (o % 4) < 2 else -t for o in range(K)], np.float32)
+    else:
+        x = np.zeros((N, C, H, W), np.float32)
+        vals = np.array([just_below_half, -just_below_half, 0.5, 0.25, np.nextafter(np.float32(1.5), np.float32(0)), -2.5, 0.0],
+                        np.float32)
+        chans = range(C) if g == C else [0]
+        for c in chans:
+            x[:, c] = rng.choice(vals, size=(N, H, W), p=[0.3, 0.3, 0.1, 0.1, 0.1, 0.05, 0.05])
+        in_scale, w_scale = np.float32(1), np.float32(0.125)
+        b = np.full(K, 0.25, np.float32)
+    return dict(x=x, wq=wq, w_scales=np.full(K, w_scale, np.float32), in_scale=in_scale, bias=b, top_scale=np.float32(1.0))

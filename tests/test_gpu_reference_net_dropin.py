@@ -16,6 +16,9 @@ pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NANODET = os.path.join(GOLDEN, "nanodet-plus-m-1.5x_416_int8_fused.otter")
+# the reference's other int8 description (benchmark/benchotter.cpp:88-90 runs both): the same network with conv_1 kept
+# in fp32 (int8_scale_term 0)
+NANODET_MIXED = os.path.join(GOLDEN, "nanodet-plus-m-1.5x_416_int8_mixed.otter")
 HEADS = ["conv_95", "conv_100", "conv_105", "conv_110"]  # what feeds the detection post-processing
 
 
@@ -27,11 +30,17 @@ def ref_hip():
     return Ref(hip=True)
 
 
-def test_reference_net_with_the_gpu_convolution_layer_registered(ref_hip, tmp_path):
+@pytest.mark.parametrize("description,n_gpu", [(NANODET, 110), (NANODET_MIXED, 109)], ids=["int8_fused", "int8_mixed"])
+def test_reference_net_with_the_gpu_convolution_layer_registered(ref_hip, tmp_path, description, n_gpu):
+    """int8_mixed: the fp32 conv_1 must fall through to the stock ConvolutionLayer inside the GPU layer (its
+    create_pipeline makes no handle for an fp32 layer), the other 109 convolutions go through the C ABI."""
     rng = np.random.default_rng(23)
     probe = hostnet.Net(lightmode=False)  # only to enumerate the layers for the synthetic weight file
-    probe.load_otter(NANODET)
+    probe.load_otter(NANODET)             # (the two descriptions differ in conv_1's int8_scale_term only)
     layers = probe.describe()
+    if description == NANODET_MIXED:
+        assert layers[1][0] == "Convolution" and layers[1][1] == "conv_1"
+        layers[1][4]["int8_scale_term"] = 0
     blob, _ = modelfile.synthetic_int8_weights(layers, rng)
     path = str(tmp_path / "nanodet_int8.bin")
     with open(path, "wb") as f:
@@ -42,17 +51,17 @@ def test_reference_net_with_the_gpu_convolution_layer_registered(ref_hip, tmp_pa
     names = HEADS + int8_convs[::6]
     x = rng.uniform(0, 1, (1, 3, 416, 416)).astype(np.float32)
 
-    stock = ref_hip.net(NANODET, path)
+    stock = ref_hip.net(description, path)
     want, _ = stock.run("data_1", x, names)
-    assert ref_hip.hip_forward_count() == 0
 
     ref_hip.use_hip_convolution(True)
     try:
-        gpu = ref_hip.net(NANODET, path)  # compiled now: its 110 "Convolution" layers come from the new creator
+        gpu = ref_hip.net(description, path)  # compiled now: its 110 "Convolution" layers come from the new creator
     finally:
         ref_hip.use_hip_convolution(False)
+    before = ref_hip.hip_forward_count()
     got, _ = gpu.run("data_1", x, names)
-    assert ref_hip.hip_forward_count() == 110  # every convolution of the net went through the C ABI
+    assert ref_hip.hip_forward_count() - before == n_gpu  # every int8 convolution of the net went through the C ABI
 
     n_int8 = 0
     for n in names:
@@ -68,6 +77,7 @@ def test_reference_net_with_the_gpu_convolution_layer_registered(ref_hip, tmp_pa
 
     # the stock creator is back: a net compiled now runs on the CPU again
     before = ref_hip.hip_forward_count()
-    again = ref_hip.net(NANODET, path)
+    again = ref_hip.net(description, path)
     again.run("data_1", x, HEADS[:1])
     assert ref_hip.hip_forward_count() == before
+

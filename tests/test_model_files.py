@@ -108,3 +108,13 @@ def test_quantize_weights_definition():
     np.testing.assert_allclose(ws, [127.0, 635.0, 127.0])
     wq1, ws1 = calibration.quantize_weights(w, per_channel=False)
     assert ws1.shape == (1,) and wq1.reshape(-1)[1] == -127 and wq1.reshape(-1)[2] == 25
+
+
+@pytest.mark.gpu
+def test_host_net_refuses_the_mixed_description_by_name():
+    """The library's own Net runs int8 convolutions only: it refuses a graph with an fp32 convolution when it is compiled,
+    naming the layer, rather than fail inside a forward pass."""
+    net = hostnet.Net()
+    with pytest.raises(hostnet.HostError, match="conv_1.*fp32 convolution"):
+        net.load_otter(os.path.join(GOLDEN, "nanodet-plus-m-1.5x_416_int8_mixed.otter"))
+    net.close()

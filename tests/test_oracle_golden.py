@@ -3,7 +3,7 @@
 import numpy as np
 import pytest
 
-from cases import LAYER_CASES, UNPACKED_LAYER_CASES
+from cases import LAYER_CASES, TIE_ROUTE_CASES, UNPACKED_LAYER_CASES, make_tie_inputs
 from oracle.binding import ROUND_EXACT, ROUND_SSE
 
 ACT = {"": 0, "Relu": 1, "LRelu": 2, "Relu6": 3}
@@ -192,3 +192,45 @@ def test_eltwise_add_is_the_fp32_sum(oracle):
     a = rng.normal(0, 1e3, 1001).astype(np.float32)
     b = rng.normal(0, 1e-3, 1001).astype(np.float32)
     np.testing.assert_array_equal(oracle.eltwise_add(a, b), a + b)
+
+
+@pytest.mark.parametrize("case", TIE_ROUTE_CASES, ids=[c[0] for c in TIE_ROUTE_CASES])
+def test_layer_routing_of_the_rounding_primitive_matches_reference(oracle, tie_golden, case):
+    """Which rounding primitive a layer ends in (otter_oracle_quantize_round_mode / otter_oracle_requantize_round_mode
+    inside otter_oracle_conv_layer_forward) against layer results of the compiled reference that sit exactly on
+    +-0.49999997f, the one value the two primitives round differently. The layer as a whole must reproduce the vector;
+    put together from its steps with the OTHER primitive in the step under test it must not (so the vector does
+    discriminate), and with the primitive the routing function names it must."""
+    name, C, K, k, s, p, d, g, H, W, N, in_i8, i8_out, bias, act, act_params, packing = case
+    t = make_tie_inputs(case)
+    want = tie_golden[name + "/out"]
+    np.testing.assert_array_equal(oracle.scale_in(t["w_scales"], float(t["in_scale"])).view(np.int32),
+                                  tie_golden[name + "/scale_in"].view(np.int32))
+    out = oracle.conv_layer_forward(t["x"], t["wq"], t["w_scales"], float(t["in_scale"]), stride=(s, s), pad=(p, p),
+                                    dil=(d, d), groups=g, bias=t["bias"], top_scale=float(t["top_scale"]), int8_out=True,
+                                    act_type=ACT[act], use_packing=packing)
+    np.testing.assert_array_equal(out, want)
+
+    def by_steps(q_mode, r_mode):
+        xq = t["x"] if in_i8 else oracle.quantize(t["x"], [t["in_scale"]], q_mode)
+        acc = oracle.conv_int32(xq, t["wq"], (s, s), (p, p), (d, d), g)
+        return oracle.requantize(acc, oracle.scale_in(t["w_scales"], float(t["in_scale"])), [t["top_scale"]], t["bias"],
+                                 ACT[act], None, r_mode)
+
+    other = {ROUND_SSE: ROUND_EXACT, ROUND_EXACT: ROUND_SSE}
+    q_mode, r_mode = oracle.quantize_round_mode(C, packing), oracle.requantize_round_mode(C, K, g, packing)
+    np.testing.assert_array_equal(by_steps(q_mode, r_mode), want)
+    if in_i8:
+        assert (by_steps(q_mode, other[r_mode]) != want).any(), "the vector does not tell the requantize primitives apart"
+    else:
+        assert (by_steps(other[q_mode], r_mode) != want).any(), "the vector does not tell the quantize primitives apart"
+
+
+def test_tie_route_cases_cover_both_primitives_on_both_sides(oracle):
+    """The case table meets every branch of the routing: SIMD and scalar rounding, in quantize and in requantize."""
+    seen = set()
+    for case in TIE_ROUTE_CASES:
+        C, K, g, in_i8, packing = case[1], case[2], case[7], case[11], case[16]
+        seen.add(("requantize", oracle.requantize_round_mode(C, K, g, packing)) if in_i8 else
+                 ("quantize", oracle.quantize_round_mode(C, packing)))
+    assert seen == {("quantize", ROUND_SSE), ("quantize", ROUND_EXACT), ("requantize", ROUND_SSE), ("requantize", ROUND_EXACT)}

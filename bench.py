@@ -155,7 +155,10 @@ def build_c3(hip, capi, rng):
 
 
 def build_c1(hip, capi, rng, stride):
-    """configs[1]: depthwise 3x3 p1 on 8x256x112x112 fp32, bias, ReLU6, requantize to int8 with 127/6."""
+    """configs[1]: depthwise 3x3 p1 on 8x256x112x112 fp32, bias, ReLU6, requantize to int8 with 127/6. The step is the
+    configuration as stated: the layer on the fp32 Float8 blob, ONE launch that quantizes on the way in
+    (conv_dw3x3_f32in_kernel). The layer on an int8 blob (what a depthwise layer inside a network sees) and the
+    standalone quantize pass are timed beside it."""
     N, C, H, W = 8, 256, 112, 112
     x = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
     wq, ws = quantize_weights(rng.normal(0, 0.1, (C, 1, 3, 3)).astype(np.float32))
@@ -172,29 +175,34 @@ def build_c1(hip, capi, rng, stride):
     scale_dev = hip.to_device(np.array([in_scale], np.float32))
 
     def step():
-        hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
-        conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out)
+        conv.forward(xd, capi.F32_P8, N, H, W, capi.I8_P8, out=out, workspace=xq)
         return out
 
     in_b, out_b = N * C * H * W, N * C * oh * ow
     # the same launches over enough buffer sets that nothing a launch reads is still in a cache from the last time
-    step()
-    n_dom = cold_sets(in_b + out_b)
-    xqs, outs = [xq.clone() for _ in range(n_dom)], [hip.empty(out_b, np.int8) for _ in range(n_dom)]
-    dom_cold = [lambda i=i: conv.forward(xqs[i], capi.I8_P8, N, H, W, capi.I8_P8, out=outs[i]) for i in range(n_dom)]
-    n_aux = cold_sets(5 * in_b)
-    xds, xq2 = [xd.clone() for _ in range(n_aux)], [hip.empty(in_b, np.int8) for _ in range(n_aux)]
-    aux_cold = [lambda i=i: hip.quantize(xds[i], capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq2[i])
-                for i in range(n_aux)]
-    return dict(name="c1s%d" % stride, step=step, dom_fn_cold=dom_cold, ops=2.0 * N * C * 9 * oh * ow, launches=2,
-                bytes=5 * in_b + in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=in_b + out_b, bound="hbm",
-                workload="depthwise int8 3x3 s%d p1, 8x256x112x112 fp32 in -> quantize -> conv+bias+ReLU6+requantize "
-                         "-> int8" % stride,
-                dom_kernel="depthwise 3x3 s%d + requantize (int8 in -> int8 out)" % stride,
-                dom_fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out),
-                aux=dict(kernel="quantize fp32 Float8 -> Byte8", bytes=5 * in_b, fn_cold=aux_cold,
-                         fn=lambda: hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8,
-                                                 dst=xq)),
+    hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq)
+    n_dom = cold_sets(4 * in_b + out_b)
+    xds, outs = [xd.clone() for _ in range(n_dom)], [hip.empty(out_b, np.int8) for _ in range(n_dom)]
+    dom_cold = [lambda i=i: conv.forward(xds[i], capi.F32_P8, N, H, W, capi.I8_P8, out=outs[i], workspace=xq) for i in range(n_dom)]
+    n_i8 = cold_sets(in_b + out_b)
+    xqs, outs8 = [xq.clone() for _ in range(n_i8)], [hip.empty(out_b, np.int8) for _ in range(n_i8)]
+    i8_cold = [lambda i=i: conv.forward(xqs[i], capi.I8_P8, N, H, W, capi.I8_P8, out=outs8[i]) for i in range(n_i8)]
+    xq2 = [hip.empty(in_b, np.int8) for _ in range(n_dom)]
+    q_cold = [lambda i=i: hip.quantize(xds[i], capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq2[i])
+              for i in range(n_dom)]
+    return dict(name="c1s%d" % stride, step=step, dom_fn_cold=dom_cold, ops=2.0 * N * C * 9 * oh * ow, launches=1,
+                bytes=4 * in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=4 * in_b + out_b, bound="hbm",
+                workload="depthwise int8 3x3 s%d p1, 8x256x112x112 fp32 in -> quantize + conv + bias + ReLU6 + requantize "
+                         "-> int8, one launch" % stride,
+                dom_kernel="conv_dw3x3_f32in_kernel: quantize + depthwise 3x3 s%d + requantize (fp32 Float8 in -> int8 "
+                           "out)" % stride,
+                dom_fn=step,
+                aux=[dict(kernel="conv_dw3x3_mfma_kernel: the same layer on an int8 Byte8 blob (int8 in -> int8 out)",
+                          bytes=in_b + out_b, fn_cold=i8_cold,
+                          fn=lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out)),
+                     dict(kernel="quantize fp32 Float8 -> Byte8 as a pass of its own", bytes=5 * in_b, fn_cold=q_cold,
+                          fn=lambda: hip.quantize(xd, capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8,
+                                                  dst=xq))],
                 x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
                 shape=(N, C, H, W), stride=stride)
 
@@ -694,16 +702,15 @@ def measure(wl, timer, steps, warmup, unit_main):
             res["roofline_resident"] = dict(kernel_ms=kms_resident, achieved=wl["dom_bytes"] / (kms_resident * 1e-3) / 1e9,
                                             frac=wl["dom_bytes"] / (kms_resident * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                             working_set="one buffer set, %d MB (cache-resident)" % (wl["dom_bytes"] >> 20))
-    if "aux" in wl:
-        aux = wl["aux"]
+    for aux in wl.get("aux", []):
         ams_res, _ = timer.run(aux["fn"], max(steps * 4, 50), 5)
         ams = ams_res
         if aux.get("fn_cold"):
             ams, _ = timer.run(aux["fn_cold"], max(steps * 4, 50), 2 * len(aux["fn_cold"]))
-        res["aux_kernel"] = dict(kernel=aux["kernel"], kernel_ms=ams, gbs=aux["bytes"] / (ams * 1e-3) / 1e9,
-                                 frac_hbm=aux["bytes"] / (ams * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                                 resident_kernel_ms=ams_res,
-                                 resident_frac_hbm=aux["bytes"] / (ams_res * 1e-3) / 1e9 / PEAK_HBM_GBS)
+        res.setdefault("aux_kernels", []).append(
+            dict(kernel=aux["kernel"], kernel_ms=ams, gbs=aux["bytes"] / (ams * 1e-3) / 1e9,
+                 frac_hbm=aux["bytes"] / (ams * 1e-3) / 1e9 / PEAK_HBM_GBS, resident_kernel_ms=ams_res,
+                 resident_frac_hbm=aux["bytes"] / (ams_res * 1e-3) / 1e9 / PEAK_HBM_GBS))
     return res
 
 
@@ -808,8 +815,8 @@ def main():
                        ("layers_per_step" if wl["name"] in ("c4", "det") else "launches_per_step"): wl["launches"],
                        "settle_s": SETTLE_S},
             "roofline": res["roofline"], "wall_ms_per_step": res["wall_ms_per_step"]}
-    if "aux_kernel" in res:
-        line["aux_kernel"] = res["aux_kernel"]
+    if "aux_kernels" in res:
+        line["aux_kernels"] = res["aux_kernels"]
     if "roofline_resident" in res:
         line["roofline_resident"] = res["roofline_resident"]
     if no_settle is not None:

@@ -392,6 +392,14 @@ static bool use_stem(const otter_hip_conv* h, int in_layout, const ConvGeom& g_i
 
 // 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS, 4 few-channel 3x3 (image stem),
 // 5 streamed 1x1 over few input channels
+// a depthwise 3x3 layer that reads an fp32 Float8 blob and can run quantize + convolution as one launch
+static bool use_dw_f32in(const otter_hip_conv* h, int in_layout, const ConvGeom& g, int out_layout) {
+    if (in_layout != OTTER_HIP_F32_P8 || !h->w_dw_mfma || h->c_pad || h->force_tm == -3 || h->force_tm == -6) return false;
+    if (g.OH < 1 || g.OW < 1 || !dw_f32in_applicable(g, in_layout)) return false;
+    const Epilogue ep = make_epilogue(h, out_layout);
+    return dw_mfma_applicable(g, ep, dw_mfma_epilogue(ep, g.K), h->so_positive);
+}
+
 static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom& g, const Epilogue& ep) {
     if (int8_layout == OTTER_HIP_I8_P8) {
         if (h->w_dw) return 2;
@@ -474,6 +482,15 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
     if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) {
         OHIP_CHECK(run_conv_stem(in, layout_elem(in_layout) == 0, h->w_stem, out, g, make_epilogue(h, out_layout), h->in_scale,
                                  d.in_round_mode, stream));
+        return quantize_twin();
+    }
+
+    // A depthwise 3x3 layer on an fp32 Float8 blob: quantize_to_int8 and the convolution in one launch (no int8 copy of
+    // the blob is written or read back). set_tile(-3, s) keeps the vector-ALU kernels, set_tile(-6, 0) the two launches.
+    if (use_dw_f32in(h, in_layout, g, out_layout)) {
+        const Epilogue ep = make_epilogue(h, out_layout);
+        OHIP_CHECK(run_conv_dw_f32in((const float*)in, h->w_dw_mfma, out, g, ep, dw_mfma_epilogue(ep, g.K), h->in_scale,
+                                     d.in_round_mode, h->force_tm == -2 ? h->force_tn : 0, stream));
         return quantize_twin();
     }
 

@@ -333,6 +333,329 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The same layer straight from an fp32 blob: quantize_to_int8 (Tensor/ConvolutionLayer.cpp:770-775,
+// Tensor/QuantizeX86.cpp:402-490) and the depthwise convolution in ONE launch, for a Float8 input ([N][C/8][H*W][8
+// floats]) of at most 128 columns. As two launches the int8 copy of the blob is written and read back (c1: 103 MB in +
+// 26 MB out + 26 MB back in + 26 MB out); here every fp32 value is read once and nothing but the result is written.
+//
+// A wave owns one channel octet x the full width x a strip of output rows and walks along the input rows. A row of the
+// blob is W x 32 contiguous bytes; lane l of load k takes bytes 16 (64 k + l) .. + 15 of it -- half a pixel, four
+// channels -- so that one load instruction reads 1 KB of whole cache lines (NL = 1..4 loads per row for up to 128
+// columns). Loading a whole pixel per lane instead (two 16-byte loads 32 bytes apart) touches every cache line twice,
+// and the texture addresser, which works per cache line touched, then bounds the kernel: measured 30 us against 24 us.
+// The lane quantizes its four values with the layer's input scale and rounding primitive -- every value once -- and
+// writes the four bytes into the wave's own ring of four LDS lines [pixel + 2][8 B] (pixels -2, -1 and the ones past
+// the row's end are zero: the padding columns). The matrix operand of lane (n, g) for column chunk c -- pixels 64c + 4n -
+// 2 + 2g and + 1 -- is then one aligned 16-byte LDS read per kernel row. LDS instructions of one wave execute in order, so
+// the wave needs no barrier between its lanes' writes and reads. The loads run four input rows ahead of the
+// quantization in a ring of registers; the matrix instructions of a row run under the quantization of the next one, its
+// epilogue follows that. Rows outside the image or past the strip read zero through the buffer descriptor.
+#ifdef OHIP_DWF_STAMPS
+__device__ unsigned long long dwf_stamps[8][64];
+#define DWF_STAMP(i) do { if (stamp_me && lane == 0 && (i) < 64) dwf_stamps[stamp_w][(i)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define DWF_STAMP(i) do { } while (0)
+#endif
+template <int S, int EPI, int NL>
+__global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* __restrict__ x, const int8_t* __restrict__ wa,
+                                                               void* __restrict__ out, ConvGeom g, Epilogue ep,
+                                                               const float* __restrict__ in_scale_p, float in_half,
+                                                               int n_strips, int rps, unsigned in_bytes, unsigned out_bytes) {
+    constexpr int RL = 4, PF = 4;      // LDS lines / register stages per wave
+    constexpr int NCH = (NL + 1) / 2;  // column chunks of 64 pixels (a matrix operand covers 4 x 16 of them)
+    const float in_scale = in_scale_p[0];
+    constexpr int T = S == 1 ? 2 : 1;  // A sets
+    constexpr int PH = 4 / S;          // output pixels per lane column
+    constexpr int LINE = (64 * NCH + 8) * 8;
+    __shared__ __attribute__((aligned(16))) int8_t lds_all[4][RL][LINE];
+    const int C8 = g.C / 8;
+    unsigned bx = blockIdx.x, by = blockIdx.y;
+    {  // consecutive strips of a plane and consecutive planes on one XCD (see conv_dw3x3_mfma_kernel)
+        const unsigned id = by * gridDim.x + bx, total = gridDim.x * gridDim.y, per = total / 8;
+        if (id < per * 8) {
+            const unsigned w = (id % 8) * per + id / 8;
+            bx = w % gridDim.x, by = w / gridDim.x;
+        }
+    }
+    const int o = by % C8, img = by / C8;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int strip = __builtin_amdgcn_readfirstlane(bx * (blockDim.x >> 6) + wave);
+    if (strip >= n_strips) return;  // whole wave
+    const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    int8_t* const lds = &lds_all[wave][0][0];
+#ifdef OHIP_DWF_STAMPS
+    const bool stamp_me = blockIdx.y % 37 == 0 && blockIdx.y / 37 < 2 && blockIdx.x == 0;
+    const int stamp_w = (blockIdx.y / 37) * 4 + wave;
+    int stamp_i = 0;
+#endif
+    DWF_STAMP(stamp_i++);
+
+    // the padding slots of every line: pixels -2, -1 and 32 NL .. 64 NCH + 5 (the row's own pixels from W on are written
+    // as zeros with every row)
+    for (int i = lane; i < (2 + 64 * NCH + 6 - 32 * NL) * RL; i += 64) {
+        constexpr int PADS = 2 + 64 * NCH + 6 - 32 * NL;
+        const int line = i / PADS, k = i % PADS;
+        const int slot = k < 2 ? k : 32 * NL + k;
+        *reinterpret_cast<v2i*>(lds + line * LINE + slot * 8) = v2i{0, 0};
+    }
+
+    // ---- input: this lane's 16 bytes of the row in every load ---------------------------------------------------------
+    const unsigned HW32 = (unsigned)(g.H * g.W) * 32u;
+    const unsigned s_in = (unsigned)(img * C8 + o) * HW32;
+    unsigned v_in[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) v_in[k] = 64 * k + lane < 2 * g.W ? (unsigned)(64 * k + lane) * 16u : DW_OOB;
+    const __amdgpu_buffer_rsrc_t rin = dw_rsrc(x, in_bytes);
+    const int oy0 = strip * rps;
+    const int nrows = min(rps, g.OH - oy0);
+    const int iy0 = oy0 * S - g.ph;
+    const int nq = (nrows - 1) * S + 3;  // input rows this strip reads
+    // Odd strips walk UP: a strip and its neighbour below then read the rows they share at the same end of their walks
+    // (both last, or both first), i.e. at about the same time, and the second reader finds them in the XCD's L2 instead
+    // of fetching them from memory again (the strips of a plane run side by side on one XCD). Walking up only mirrors
+    // the row indices: input row j of the walk is row iy0 + nq - 1 - j, output row r of the walk is the strip's row
+    // nrows - 1 - r, and kernel row dy meets the line that holds walk row 2 - dy (the weights are loaded mirrored).
+    const bool up = (strip & 1) != 0;  // wave-uniform
+    auto issue = [&](int j, v4i (&dst)[NL]) {  // j: input row of the walk
+        const int iy = up ? iy0 + nq - 1 - j : iy0 + j;
+        const bool ok = iy >= 0 && iy < g.H && j < nq;  // wave-uniform
+        // (said to the compiler in so many words: it otherwise loops over the lanes' "different" scalar offsets)
+        const unsigned s_row = (unsigned)__builtin_amdgcn_readfirstlane((int)(ok ? s_in + (unsigned)(iy * g.W) * 32u : 0u));
+#pragma unroll
+        for (int k = 0; k < NL; ++k)
+            dst[k] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)(ok ? v_in[k] : DW_OOB), (int)s_row, 0));
+    };
+    // float2int8 of four values into four bytes (the arithmetic of otter_hip_quantize)
+    auto quant4 = [&](const v4i& f) -> int {
+        int k[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float t = __fmul_rn(__int_as_float(f[e]), in_scale);
+            k[e] = (int)__fadd_rn(t, __builtin_copysignf(in_half, t));  // toward zero, saturating
+        }
+        const ohip_v2s top = {127, 127}, bot = {-127, -127};
+        ohip_v2s a = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[0], k[1]));
+        ohip_v2s b = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[2], k[3]));
+        a = __builtin_elementwise_max(__builtin_elementwise_min(a, top), bot);
+        b = __builtin_elementwise_max(__builtin_elementwise_min(b, top), bot);
+        return (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, a), 0x06040200u);
+    };
+    // lane l of load k holds pixel 32 k + l / 2, channels 4 (l & 1) ..: byte (pixel + 2) * 8 + 4 (l & 1) = 16 + 256 k + 4 l
+    auto quant_write = [&](int line, const v4i (&src)[NL]) {
+#pragma unroll
+        for (int k = 0; k < NL; ++k) *reinterpret_cast<int*>(lds + line * LINE + 16 + 256 * k + 4 * lane) = quant4(src[k]);
+    };
+
+    v4i a[3][T];  // a[k]: the kernel row that meets the k-th of an output row's three lines
+    {
+        const v4i* ap = reinterpret_cast<const v4i*>(wa) + (size_t)o * 3 * T * 64 + lane;
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+#pragma unroll
+            for (int t = 0; t < T; ++t) a[k][t] = ap[((up ? 2 - k : k) * T + t) * 64];
+    }
+    // (requested before any input row: loads return in order, so the wait for these in front of the first matrix
+    // instruction -- which sits inside the loop and is executed on every pass -- then never reaches past a row's loads)
+    __builtin_amdgcn_sched_barrier(0);
+
+    v4i ld[PF][NL];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) issue(j, ld[j]);
+
+    // ---- epilogue constants (as in conv_dw3x3_mfma_kernel) -----------------------------------------------------------
+    const int ch = 8 * o + (S == 1 ? 0 : 4 * (q & 1));
+    v4i si[T], bi[T], so[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        si[t] = *reinterpret_cast<const v4i*>(ep.scale_in + ch + 4 * t);
+        bi[t] = *reinterpret_cast<const v4i*>(ep.bias + ch + 4 * t);
+        so[t] = v4i{0, 0, 0, 0};
+        if constexpr (EPI != EPI_F32_P4 && EPI != EPI_F32_P8) so[t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
+    }
+    unsigned qh[T][2] = {};
+    if constexpr (EPI == EPI_I8_P8_NONNEG) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            qh[t][0] = dw_clamp_pair(ep, so[t][0], so[t][1]);
+            qh[t][1] = dw_clamp_pair(ep, so[t][2], so[t][3]);
+        }
+    }
+    // ---- output: this lane's pixel of the row in every column chunk --------------------------------------------------
+    const unsigned OHW = (unsigned)(g.OH * g.OW);
+    unsigned v_out[NCH], s_out, row_bytes;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int ox = PH * (16 * c + n) + (S == 1 ? q : (q >> 1));
+        const bool st_ok = ox < g.OW;
+        if constexpr (EPI == EPI_F32_P4)
+            v_out[c] = st_ok ? (S == 1 ? 0u : (unsigned)(q & 1)) * OHW * 16u + (unsigned)ox * 16u : DW_OOB;
+        else if constexpr (EPI == EPI_F32_P8)
+            v_out[c] = st_ok ? (unsigned)ox * 32u + (S == 1 ? 0u : (unsigned)(q & 1) * 16u) : DW_OOB;
+        else
+            v_out[c] = st_ok ? (unsigned)ox * 8u + (S == 1 ? 0u : (unsigned)(q & 1) * 4u) : DW_OOB;
+    }
+    if constexpr (EPI == EPI_F32_P4) s_out = (unsigned)(img * (g.C / 4) + 2 * o) * OHW * 16u, row_bytes = (unsigned)g.OW * 16u;
+    else if constexpr (EPI == EPI_F32_P8) s_out = (unsigned)(img * C8 + o) * OHW * 32u, row_bytes = (unsigned)g.OW * 32u;
+    else s_out = (unsigned)(img * C8 + o) * OHW * 8u, row_bytes = (unsigned)g.OW * 8u;
+    const __amdgpu_buffer_rsrc_t rout = dw_rsrc(out, out_bytes);
+
+    v4i cur[NCH][T];
+    auto epilogue_store = [&](int r) {  // output row r of the walk, from cur
+        const unsigned s_row =
+            (unsigned)__builtin_amdgcn_readfirstlane((int)(s_out + (unsigned)(oy0 + (up ? nrows - 1 - r : r)) * row_bytes));
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P8) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    const v4i res = dw_dequant4(ep, cur[c][t], si[t], bi[t]);
+                    const unsigned vo_t = (t == 0 || v_out[c] == DW_OOB) ? v_out[c] : v_out[c] + (EPI == EPI_F32_P4 ? OHW * 16u : 16u);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, res), rout, (int)vo_t, (int)s_row, 0);
+                }
+            } else {
+                constexpr bool NONNEG = EPI == EPI_I8_P8_NONNEG;
+                if constexpr (S == 1) {
+                    v2i w2;
+                    w2[0] = (int)dw_requant4<NONNEG>(ep, cur[c][0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                    w2[1] = (int)dw_requant4<NONNEG>(ep, cur[c][T - 1], si[T - 1], bi[T - 1], so[T - 1], qh[T - 1][0], qh[T - 1][1]);
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, w2), rout, (int)v_out[c], (int)s_row, 0);
+                } else {
+                    const unsigned w1 = dw_requant4<NONNEG>(ep, cur[c][0], si[0], bi[0], so[0], qh[0][0], qh[0][1]);
+                    __builtin_amdgcn_raw_buffer_store_b32(w1, rout, (int)v_out[c], (int)s_row, 0);
+                }
+            }
+        }
+    };
+    auto row_mfma = [&](int line0) {  // the three input rows of an output row sit in lines line0, +1, +2 (mod RL)
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            v4i b[3];
+#pragma unroll
+            for (int dy = 0; dy < 3; ++dy)
+                b[dy] = *reinterpret_cast<const v4i*>(lds + ((line0 + dy) % RL) * LINE + (64 * c + 4 * n + 2 * q) * 8);
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                cur[c][t] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int dy = 0; dy < 3; ++dy) cur[c][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[dy][t], b[dy], cur[c][t], 0, 0, 0);
+            }
+        }
+    };
+
+    // Input row j of the walk sits in line and register stage j % 4 and completes output row (j - 2) / S when that is
+    // whole. Rows 0..2 (everything up to the first output row) run in front of the loop, so that every pass of the loop
+    // issues the same loads and stores on every path: the waits for a row's loads are counted back from the youngest
+    // request, and a path with fewer requests would pull them (and with them the loads in flight) closer.
+    // (where the rows in front of the loop have no output row to store yet they issue stores that go nowhere -- an
+    // out-of-range offset -- so that the count of requests behind a row's loads is the loop's own from the first pass on)
+    auto no_store = [&]() {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P8) {
+#pragma unroll
+                for (int t = 0; t < T; ++t)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, v4i{0, 0, 0, 0}), rout, (int)DW_OOB, 0, 0);
+            } else if constexpr (S == 1) {
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, v2i{0, 0}), rout, (int)DW_OOB, 0, 0);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b32(0u, rout, (int)DW_OOB, 0, 0);
+            }
+        }
+    };
+    auto input_row = [&](int j, int jj, bool store_prev) {  // jj = j modulo 4; both a compile-time constant at every call
+        quant_write(jj % RL, ld[jj % PF]);
+        issue(j + PF, ld[jj % PF]);
+        if ((jj - 2 + 4) % S == 0) {
+            if (store_prev) epilogue_store((j - 2) / S - 1);
+            else no_store();
+            row_mfma((jj - 2 + 4) % RL);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        DWF_STAMP(stamp_i++);
+    };
+    no_store();
+    input_row(0, 0, false);
+    input_row(1, 1, false);
+    input_row(2, 2, false);
+    // (eight rows per pass: the waits the compiler places in the first rows of a pass reach a row or two further back
+    // than the ring needs, so the passes are long)
+    constexpr int UNR = 8;
+    const int steps = (nq - 3) / UNR;
+    int jb = 3;
+    for (int st = 0; st < steps; ++st, jb += UNR) {
+#pragma unroll
+        for (int i = 0; i < UNR; ++i) input_row(jb + i, 3 + i, true);
+    }
+#pragma unroll
+    for (int i = 0; i < UNR - 1; ++i)
+        if (jb + i < nq) input_row(jb + i, 3 + i, true);  // wave-uniform
+    epilogue_store(nrows - 1);
+    DWF_STAMP(stamp_i++);
+}
+#ifdef OHIP_DWF_STAMPS
+extern "C" int otter_hip_debug_dwf_stamps(unsigned long long* out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(dwf_stamps), sizeof(dwf_stamps));
+}
+#endif
+
+// true when the fused fp32 -> depthwise launch takes this layer and blob (Float8 input; the caller has checked
+// dw_mfma_applicable)
+bool dw_f32in_applicable(const ConvGeom& g, int in_layout) {
+    if (in_layout != OTTER_HIP_F32_P8 || g.kh != 3 || g.kw != 3) return false;
+    if (g.W > 128 || g.W < 17 || g.C % 8 != 0) return false;
+    if ((size_t)g.N * g.C * g.H * g.W * 4 >= ((size_t)1 << 31)) return false;  // 32-bit buffer offsets
+    return (long)g.N * (g.C / 8) <= 65535;
+}
+
+hipError_t run_conv_dw_f32in(const float* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
+                             const float* in_scale, int in_round_mode, int strip_rows, hipStream_t stream) {
+    if (g.N == 0 || g.OH * g.OW == 0) return hipSuccess;
+    const int C8 = g.C / 8;
+    const long planes = (long)g.N * C8;
+    if (planes > 65535) return hipErrorInvalidValue;
+    // strips of equal height, about two waves per SIMD over the chip (as in run_conv_dw_mfma)
+    int rps;
+    if (strip_rows > 0) {
+        rps = std::min(strip_rows, g.OH);
+    } else {
+        int ns = 1;
+        while (ns < g.OH && ns * planes < 2048) ++ns;
+        rps = (g.OH + ns - 1) / ns;
+    }
+    const int n_strips = (g.OH + rps - 1) / rps;
+    const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
+    const dim3 grid((unsigned)(n_strips / wpb), (unsigned)planes), block(64 * wpb);
+    const float in_half = in_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W * 4);
+    const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 || epi == EPI_F32_P8 ? 4 : 1));
+#define OHIP_DWF_L(S_, E_, L_)                                                                                           \
+    hipLaunchKernelGGL((conv_dw3x3_f32in_kernel<S_, E_, L_>), grid, block, 0, stream, x, wa, out, g, ep, in_scale, in_half, \
+                       n_strips, rps, in_bytes, out_bytes)
+#define OHIP_DWF_N(S_, E_)                       \
+    do {                                         \
+        switch ((g.W + 31) / 32) {               \
+        case 1: OHIP_DWF_L(S_, E_, 1); break;    \
+        case 2: OHIP_DWF_L(S_, E_, 2); break;    \
+        case 3: OHIP_DWF_L(S_, E_, 3); break;    \
+        default: OHIP_DWF_L(S_, E_, 4); break;   \
+        }                                        \
+    } while (0)
+#define OHIP_DWF_E(S_)                                                  \
+    do {                                                                \
+        if (epi == EPI_I8_P8_NONNEG) OHIP_DWF_N(S_, EPI_I8_P8_NONNEG);  \
+        else if (epi == EPI_I8_P8) OHIP_DWF_N(S_, EPI_I8_P8);           \
+        else if (epi == EPI_F32_P8) OHIP_DWF_N(S_, EPI_F32_P8);         \
+        else OHIP_DWF_N(S_, EPI_F32_P4);                                \
+    } while (0)
+    if (g.sh == 1) OHIP_DWF_E(1);
+    else OHIP_DWF_E(2);
+#undef OHIP_DWF_E
+#undef OHIP_DWF_N
+#undef OHIP_DWF_L
+    return hipGetLastError();
+}
+
 // the epilogue code of a depthwise layer: the common rule, plus fp32 output in the depthwise default layout Float8
 int dw_mfma_epilogue(const Epilogue& ep, int K) {
     const int epi = pick_epilogue(ep, K);

@@ -62,6 +62,10 @@ bool dw_mfma_window_fits(int ks, int stride, int pad_w);
 void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks, int8_t* dst);
 int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
+// the same layer straight from an fp32 Float8 blob (quantize + depthwise convolution in one launch)
+bool dw_f32in_applicable(const ConvGeom& g, int in_layout);
+hipError_t run_conv_dw_f32in(const float* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
+                             const float* in_scale, int in_round_mode, int strip_rows, hipStream_t stream);
 hipError_t run_conv_dw_mfma(const int8_t* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
                             int strip_shift, hipStream_t stream);
 size_t dw_packed_weight_bytes(int C, int kh, int kw);

@@ -200,6 +200,9 @@ typedef float ip_v4f __attribute__((ext_vector_type(4)));
 constexpr int IPM_WAVES = 16;  // the inputs are dealt to 16 waves: a wave requests all its loads at once (one memory latency)
 // A workgroup owns 16 outputs x 16 rows of x: enough workgroups to put every compute unit's memory pipeline to work
 // (1000 outputs x 64 rows: 252 of them), each weight row read once per 16 rows of x.
+// ALIGNED: both pointers are multiples of 16 bytes (one 16-byte load per operand); otherwise the same four floats come
+// from four 4-byte loads -- the arithmetic, and so every bit of the result, is the same either way.
+template <bool ALIGNED>
 __global__ void __launch_bounds__(64 * IPM_WAVES) inner_product_mfma_kernel(const float* __restrict__ x,
                                                                             const float* __restrict__ w,
                                                                             const float* __restrict__ b, float* __restrict__ y,
@@ -214,8 +217,14 @@ __global__ void __launch_bounds__(64 * IPM_WAVES) inner_product_mfma_kernel(cons
     const int steps = IN / 16;
 #pragma unroll 5
     for (int st = wave; st < steps; st += IPM_WAVES) {
-        const ip_v4f a = *reinterpret_cast<const ip_v4f*>(wr + 16 * st);
-        const ip_v4f bv = *reinterpret_cast<const ip_v4f*>(xr + 16 * st);
+        ip_v4f a, bv;
+        if constexpr (ALIGNED) {
+            a = *reinterpret_cast<const ip_v4f*>(wr + 16 * st);
+            bv = *reinterpret_cast<const ip_v4f*>(xr + 16 * st);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) a[m] = wr[16 * st + m], bv[m] = xr[16 * st + m];
+        }
 #pragma unroll
         for (int m = 0; m < 4; ++m) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m], bv[m], acc, 0, 0, 0);
     }
@@ -242,10 +251,15 @@ __global__ void __launch_bounds__(64 * IPM_WAVES) inner_product_mfma_kernel(cons
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream) {
     if (N * OUT == 0) return hipSuccess;
-    // (the choice must not depend on N: a row's result is then the same bits whatever batch it sits in)
-    if (IN % 16 == 0 && IN >= 64 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {
-        hipLaunchKernelGGL(inner_product_mfma_kernel, dim3((OUT + 15) / 16, (N + 15) / 16), dim3(64 * IPM_WAVES), 0, stream, x, w, b, y,
-                           N, IN, OUT);
+    // The choice depends on the layer's shape only -- not on N (a row's result is then the same bits whatever batch it
+    // sits in) and not on where the buffers lie (the two kernels add in different orders, so the same call must not give
+    // different bits from one allocation to the next); alignment only picks how the matrix-core kernel loads.
+    if (IN % 16 == 0 && IN >= 64) {
+        const dim3 grid((OUT + 15) / 16, (N + 15) / 16), block(64 * IPM_WAVES);
+        if ((((uintptr_t)x | (uintptr_t)w) & 15) == 0)
+            hipLaunchKernelGGL(inner_product_mfma_kernel<true>, grid, block, 0, stream, x, w, b, y, N, IN, OUT);
+        else
+            hipLaunchKernelGGL(inner_product_mfma_kernel<false>, grid, block, 0, stream, x, w, b, y, N, IN, OUT);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(inner_product_kernel, dim3((OUT + IP_OB - 1) / IP_OB, (N + IP_NB - 1) / IP_NB), dim3(256), 0, stream,

@@ -175,28 +175,6 @@ def build_net(hostnet, layers, params, batch, hw, num_classes=1000):
     return net
 
 
-def oracle_forward(oracle, layers, params, x, upto=None):
-    """The same network on the CPU oracle, layer by layer (ConvolutionLayer::forward_int8 semantics)."""
-    blobs = {"data": x}
-    for l in layers:
-        if l["kind"] == "conv":
-            p = params[l["name"]]
-            blobs[l["name"]] = oracle.conv_layer_forward(
-                blobs[l["input"]], p["wq"], p["ws"], p["in_scale"], stride=(l["stride"],) * 2, pad=(l["k"] // 2,) * 2,
-                groups=l["groups"], bias=p["bias"], top_scale=p["top_scale"], int8_out=l["int8_out"],
-                act_type=_act_id(l["act"]))
-        elif l["kind"] == "add":
-            blobs[l["name"]] = blobs[l["a"]] + blobs[l["b"]]
-        elif l["kind"] == "pool":
-            blobs[l["name"]] = oracle.global_avgpool(blobs[l["input"]])
-        elif l["kind"] == "fc":
-            p = params[l["name"]]
-            blobs[l["name"]] = oracle.inner_product(blobs[l["input"]].reshape(x.shape[0], -1), p["w"], p["bias"])
-        if upto == l["name"]:
-            break
-    return blobs
-
-
 def build_bench(hip, capi, rng, batch=64, hw=224, calib=32):
     from . import hostnet
     layers = describe()

@@ -53,3 +53,27 @@ def run_conv(hip, oracle, x, wq, w_scales, in_scale, *, stride=1, pad=0, dil=1, 
     res = capi.unpack_np(out.cpu().numpy(), capi.layout_pack(out_layout), (n, K, oh, ow))
     conv.close()
     return res, kind
+
+
+def mobilenet_oracle_forward(oracle, layers, params, x, upto=None):
+    """The MobileNetV2-style network of tensor_amd.mobilenet on the CPU oracle, layer by layer
+    (ConvolutionLayer::forward_int8 semantics, Tensor/ConvolutionLayer.cpp:754-847). Returns every blob by name."""
+    from tensor_amd.mobilenet import _act_id
+    blobs = {"data": x}
+    for l in layers:
+        if l["kind"] == "conv":
+            p = params[l["name"]]
+            blobs[l["name"]] = oracle.conv_layer_forward(
+                blobs[l["input"]], p["wq"], p["ws"], p["in_scale"], stride=(l["stride"],) * 2, pad=(l["k"] // 2,) * 2,
+                groups=l["groups"], bias=p["bias"], top_scale=p["top_scale"], int8_out=l["int8_out"],
+                act_type=_act_id(l["act"]))
+        elif l["kind"] == "add":
+            blobs[l["name"]] = blobs[l["a"]] + blobs[l["b"]]
+        elif l["kind"] == "pool":
+            blobs[l["name"]] = oracle.global_avgpool(blobs[l["input"]])
+        elif l["kind"] == "fc":
+            p = params[l["name"]]
+            blobs[l["name"]] = oracle.inner_product(blobs[l["input"]].reshape(x.shape[0], -1), p["w"], p["bias"])
+        if upto == l["name"]:
+            break
+    return blobs

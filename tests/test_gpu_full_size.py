@@ -12,7 +12,9 @@ import numpy as np
 import pytest
 
 from tensor_amd import capi
-from gpu_util import run_conv
+from gpu_util import run_conv, mobilenet_oracle_forward
+
+FP32_RTOL = 1e-5  # the bar for fp32 results
 
 pytestmark = pytest.mark.gpu
 
@@ -232,6 +234,27 @@ def test_c4_as_stated_batch_64_at_224(hip, oracle):
     for n in (0, 40, batch - 1):
         np.testing.assert_array_equal(net1.run("data", x[n:n + 1], "fc").reshape(1, -1), logits[n:n + 1])
         np.testing.assert_array_equal(net1.run("data", x[n:n + 1], "b7_dw"), mid[n:n + 1])
-    want = mobilenet.oracle_forward(oracle, layers, params, x[:1])
+    want = mobilenet_oracle_forward(oracle, layers, params, x[:1])
     np.testing.assert_array_equal(mid[:1], want["b7_dw"])
-    np.testing.assert_allclose(logits[:1], want["fc"], rtol=1e-4, atol=1e-5)
+    # Behind the blocks that run as one launch under the DEFAULT policy at this size (the 28x28, 14x14 and 7x7 blocks,
+    # the 7x7 ones with a band's expanded channels dealt to several workgroups whose partial sums meet in memory): the
+    # last block's int8 result bit for bit, the head convolution's fp32 result and the pooled features at 1e-5.
+    blocks = hostnet.block_forward_count()
+    prj = net.run("data", x, "b16_project")
+    assert hostnet.block_forward_count() >= blocks + 11  # (asking for a block's own result keeps it one launch)
+    assert prj.dtype == np.int8
+    np.testing.assert_array_equal(prj[:1], want["b16_project"])
+    np.testing.assert_array_equal(prj[40:41], net1.run("data", x[40:41], "b16_project"))
+    np.testing.assert_allclose(net.run("data", x, "head")[:1], want["head"], rtol=FP32_RTOL, atol=1e-30)
+    pooled = net.run("data", x, "pool").reshape(batch, -1)
+    np.testing.assert_allclose(pooled[:1], want["pool"].reshape(1, -1), rtol=FP32_RTOL, atol=1e-30)
+    # The logits are 1280-term fp32 dot products whose terms cancel; the GPU adds them in another order than the oracle
+    # (sixteen partial sums on the matrix cores), so the bound that holds is relative to the sum of the terms' magnitudes,
+    # not to the (possibly much smaller) result: |got - exact| <= 1e-5 * (|w| . |x| + |b|), exact in float64 from the
+    # GPU's own pooled features; and the oracle's logits lie inside the same bound.
+    fc = params["fc"]
+    w64, p64 = fc["w"].astype(np.float64), pooled[:1].astype(np.float64)
+    exact = p64 @ w64.T + fc["bias"].astype(np.float64)
+    bound = FP32_RTOL * (np.abs(p64) @ np.abs(w64).T + np.abs(fc["bias"].astype(np.float64)))
+    assert (np.abs(logits[:1] - exact) <= bound).all()
+    assert (np.abs(want["fc"] - exact) <= 2 * bound).all()

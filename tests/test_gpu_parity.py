@@ -626,6 +626,58 @@ def test_forward_residual_equals_forward_then_add(hip, oracle, C, K, k, s, p, g,
     conv.close()
 
 
+@pytest.mark.parametrize("s", [1, 2])
+def test_depthwise3x3_from_an_fp32_blob_in_one_launch(hip, oracle, s):
+    """A depthwise 3x3 layer on an fp32 Float8 blob of 17..128 columns runs quantize_to_int8 and the convolution as ONE
+    launch (every value quantized once, through the wave's LDS lines). Against the oracle's layer, and bit for bit
+    against the two launches (set_tile(-6, 0)): both column-chunk counts, odd widths, widths that end inside and on a
+    chunk, ragged and forced strips (one row per strip, more rows than the image), pad 0, batch > 1, values on rounding
+    ties and beyond saturation, both rounding primitives, every fast epilogue."""
+    rng = np.random.default_rng(300 + s)
+    shapes = [(16, 3, 19, 70, 1), (8, 2, 13, 17, 1), (24, 2, 8, 64, 0), (8, 1, 33, 65, 1), (8, 2, 9, 128, 1), (16, 1, 30, 112, 1),
+              (8, 2, 5, 33, 0), (32, 2, 3, 40, 1)]
+    for i, (C, N, H, W, p) in enumerate(shapes):
+        x, wq, ws, bias = _rand_problem(rng, C, C, 3, C, N, H, W, in_i8=False)
+        in_scale = np.float32(100.0)
+        # some values exactly on a tie of the quantization, on the value the two primitives round differently, and
+        # beyond saturation
+        flat = x.reshape(-1)
+        flat[::7] = (rng.integers(-140, 141, flat[::7].size) + 0.5) / in_scale
+        flat[3::11] = np.nextafter(np.float32(0.5), np.float32(0)) / in_scale * rng.choice([-1, 1], flat[3::11].size)
+        for act, int8_out, tile in ((3, True, None), (0, True, (-2, 1)), (1, False, (-2, 200)), (2, True, (-2, 5))):
+            kw = dict(stride=(s, s), pad=(p, p), groups=C, bias=bias, top_scale=9.0, int8_out=int8_out, act_type=act,
+                      act_params=[0.1] if act == 2 else None)
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, **kw)
+            args = dict(stride=s, pad=p, groups=C, bias=bias, top_scale=9.0, act=act, act_p0=0.1,
+                        out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, tile=tile, **args)
+            two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **args)
+            assert kind == 2
+            what = str((C, N, H, W, p, act, int8_out, tile))
+            assert out.tobytes() == two.tobytes(), what
+            if int8_out:
+                np.testing.assert_array_equal(out, want, err_msg=what)
+            else:
+                assert_f32_close(out, want)
+    # the scalar rounding primitive on the input side (what an unpacked net would ask for) through the same launch; with a
+    # power-of-two input scale a fifth of the values land exactly on the one float the two primitives round differently
+    x, wq, ws, bias = _rand_problem(rng, 8, 8, 3, 8, 2, 9, 40, in_i8=False)
+    x.reshape(-1)[::5] = np.nextafter(np.float32(0.5), np.float32(0)) / np.float32(128.0)
+    si = (np.float32(1.0) / (np.float32(128.0) * ws)).astype(np.float32)
+    outs = {}
+    for mode in (capi.ROUND_SSE, capi.ROUND_EXACT):
+        conv = hip.conv(wq=wq, scale_in=si, bias=bias, in_scale=128.0, out_scale=[900.0], stride=(s, s), pad=(1, 1), groups=8,
+                        act=0, out_kind=capi.OUT_I8, in_round=mode)
+        xq = oracle.quantize(x, [np.float32(128.0)], mode)
+        want = oracle.requantize(oracle.conv_int32(xq, wq, (s, s), (1, 1), (1, 1), 8), si, [900.0], bias, 0, None, capi.ROUND_SSE)
+        got = conv.forward(hip.to_device(capi.pack_np(x, 8)), capi.F32_P8, 2, 9, 40, capi.I8_P8)
+        oh, ow = conv.out_hw(9, 40)
+        outs[mode] = capi.unpack_np(got.cpu().numpy(), 8, (2, 8, oh, ow))
+        np.testing.assert_array_equal(outs[mode], want)
+        conv.close()
+    assert (outs[capi.ROUND_SSE] != outs[capi.ROUND_EXACT]).any()
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

@@ -115,10 +115,10 @@ def test_one_net_two_extractors_in_two_threads(hip, oracle):
     its shortcut sum that goes through the block entry point), two threads that each run their own passes over it on
     their own input: each gets what a single-threaded pass over that input gives."""
     rng = np.random.default_rng(92)
-    N, C, E, H, W = 4, 64, 384, 14, 14
+    N, C0, C, E, H, W = 4, 16, 64, 384, 14, 14
     net = hostnet.Net()
-    net.add_layer(type="Input", name="data", batchsize=N, channel=C, height=H, width=W)
-    names = ["c1", "c2", "c3"]
+    net.add_layer(type="Input", name="data", batchsize=N, channel=C0, height=H, width=W)
+    names = ["c0", "c1", "c2", "c3"]  # c0 reads the fp32 image and changes the channel count; c1..c3 are the run
     for nm in names:
         net.add_layer(type="Convolution", name=nm, out_channels=C, kernel=3, padding=1, int8_scale_term=102, activation="Relu")
     net.add_layer(type="Convolution", name="stem", out_channels=C, kernel=1, int8_scale_term=2)
@@ -131,7 +131,7 @@ def test_one_net_two_extractors_in_two_threads(hip, oracle):
     net.compile()
     scale = np.float32(127.0)
     for nm in names:
-        w, s = _qweights(rng, C, C, 3)
+        w, s = _qweights(rng, C, C0 if nm == "c0" else C, 3)
         top = np.float32(rng.uniform(15, 30))
         net.set_conv(nm, w, rng.normal(0, 0.05, C).astype(np.float32), s, scale, top)
         scale = top
@@ -147,7 +147,7 @@ def test_one_net_two_extractors_in_two_threads(hip, oracle):
     always = hip.conv_block_set_always(1)
     old_tiles = hip.conv_chain_set_min_tiles(0)
     try:
-        xs = [rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32) for _ in range(2)]
+        xs = [rng.uniform(-1, 1, (N, C0, H, W)).astype(np.float32) for _ in range(2)]
         chains, blocks = hostnet.chain_forward_count(), hostnet.block_forward_count()
         wants = [net.run("data", x, "add") for x in xs]
         assert hostnet.chain_forward_count() > chains and hostnet.block_forward_count() > blocks  # both entry points in play

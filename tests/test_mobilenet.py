@@ -2,6 +2,7 @@
 import numpy as np
 import pytest
 
+from gpu_util import mobilenet_oracle_forward
 from tensor_amd import capi, hostnet, mobilenet
 
 
@@ -26,7 +27,7 @@ def test_network_matches_oracle_layer_by_layer(hip, oracle):
     mobilenet.calibrate(hip, capi, layers, params, rng.uniform(0, 1, (4, 3, hw, hw)).astype(np.float32))
     net = mobilenet.build_net(hostnet, layers, params, batch, hw, num_classes=50)
     x = rng.uniform(0, 1, (batch, 3, hw, hw)).astype(np.float32)
-    want = mobilenet.oracle_forward(oracle, layers, params, x)
+    want = mobilenet_oracle_forward(oracle, layers, params, x)
     for name in ("stem", "b0_project", "b1_dw", "b2_add", "b5_project", "b9_add", "b16_project", "head"):
         got = net.run("data", x, name)
         if got.dtype == np.int8:
@@ -49,7 +50,7 @@ def test_network_with_blocks_as_single_launches(hip, oracle):
     mobilenet.calibrate(hip, capi, layers, params, rng.uniform(0, 1, (4, 3, hw, hw)).astype(np.float32))
     net = mobilenet.build_net(hostnet, layers, params, batch, hw, num_classes=50)
     x = rng.uniform(0, 1, (batch, 3, hw, hw)).astype(np.float32)
-    want = mobilenet.oracle_forward(oracle, layers, params, x)
+    want = mobilenet_oracle_forward(oracle, layers, params, x)
     names = ("b2_add", "b5_add", "b9_add", "b10_project", "b12_add", "b15_add", "b16_project", "head")
     plain = {name: net.run("data", x, name) for name in names}
     before = hip.conv_block_set_always(1)

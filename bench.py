@@ -154,11 +154,12 @@ def build_c3(hip, capi, rng):
                 x=x, params=params, shape=(N, C, H, W))
 
 
-def build_c1(hip, capi, rng, stride):
+def build_c1(hip, capi, rng, stride, variant=""):
     """configs[1]: depthwise 3x3 p1 on 8x256x112x112 fp32, bias, ReLU6, requantize to int8 with 127/6. The step is the
     configuration as stated: the layer on the fp32 Float8 blob, ONE launch that quantizes on the way in
     (conv_dw3x3_f32in_kernel). The layer on an int8 blob (what a depthwise layer inside a network sees) and the
-    standalone quantize pass are timed beside it."""
+    standalone quantize pass are timed beside it. variant "i8": the step is the layer on the int8 blob (matrix-core
+    kernel); "valu": the same on the vector-ALU kernels (v_dot4_i32_i8), kept for comparison."""
     N, C, H, W = 8, 256, 112, 112
     x = rng.uniform(-1, 1, (N, C, H, W)).astype(np.float32)
     wq, ws = quantize_weights(rng.normal(0, 0.1, (C, 1, 3, 3)).astype(np.float32))
@@ -190,6 +191,18 @@ def build_c1(hip, capi, rng, stride):
     xq2 = [hip.empty(in_b, np.int8) for _ in range(n_dom)]
     q_cold = [lambda i=i: hip.quantize(xds[i], capi.F32_P8, (N, C, H, W), scale_dev, capi.ROUND_SSE, capi.I8_P8, dst=xq2[i])
               for i in range(n_dom)]
+    if variant:
+        if variant == "valu":
+            conv.set_tile(-3, 0)
+        fn = lambda: conv.forward(xq, capi.I8_P8, N, H, W, capi.I8_P8, out=out)  # noqa: E731
+        kern = "conv_dw3x3_mfma_kernel (matrix cores)" if variant == "i8" else "conv_dw3x3_i8_kernel (vector ALU, v_dot4_i32_i8)"
+        return dict(name="c1s%d%s" % (stride, variant), step=fn, dom_fn_cold=i8_cold, ops=2.0 * N * C * 9 * oh * ow, launches=1,
+                    bytes=in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=in_b + out_b, bound="hbm",
+                    workload="depthwise int8 3x3 s%d p1 on an int8 Byte8 blob 8x256x112x112 -> conv + bias + ReLU6 + "
+                             "requantize -> int8" % stride,
+                    dom_kernel=kern + ": depthwise 3x3 s%d + requantize (int8 in -> int8 out)" % stride, dom_fn=fn,
+                    x=x, params=[dict(wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale))],
+                    shape=(N, C, H, W), stride=stride, int8_in=True)
     return dict(name="c1s%d" % stride, step=step, dom_fn_cold=dom_cold, ops=2.0 * N * C * 9 * oh * ow, launches=1,
                 bytes=4 * in_b + out_b, dom_ops=2.0 * N * C * 9 * oh * ow, dom_bytes=4 * in_b + out_b, bound="hbm",
                 workload="depthwise int8 3x3 s%d p1, 8x256x112x112 fp32 in -> quantize + conv + bias + ReLU6 + requantize "
@@ -755,6 +768,8 @@ def main():
         return
     builders = {"c3": lambda r: build_c3(hip, capi, r), "c1s1": lambda r: build_c1(hip, capi, r, 1),
                 "c1s2": lambda r: build_c1(hip, capi, r, 2), "c2": lambda r: build_c2(hip, capi, r),
+                "c1s1i8": lambda r: build_c1(hip, capi, r, 1, "i8"), "c1s2i8": lambda r: build_c1(hip, capi, r, 2, "i8"),
+                "c1s1valu": lambda r: build_c1(hip, capi, r, 1, "valu"), "c1s2valu": lambda r: build_c1(hip, capi, r, 2, "valu"),
                 "c0": lambda r: build_c0(hip, capi, r), "copy": lambda r: build_copy(hip, capi, r),
                 "c2i8": lambda r: build_c2(hip, capi, r, int8_out=True), "c0n64": lambda r: build_c0(hip, capi, r, batch=64)}
     try:

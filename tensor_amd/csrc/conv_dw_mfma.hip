@@ -428,6 +428,9 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
     };
     // float2int8 of four values into four bytes (the arithmetic of otter_hip_quantize)
     auto quant4 = [&](const v4i& f) -> int {
+#ifdef OHIP_DWF_NOQUANT
+        return f[0] ^ f[1] ^ f[2] ^ f[3];
+#endif
         int k[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -549,17 +552,18 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
     // request, and a path with fewer requests would pull them (and with them the loads in flight) closer.
     // (where the rows in front of the loop have no output row to store yet they issue stores that go nowhere -- an
     // out-of-range offset -- so that the count of requests behind a row's loads is the loop's own from the first pass on)
-    auto no_store = [&]() {
+    auto no_store = [&](int i) {  // (a different nowhere each time, or the compiler drops all but the last as dead stores)
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
+            const int nowhere = (int)(DW_OOB + 256u * (unsigned)i + 64u * (unsigned)c);
             if constexpr (EPI == EPI_F32_P4 || EPI == EPI_F32_P8) {
 #pragma unroll
                 for (int t = 0; t < T; ++t)
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, v4i{0, 0, 0, 0}), rout, (int)DW_OOB, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, v4i{0, 0, 0, 0}), rout, nowhere + 16 * t, 0, 0);
             } else if constexpr (S == 1) {
-                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, v2i{0, 0}), rout, (int)DW_OOB, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, v2i{0, 0}), rout, nowhere, 0, 0);
             } else {
-                __builtin_amdgcn_raw_buffer_store_b32(0u, rout, (int)DW_OOB, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(0u, rout, nowhere, 0, 0);
             }
         }
     };
@@ -568,13 +572,13 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
         issue(j + PF, ld[jj % PF]);
         if ((jj - 2 + 4) % S == 0) {
             if (store_prev) epilogue_store((j - 2) / S - 1);
-            else no_store();
+            else no_store(j);
             row_mfma((jj - 2 + 4) % RL);
         }
         __builtin_amdgcn_sched_barrier(0);
         DWF_STAMP(stamp_i++);
     };
-    no_store();
+    no_store(3);
     input_row(0, 0, false);
     input_row(1, 1, false);
     input_row(2, 2, false);
@@ -627,10 +631,17 @@ hipError_t run_conv_dw_f32in(const float* x, const int8_t* wa, void* out, const 
     const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);
     const dim3 grid((unsigned)(n_strips / wpb), (unsigned)planes), block(64 * wpb);
     const float in_half = in_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+    // A grid of a few workgroups per CU is resident all at once, and the dispatcher is free to give one CU three of them
+    // and another one: the kernel then lasts as long as the fullest CU. Reserving a share of the CU's 160 KB of LDS per
+    // workgroup (beyond the 17 KB of lines the kernel uses) caps the workgroups per CU at the even share.
+    const long wgs = (long)grid.x * grid.y, per_cu = (wgs + 255) / 256;
+    unsigned lds_reserve = 0;
+    if (wpb == 4 && per_cu >= 2 && per_cu <= 3) lds_reserve = (unsigned)(160 * 1024 / per_cu - 18 * 1024) / 1024 * 1024;
+    if (lds_reserve > 46 * 1024) lds_reserve = 46 * 1024;  // static + dynamic stay within the default 64 KB limit
     const unsigned in_bytes = (unsigned)((size_t)g.N * g.C * g.H * g.W * 4);
     const unsigned out_bytes = (unsigned)((size_t)g.N * g.K * g.OH * g.OW * (epi == EPI_F32_P4 || epi == EPI_F32_P8 ? 4 : 1));
 #define OHIP_DWF_L(S_, E_, L_)                                                                                           \
-    hipLaunchKernelGGL((conv_dw3x3_f32in_kernel<S_, E_, L_>), grid, block, 0, stream, x, wa, out, g, ep, in_scale, in_half, \
+    hipLaunchKernelGGL((conv_dw3x3_f32in_kernel<S_, E_, L_>), grid, block, lds_reserve, stream, x, wa, out, g, ep, in_scale, in_half, \
                        n_strips, rps, in_bytes, out_bytes)
 #define OHIP_DWF_N(S_, E_)                       \
     do {                                         \

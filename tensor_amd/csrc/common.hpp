@@ -157,6 +157,9 @@ struct ConvGeom {
     // channels per image of the tensors in memory, when the kernel works on a channel slice of them (one group of a
     // grouped convolution: C, K are the group's, Cs, Ks the tensors'); 0 = the same as C / K
     int Cs = 0, Ks = 0;
+    // implicit-GEMM kernel only: kernel taps that share one 64-deep reduction step (2 for at most 32 input channels, 4 for
+    // at most 16; the weights are packed to match, igemm_tap_pack); 0 or 1 = a step is one tap x 64 channels
+    int tap_pack = 0;
 };
 
 // ---------------------------------------------------------------------------------------------------

@@ -71,7 +71,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     if (blockIdx.z) {
         const int grp = blockIdx.z;
         x += (size_t)grp * (g.C / 8) * g.H * g.W * 8;
-        wpk += (size_t)grp * (g.kh * g.kw * c_groups) * m_tiles16 * 1024;
+        wpk += (size_t)grp * (g.tap_pack > 1 ? (g.kh * g.kw + g.tap_pack - 1) / g.tap_pack : g.kh * g.kw * c_groups) * m_tiles16 * 1024;
         out = (char*)out + (size_t)grp * g.K * OHW * (EPI == EPI_I8_P8 || EPI == EPI_I8_P8_NONNEG ? 1 : 4);
         ep.scale_in += grp * g.K;
         ep.bias += grp * g.K;
@@ -127,9 +127,29 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
 
     v2i breg[KC][Cfg::B_V][2];
     v4i areg[KC][Cfg::A_V];
-    const int n_chunks = g.kh * g.kw * c_groups;
+    // Few input channels (a group of a grouped convolution with at most 32): tap_pack kernel taps share a reduction
+    // step, the 16-channel quarter j of the step being channels 16 (j % per) .. of tap tap_pack * kc + j / per with
+    // per = 4 / tap_pack quarters per tap (j is the same for a whole wave: a pixel tile is at least 64 wide)
+    const int tpk = g.tap_pack > 1 ? g.tap_pack : 1;
+    const int n_chunks = tpk > 1 ? (g.kh * g.kw + tpk - 1) / tpk : g.kh * g.kw * c_groups;
 
     auto load_global = [&](int kc, int q) {
+        if (tpk > 1) {  // (uniform)
+            const int per = 4 / tpk;
+#pragma unroll
+            for (int r = 0; r < Cfg::B_V; ++r) {
+                const int j = j0 + r * J_STEP;
+                const int tap = kc * tpk + j / per;
+                const int u = tap / g.kw, v = tap - u * g.kw;
+                const int iy = iy0 + u * g.dh, ix = ix0 + v * g.dw;
+                const bool inb = pvalid && tap < g.kh * g.kw && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                const int o0 = 2 * (j % per);
+                const unsigned v_lo = (unsigned)(px_ofs + ((u * g.dh) * g.W + v * g.dw) * 8 + o0 * HW * 8);
+                breg[q][r][0] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(inb && o0 < C8 ? v_lo : IG_OOB), 0, 0));
+                breg[q][r][1] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(
+                    rin, (int)(inb && o0 + 1 < C8 ? v_lo + (unsigned)(HW * 8) : IG_OOB), 0, 0));
+            }
+        } else {
         const int tap = kc / c_groups, cgp = kc % c_groups;
         const int u = tap / g.kw, v = tap % g.kw;
         bool inb = pvalid;
@@ -145,6 +165,7 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             breg[q][r][0] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(inb && o0 < C8 ? v_lo : IG_OOB), 0, 0));
             breg[q][r][1] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(
                 rin, (int)(inb && o0 + 1 < C8 ? v_lo + (unsigned)(HW * 8) : IG_OOB), 0, 0));
+        }
         }
         const int8_t* wa = wpk + ((size_t)kc * m_tiles16 + mt0) * 1024;
 #pragma unroll
@@ -368,14 +389,39 @@ int igemm_row_channel(int row) {
     return 32 * (mt / 2) + 8 * (r / 4) + 4 * (mt % 2) + (r % 4);
 }
 
-size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw) {
-    return (size_t)kh * kw * igemm_channel_groups(C) * (igemm_padded_rows(K) / 16) * 1024;
+// how many kernel taps of a layer with C input channels fit one 64-deep reduction step (1: none are packed)
+int igemm_tap_pack(int C, int kh, int kw) {
+    if (kh * kw < 2) return 1;
+    return C <= 16 ? 4 : (C <= 32 ? 2 : 1);
 }
 
-// weight [K, C, kh, kw] int8 -> [k-chunk = (tap, channel group)][16-row tile][lane][16 bytes]
-void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst) {
+static int igemm_k_chunks(int C, int kh, int kw, int tap_pack) {
+    return tap_pack > 1 ? (kh * kw + tap_pack - 1) / tap_pack : kh * kw * igemm_channel_groups(C);
+}
+
+size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw, int tap_pack) {
+    return (size_t)igemm_k_chunks(C, kh, kw, tap_pack) * (igemm_padded_rows(K) / 16) * 1024;
+}
+
+// weight [K, C, kh, kw] int8 -> [k-chunk = (tap, channel group)][16-row tile][lane][16 bytes]; with tap_pack > 1 a
+// k-chunk is tap_pack taps: its 16-byte quarter j (= lane / 16) holds channels 16 (j % per) .. of tap tap_pack * kc + j / per
+void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst, int tap_pack) {
     const int mt16 = igemm_padded_rows(K) / 16, cgs = igemm_channel_groups(C);
     size_t o = 0;
+    if (tap_pack > 1) {
+        const int per = 4 / tap_pack;
+        for (int kc = 0; kc < igemm_k_chunks(C, kh, kw, tap_pack); ++kc)
+            for (int mt = 0; mt < mt16; ++mt)
+                for (int lane = 0; lane < 64; ++lane) {
+                    const int ch = igemm_row_channel(mt * 16 + (lane & 15));
+                    const int j = lane >> 4, tap = kc * tap_pack + j / per;
+                    for (int b = 0; b < 16; ++b, ++o) {
+                        const int c = 16 * (j % per) + b;
+                        dst[o] = (ch < K && c < C && tap < kh * kw) ? w[((size_t)ch * C + c) * kh * kw + tap] : 0;
+                    }
+                }
+        return;
+    }
     for (int tap = 0; tap < kh * kw; ++tap)
         for (int cg = 0; cg < cgs; ++cg)
             for (int mt = 0; mt < mt16; ++mt)
@@ -413,7 +459,7 @@ static hipError_t launch_igemm_e(const int8_t* x, const int8_t* wpk, void* out, 
     // The staged variant shortens a workgroup's life (one global-memory latency per KC chunks) but needs KC times the
     // LDS. It pays when the whole grid is resident at once even so - the launch is then one workgroup life long -
     // and costs where the grid runs in rounds, which the smaller footprint packs tighter. (256 compute units.)
-    const int n_chunks = g.kh * g.kw * igemm_channel_groups(g.C);
+    const int n_chunks = igemm_k_chunks(g.C, g.kh, g.kw, g.tap_pack);
     bool staged = false;
     if (n_chunks >= 2) {
         constexpr int KCS = IgemmStage<TM, TN>::KC;
@@ -451,7 +497,7 @@ static hipError_t launch_igemm(const int8_t* x, const int8_t* wpk, void* out, co
 void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn) {
     const int mpad = igemm_padded_rows(g.K);
     const long total_pix = (long)g.N * g.OH * g.OW;
-    const int n_chunks = g.kh * g.kw * igemm_channel_groups(g.C);
+    const int n_chunks = igemm_k_chunks(g.C, g.kh, g.kw, g.tap_pack);
     auto wgs = [&](int TM, int TN) { return ((total_pix + TN - 1) / TN) * ((g.K + TM - 1) / TM); };
     int TM = 32, TN = 64;
     if (n_chunks > 16) {
@@ -487,15 +533,16 @@ bool igemm_grouped_applicable(const ConvGeom& g, const Epilogue& ep) {
 }
 
 size_t igemm_grouped_weight_bytes(int K, int C, int groups, int kh, int kw) {
-    return (size_t)groups * igemm_packed_weight_bytes(K / groups, C / groups, kh, kw);
+    return (size_t)groups * igemm_packed_weight_bytes(K / groups, C / groups, kh, kw, igemm_tap_pack(C / groups, kh, kw));
 }
 
 // weight [K, C/groups, kh, kw]: every group's [K/groups, C/groups, kh, kw] block packed by itself, one after the other
 void igemm_pack_weights_grouped(const int8_t* w, int K, int C, int groups, int kh, int kw, int8_t* dst) {
     const int kg = K / groups, cg = C / groups;
-    const size_t per = igemm_packed_weight_bytes(kg, cg, kh, kw);
+    const int tp = igemm_tap_pack(cg, kh, kw);  // groups of at most 32 channels: two or four taps per reduction step
+    const size_t per = igemm_packed_weight_bytes(kg, cg, kh, kw, tp);
     for (int grp = 0; grp < groups; ++grp)
-        igemm_pack_weights(w + (size_t)grp * kg * cg * kh * kw, kg, cg, kh, kw, dst + grp * per);
+        igemm_pack_weights(w + (size_t)grp * kg * cg * kh * kw, kg, cg, kh, kw, dst + grp * per, tp);
 }
 
 hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const ConvGeom& g_in, const Epilogue& ep,
@@ -506,6 +553,7 @@ hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const C
         g.Cs = g_in.C, g.Ks = g_in.K;
         g.C = g_in.C / g_in.groups, g.K = g_in.K / g_in.groups;
         g.groups = 1;
+        g.tap_pack = igemm_tap_pack(g.C, g.kh, g.kw);  // (as igemm_pack_weights_grouped packed the weights)
     }
     // a forced pixel tile may carry the stage choice in its low bits (1: one chunk per stage, 2: the staged variant)
     const int stage = tn & 3;

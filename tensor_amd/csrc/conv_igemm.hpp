@@ -8,8 +8,10 @@ namespace ohip {
 int igemm_padded_rows(int K);
 int igemm_channel_groups(int C);
 int igemm_row_channel(int row);
-size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw);
-void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst);
+// tap_pack > 1 (igemm_tap_pack): that many kernel taps of at most 64 / tap_pack channels share a reduction step
+size_t igemm_packed_weight_bytes(int K, int C, int kh, int kw, int tap_pack = 1);
+void igemm_pack_weights(const int8_t* w, int K, int C, int kh, int kw, int8_t* dst, int tap_pack = 1);
+int igemm_tap_pack(int C, int kh, int kw);
 void igemm_choose_tiles(const ConvGeom& g, int* tm, int* tn);
 bool igemm_grouped_applicable(const ConvGeom& g, const Epilogue& ep);
 size_t igemm_grouped_weight_bytes(int K, int C, int groups, int kh, int kw);

@@ -48,8 +48,9 @@ SETTLE_S = 0.15  # untimed run-in before the warm-up steps, seconds of the workl
 
 
 class Timer:
-    def __init__(self, torch):
+    def __init__(self, torch, hip=None):
         self.torch = torch
+        self.hip = hip  # the library binding, for the clock measurement behind a matrix-bound loop
 
     def run(self, fn, steps, warmup, settle=None):
         """fn: a closure, or a list of closures taken in turn (the same launch over different buffer sets, so that the
@@ -704,6 +705,22 @@ def measure(wl, timer, steps, warmup, unit_main):
         ach = wl["dom_ops"] / (kms * 1e-3) / 1e12
         res["roofline"] = dict(bound="mfma", achieved=ach, peak=PEAK_INT8_TOPS, unit="TOP/s", frac=ach / PEAK_INT8_TOPS,
                                traffic=measured_traffic(wl["name"]), kernel=wl["dom_kernel"], kernel_ms=kms)
+        # The published peak assumes the maximum engine clock. What the matrix cores can do on THIS box: compute units
+        # x 4 SIMDs x 2048 int8 operations per cycle x the shader clock it holds under matrix load, measured right behind
+        # the timed loop (the clock is in its loaded state then).
+        hipl = timer.hip
+        if hipl is not None:
+            info = hipl.device_info()
+            # (the chain launch times itself with the shader-cycle counter; other kernels get the clock of a millisecond
+            # of bare matrix instructions, which is an upper bound: a kernel that also keeps the vector ALU and LDS busy
+            # holds a lower clock)
+            mhz = hipl.conv_chain_clock_mhz() if wl["name"] == "c3" else 0.0
+            res["roofline"]["shader_clock_source"] = "the timed kernel's own cycle counter" if mhz > 0 else "a bare matrix-instruction loop"
+            if mhz <= 0:
+                mhz = hipl.shader_clock_mhz()
+            peak_clk = info["compute_units"] * 4 * 2048 * mhz * 1e6 / 1e12
+            res["roofline"].update(shader_clock_mhz=mhz, max_clock_mhz=info["clock_mhz"], compute_units=info["compute_units"],
+                                   peak_at_shader_clock=peak_clk, frac_of_peak_at_shader_clock=ach / peak_clk)
     else:
         ach = wl["dom_bytes"] / (kms * 1e-3) / 1e9
         res["roofline"] = dict(bound="hbm", achieved=ach, peak=PEAK_HBM_GBS, unit="GB/s", frac=ach / PEAK_HBM_GBS,
@@ -755,7 +772,7 @@ def main():
 
     from tensor_amd import capi
     hip = capi.Library(0)
-    timer = Timer(hip.torch)
+    timer = Timer(hip.torch, hip)
     if a.per_layer:
         from tensor_amd import mobilenet
         rows = mobilenet.per_layer(hip, capi, np.random.default_rng(0),

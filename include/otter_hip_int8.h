@@ -70,6 +70,12 @@ const char* otter_hip_last_error(void);
 
 /* compute units, engine clock in MHz, memory clock in MHz, memory bus width in bits: inputs of the roofline */
 int otter_hip_device_info(int* compute_units, int* clock_mhz, int* mem_clock_mhz, int* mem_bus_bits);
+/* The shader clock the GPU holds under int8 matrix load, measured now: about a millisecond of matrix instructions on
+ * every SIMD, timed with the shader-cycle counter against the constant 100 MHz counter. The published matrix peak
+ * assumes the maximum engine clock of otter_hip_device_info; compute units x 4 SIMDs x 2048 int8 operations per cycle x
+ * this clock is what the matrix cores can do on the box at hand. Allocates a few KB and synchronizes `stream`. No
+ * counterpart in the reference (a CPU library). */
+int otter_hip_shader_clock_mhz(void* stream, float* mhz);
 
 /* Device memory + copies for hosts that do not link HIP themselves. Stand in for otter::empty() /
  * Tensor::data_ptr() ownership of blobs (Tensor/TensorFactory.hpp, Tensor/Net.cpp:413-505). */
@@ -196,6 +202,11 @@ int otter_hip_conv_chain_status(int* gave_up);
  * (1: the single persistent launch; n_layers: layer by layer, also when every flag set was busy; 0: none yet). The
  * reference has no counterpart (its Net runs a layer per call, Tensor/Net.cpp:413-505). */
 int otter_hip_conv_chain_last_launches(void);
+/* The shader clock the most recent single-launch chain on this GPU ran at, in MHz (0: there has been none): its last
+ * workgroup reads the shader-cycle counter and the constant 100 MHz counter over its life. For the roofline: the
+ * published matrix peak assumes the maximum engine clock, a kernel that keeps matrix cores, vector ALU and LDS busy
+ * holds less. Synchronizes the device. No counterpart in the reference. */
+int otter_hip_conv_chain_clock_mhz(float* mhz);
 /* For tests and profiling: the number of convolution launches otter_hip_conv_chain_forward makes for this chain and
  * input (1: the single persistent launch; n_layers: layer by layer), or a negative status. */
 int otter_hip_conv_chain_launches(const otter_hip_conv_t* const* handles, int n_layers, int n, int in_h, int in_w);

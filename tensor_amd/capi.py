@@ -60,7 +60,8 @@ class HipError(RuntimeError):
         self.code = code
 
 
-EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otter_hip_device_info", "otter_hip_malloc",
+EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otter_hip_device_info",
+           "otter_hip_shader_clock_mhz", "otter_hip_malloc",
            "otter_hip_free", "otter_hip_memcpy_h2d", "otter_hip_memcpy_d2h", "otter_hip_stream_create",
            "otter_hip_stream_destroy", "otter_hip_stream_synchronize", "otter_hip_conv_create",
            "otter_hip_conv_destroy", "otter_hip_conv_output_shape", "otter_hip_conv_default_out_layout",
@@ -73,7 +74,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_copy_channels_quantize", "otter_hip_channel_shuffle_quantize",
            "otter_hip_concat_channels", "otter_hip_conv_forward_static", "otter_hip_conv3x3_halo_plan", "otter_hip_conv_chain_workspace_bytes",
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
-           "otter_hip_conv_chain_last_launches",
+           "otter_hip_conv_chain_last_launches", "otter_hip_conv_chain_clock_mhz",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
            "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always",
            "otter_hip_conv_block_plan"]
@@ -125,6 +126,12 @@ class Library:
         v = [C.c_int() for _ in range(4)]
         self._check(self.lib.otter_hip_device_info(*[C.byref(x) for x in v]))
         return dict(compute_units=v[0].value, clock_mhz=v[1].value, mem_clock_mhz=v[2].value, mem_bus_bits=v[3].value)
+
+    def shader_clock_mhz(self):
+        """otter_hip_shader_clock_mhz: the shader clock under int8 matrix load, measured now on the current stream."""
+        v = C.c_float(0)
+        self._check(self.lib.otter_hip_shader_clock_mhz(self.stream(), C.byref(v)))
+        return float(v.value)
 
     # -- standalone ops (device tensors in packed storage) ------------------------------------------------
     def quantize(self, src, src_layout, shape, scales, round_mode, dst_layout, dst=None):
@@ -306,6 +313,12 @@ class Library:
     def conv_chain_last_launches(self):
         """otter_hip_conv_chain_last_launches: the launches the last chain call of this thread actually made."""
         return self.lib.otter_hip_conv_chain_last_launches()
+
+    def conv_chain_clock_mhz(self):
+        """otter_hip_conv_chain_clock_mhz: the shader clock of the last single-launch chain (synchronizes); 0 if none."""
+        v = C.c_float(0)
+        self._check(self.lib.otter_hip_conv_chain_clock_mhz(C.byref(v)))
+        return float(v.value)
 
     def conv_chain_gave_up(self):
         """otter_hip_conv_chain_status: synchronizes; True if a chain launch since the last call gave up a wait."""

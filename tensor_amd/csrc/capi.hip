@@ -142,6 +142,30 @@ int otter_hip_device_info(int* compute_units, int* clock_mhz, int* mem_clock_mhz
     return OTTER_HIP_OK;
 }
 
+int otter_hip_shader_clock_mhz(void* stream_, float* mhz) {
+    if (!mhz) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_shader_clock_mhz: null");
+    int dev = 0;
+    OHIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    OHIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    const int blocks = prop.multiProcessorCount;
+    hipStream_t stream = (hipStream_t)stream_;
+    unsigned long long* d = nullptr;
+    OHIP_CHECK(hipMalloc(&d, sizeof(unsigned long long) * 2 * blocks));
+    // about a millisecond of matrix instructions on every SIMD (4 x 20000 of 16 cycles each)
+    hipError_t e = run_shader_clock(blocks, 20000, d, stream);
+    std::vector<unsigned long long> h(2 * blocks);
+    if (e == hipSuccess) e = hipMemcpyAsync(h.data(), d, sizeof(unsigned long long) * 2 * blocks, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    (void)hipFree(d);
+    OHIP_CHECK(e);
+    double cyc = 0, ref = 0;
+    for (int i = 0; i < blocks; ++i) cyc += (double)h[2 * i], ref += (double)h[2 * i + 1];
+    if (ref <= 0) return fail(OTTER_HIP_ERR_RUNTIME, "otter_hip_shader_clock_mhz: the reference counter did not advance");
+    *mhz = (float)(cyc / ref * 100.0);  // the reference counter runs at 100 MHz
+    return OTTER_HIP_OK;
+}
+
 int otter_hip_malloc(void** ptr, size_t bytes) {
     if (!ptr) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_malloc: null");
     OHIP_CHECK(hipMalloc(ptr, bytes ? bytes : 1));
@@ -729,6 +753,12 @@ int otter_hip_conv_chain_forward(const otter_hip_conv_t* const* handles, int n_l
 }
 
 int otter_hip_conv_chain_last_launches(void) { return t_chain_last_launches; }
+
+int otter_hip_conv_chain_clock_mhz(float* mhz) {
+    if (!mhz) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_clock_mhz: null");
+    OHIP_CHECK(conv3x3_chain_clock_mhz(mhz));  // (synchronizes with the device)
+    return OTTER_HIP_OK;
+}
 
 int otter_hip_conv_chain_status(int* gave_up) {
     if (!gave_up) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_chain_status: null");

@@ -297,6 +297,14 @@ __device__ __forceinline__ void epi8_clamp_init(const Epilogue& ep, Epi8& p) {
     }
 }
 
+// float -> uint32 toward zero, everything below zero (and NaN) to 0, everything above to 2^32 - 1: v_cvt_u32_f32. (As an
+// instruction, not as a C++ conversion: that one is undefined for negative values.)
+__device__ __forceinline__ unsigned cvt_u32_floor0(float v) {
+    unsigned r;
+    asm("v_cvt_u32_f32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+
 // LRELU: 0 = no LeakyReLU, 1 = LeakyReLU, -1 = decided by ep.lrelu at run time (a select per value)
 template <bool NONNEG, int LRELU = -1>
 __device__ __forceinline__ ohip_v2i epi8_quant_i8p8(const Epilogue& ep, const Epi8& p, const int (&a8)[8]) {
@@ -309,12 +317,24 @@ __device__ __forceinline__ ohip_v2i epi8_quant_i8p8(const Epilogue& ep, const Ep
         }
         v = __fmul_rn(v, p.so[e]);
         float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
-        q[e] = (int)adj;  // toward zero, saturating
+        // toward zero, saturating. NONNEG: to UNSIGNED, which sends everything below zero to zero: the lower clamp of
+        // the activation comes with the conversion, and only the upper one is left for the packed values
+        if constexpr (NONNEG) q[e] = (int)cvt_u32_floor0(adj);
+        else q[e] = (int)adj;
     }
     ohip_v2i pk;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         // two int32 -> two saturated int16 in one dword, clamp both halves at once, then gather the low bytes
+        if constexpr (NONNEG) {
+            typedef unsigned short ohip_v2us __attribute__((ext_vector_type(2)));
+            ohip_v2us lo = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)q[4 * h], (unsigned)q[4 * h + 1]));
+            ohip_v2us hi = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)q[4 * h + 2], (unsigned)q[4 * h + 3]));
+            lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2us, p.qh[2 * h]));
+            hi = __builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2us, p.qh[2 * h + 1]));
+            pk[h] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
+            continue;
+        }
         ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h], q[4 * h + 1]));
         ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[4 * h + 2], q[4 * h + 3]));
         if (NONNEG) {

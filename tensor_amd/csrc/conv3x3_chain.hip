@@ -50,7 +50,8 @@ constexpr int CHAIN_SPIN_LIMIT = 1 << 17;  // polls of a producer flag before gi
 // different streams may overlap and must not share them.
 constexpr int CHAIN_SLOTS = 4;
 __device__ int g_chain_flags[CHAIN_SLOTS * CHAIN_MAX_FLAGS];
-__device__ int g_chain_ctl[CHAIN_SLOTS * 16];  // per slot: [0..7] queue counters, [8] workgroups that have left, [9] error, [10] launches completed
+__device__ int g_chain_ctl[CHAIN_SLOTS * 16];  // per slot: [0..7] queue counters, [8] workgroups that have left, [9] error, [10] launches completed,
+                                               // [11] shader cycles and [12] ticks of the 100 MHz counter of the last launch (its last workgroup's life)
 
 struct ChainArgs {
     const int8_t* act[CHAIN_MAX_LAYERS + 1];  // act[l]: input of layer l; act[l + 1]: its output
@@ -103,6 +104,9 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
     // The launch's epoch number = the count of completed launches on this flag set + 1, kept in device memory (ctl[10],
     // advanced by the last workgroup to leave): a launch replayed from a captured graph gets a fresh number like any other.
     const int epoch = __builtin_amdgcn_readfirstlane(__hip_atomic_load(ca.ctl + 10, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) + 1;
+    // (for the clock the kernel ran at: the shader-cycle counter and the constant 100 MHz counter, read again by the last
+    // workgroup to leave)
+    const unsigned long long clk0 = __builtin_readcyclecounter(), ref0 = __builtin_amdgcn_s_memrealtime();
 
     // ---- this XCD's tile list ------------------------------------------------------------------------------------
     const int xcd = __builtin_amdgcn_readfirstlane(chain_xcc_id() % ca.xcds);
@@ -419,6 +423,8 @@ __global__ void __launch_bounds__(256, 2) conv3x3_chain_kernel(ConvGeom g, Epilo
                     __hip_atomic_store(ca.ctl + 9, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             for (int i = 0; i < 9; ++i) __hip_atomic_store(ca.ctl + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ca.ctl[11] = (int)(__builtin_readcyclecounter() - clk0);
+            ca.ctl[12] = (int)(__builtin_amdgcn_s_memrealtime() - ref0);
             __hip_atomic_store(ca.ctl + 10, epoch == 0x7ffffffe ? 0 : epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -603,6 +609,26 @@ hipError_t conv3x3_chain_error(int* error_word) {
             for (int i = 0; i < 10; ++i) ctl[s * 16 + i] = 0;
         if ((e = hipMemcpy(g_chain_dev[dev].ctl, ctl, sizeof(ctl), hipMemcpyHostToDevice)) != hipSuccess) return e;
     }
+    return hipSuccess;
+}
+
+// the shader clock of the most recent single-launch chain on this device, from the two counters its last workgroup
+// left behind; synchronizes with the device. 0 if there has been none.
+hipError_t conv3x3_chain_clock_mhz(float* mhz) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    *mhz = 0.f;
+    std::lock_guard<std::mutex> lock(g_chain_mutex);
+    if ((e = hipDeviceSynchronize()) != hipSuccess) return e;
+    if (dev < 0 || dev >= 16 || !g_chain_dev[dev].ctl) return hipSuccess;
+    int ctl[CHAIN_SLOTS * 16];
+    if ((e = hipMemcpy(ctl, g_chain_dev[dev].ctl, sizeof(ctl), hipMemcpyDeviceToHost)) != hipSuccess) return e;
+    int best = -1;
+    for (int s = 0; s < CHAIN_SLOTS; ++s)
+        if (g_chain_dev[dev].used[s] && ctl[s * 16 + 12] > 0 && (best < 0 || g_chain_dev[dev].stamp[s] > g_chain_dev[dev].stamp[best]))
+            best = s;
+    if (best >= 0) *mhz = (float)((double)ctl[best * 16 + 11] / (double)ctl[best * 16 + 12] * 100.0);
     return hipSuccess;
 }
 

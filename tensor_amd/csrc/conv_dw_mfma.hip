@@ -91,7 +91,17 @@ __device__ __forceinline__ unsigned dw_requant4(const Epilogue& ep, const v4i& a
         if (!NONNEG && ep.lrelu) v = fmaxf(v, __fmul_rn(v, ep.act_p0));  // wave-uniform branch
         v = __fmul_rn(v, __int_as_float(so[e]));
         const float adj = NONNEG ? __fadd_rn(v, ep.round_half) : __fadd_rn(v, __builtin_copysignf(ep.round_half, v));
-        qv[e] = (int)adj;  // toward zero, saturating
+        // toward zero, saturating; NONNEG: to unsigned, which is also the activation's lower clamp
+        if constexpr (NONNEG) qv[e] = (int)cvt_u32_floor0(adj);
+        else qv[e] = (int)adj;
+    }
+    if constexpr (NONNEG) {
+        typedef unsigned short ohip_v2us __attribute__((ext_vector_type(2)));
+        ohip_v2us lo = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)qv[0], (unsigned)qv[1]));
+        ohip_v2us hi = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)qv[2], (unsigned)qv[3]));
+        lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2us, qh01));
+        hi = __builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2us, qh23));
+        return __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
     }
     ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[0], qv[1]));
     ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(qv[2], qv[3]));

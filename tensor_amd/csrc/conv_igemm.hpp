@@ -53,6 +53,7 @@ bool conv3x3_chain_applicable(const ConvGeom& g, const Epilogue& ep, int layers,
 hipError_t run_conv3x3_chain(const ConvGeom& g, const Epilogue* eps, const int8_t* const* wpk, const int8_t* const* act,
                              int layers, int* error_word_out, hipStream_t stream, int force_fn = 0);
 hipError_t conv3x3_chain_error(int* error_word);
+hipError_t conv3x3_chain_clock_mhz(float* mhz);
 
 // conv_direct.hip
 hipError_t run_conv_direct(const int8_t* x, int in_pack, const int8_t* wt, void* out, const ConvGeom& g,
@@ -98,6 +99,7 @@ hipError_t run_activation(float* x, size_t n, int act, float p0, hipStream_t str
 hipError_t run_eltwise_add_quantize(const float* a, const float* b, int pack, float* out, int8_t* q, int N, int C, int HW,
                                     float scale, int round_mode, hipStream_t stream);
 hipError_t run_global_avgpool(const float* x, int pack, int N, int C, int HW, float* out, hipStream_t stream);
+hipError_t run_shader_clock(int blocks, int iters, unsigned long long* out, hipStream_t stream);
 hipError_t run_inner_product(const float* x, const float* w, const float* b, float* y, int N, int IN, int OUT,
                              hipStream_t stream);
 

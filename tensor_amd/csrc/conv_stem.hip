@@ -328,13 +328,13 @@ __global__ void __launch_bounds__(256) conv_stem3x3_lds_kernel(const void* __res
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float t = __fmul_rn(__fmaf_rn((float)acc[i], si[m][i], bi[m][i]), so[m][i]);
-                    q[i] = (int)__fadd_rn(t, ep.round_half);
+                    q[i] = (int)cvt_u32_floor0(__fadd_rn(t, ep.round_half));  // (to unsigned: the clamp at zero comes with it)
                 }
-                const ohip_v2s zero = {0, 0};
-                ohip_v2s lo = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[0], q[1]));
-                ohip_v2s hi = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(q[2], q[3]));
-                lo = __builtin_elementwise_max(__builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2s, qh[m][0])), zero);
-                hi = __builtin_elementwise_max(__builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2s, qh[m][1])), zero);
+                typedef unsigned short ohip_v2us __attribute__((ext_vector_type(2)));
+                ohip_v2us lo = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)q[0], (unsigned)q[1]));
+                ohip_v2us hi = __builtin_bit_cast(ohip_v2us, __builtin_amdgcn_cvt_pk_u16((unsigned)q[2], (unsigned)q[3]));
+                lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ohip_v2us, qh[m][0]));
+                hi = __builtin_elementwise_min(hi, __builtin_bit_cast(ohip_v2us, qh[m][1]));
                 unsigned* o = reinterpret_cast<unsigned*>(out) + (((size_t)img * (g.K / 8) + ch0 / 8) * OHW + pix) * 2 + (ch0 / 4 & 1);
                 *o = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, hi), __builtin_bit_cast(unsigned, lo), 0x06040200u);
             } else {

@@ -267,4 +267,30 @@ hipError_t run_inner_product(const float* x, const float* w, const float* b, flo
     return hipGetLastError();
 }
 
+// The shader clock under matrix load: every wave runs int8 matrix instructions for `iters` rounds and brackets them with
+// the shader-clock counter (s_memtime) and the constant 100 MHz counter (s_memrealtime); wave 0 of every workgroup
+// writes its two differences. A workgroup per compute unit, four waves each (one per SIMD).
+__global__ void __launch_bounds__(256) shader_clock_kernel(int iters, unsigned long long* __restrict__ out) {
+    typedef int ck_v4i __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x & 63;
+    ck_v4i a = {lane, lane + 1, lane + 2, lane + 3}, b = {lane * 3, 1, 2, 3};
+    ck_v4i acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i], 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+    if (threadIdx.x == 0) {
+        out[2 * blockIdx.x] = c1 - c0;
+        out[2 * blockIdx.x + 1] = r1 - r0;
+    }
+    if (acc[0][0] + acc[1][1] + acc[2][2] + acc[3][3] == 0x7fffffff) out[0] = 0;  // (keeps the loop)
+}
+
+hipError_t run_shader_clock(int blocks, int iters, unsigned long long* out, hipStream_t stream) {
+    hipLaunchKernelGGL(shader_clock_kernel, dim3(blocks), dim3(256), 0, stream, iters, out);
+    return hipGetLastError();
+}
+
 }  // namespace ohip

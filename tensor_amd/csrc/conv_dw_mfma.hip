@@ -361,12 +361,6 @@ __global__ void __launch_bounds__(256) conv_dw3x3_mfma_kernel(const int8_t* __re
 // the wave needs no barrier between its lanes' writes and reads. The loads run four input rows ahead of the
 // quantization in a ring of registers; the matrix instructions of a row run under the quantization of the next one, its
 // epilogue follows that. Rows outside the image or past the strip read zero through the buffer descriptor.
-#ifdef OHIP_DWF_STAMPS
-__device__ unsigned long long dwf_stamps[8][64];
-#define DWF_STAMP(i) do { if (stamp_me && lane == 0 && (i) < 64) dwf_stamps[stamp_w][(i)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define DWF_STAMP(i) do { } while (0)
-#endif
 template <int S, int EPI, int NL>
 __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* __restrict__ x, const int8_t* __restrict__ wa,
                                                                void* __restrict__ out, ConvGeom g, Epilogue ep,
@@ -394,12 +388,6 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
     if (strip >= n_strips) return;  // whole wave
     const int lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
     int8_t* const lds = &lds_all[wave][0][0];
-#ifdef OHIP_DWF_STAMPS
-    const bool stamp_me = blockIdx.y % 37 == 0 && blockIdx.y / 37 < 2 && blockIdx.x == 0;
-    const int stamp_w = (blockIdx.y / 37) * 4 + wave;
-    int stamp_i = 0;
-#endif
-    DWF_STAMP(stamp_i++);
 
     // the padding slots of every line: pixels -2, -1 and 32 NL .. 64 NCH + 5 (the row's own pixels from W on are written
     // as zeros with every row)
@@ -438,9 +426,6 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
     };
     // float2int8 of four values into four bytes (the arithmetic of otter_hip_quantize)
     auto quant4 = [&](const v4i& f) -> int {
-#ifdef OHIP_DWF_NOQUANT
-        return f[0] ^ f[1] ^ f[2] ^ f[3];
-#endif
         int k[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -586,7 +571,6 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
             row_mfma((jj - 2 + 4) % RL);
         }
         __builtin_amdgcn_sched_barrier(0);
-        DWF_STAMP(stamp_i++);
     };
     no_store(3);
     input_row(0, 0, false);
@@ -605,13 +589,7 @@ __global__ void __launch_bounds__(256, 3) conv_dw3x3_f32in_kernel(const float* _
     for (int i = 0; i < UNR - 1; ++i)
         if (jb + i < nq) input_row(jb + i, 3 + i, true);  // wave-uniform
     epilogue_store(nrows - 1);
-    DWF_STAMP(stamp_i++);
 }
-#ifdef OHIP_DWF_STAMPS
-extern "C" int otter_hip_debug_dwf_stamps(unsigned long long* out) {
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(dwf_stamps), sizeof(dwf_stamps));
-}
-#endif
 
 // true when the fused fp32 -> depthwise launch takes this layer and blob (Float8 input; the caller has checked
 // dw_mfma_applicable)

@@ -231,9 +231,13 @@ int otter_hip_conv_chain_set_min_tiles(int tiles);
  * over the batch, at most 24 tiles of 32 channels x 16 pixels of the last layer per band), or for every shape that qualifies after
  * otter_hip_conv_block_set_always(1) / a forced plan. Where a batch has fewer bands than half the compute units, the
  * expanded channels of a band are dealt to several workgroups whose accumulators meet in `workspace` (the last to
- * arrive adds them up: integer sums, the same result). Otherwise the call makes three launches with the two
- * intermediate blobs in `workspace`. otter_hip_conv_block_workspace_bytes gives the size either way (0 for a single
- * launch with one workgroup per band). */
+ * arrive adds them up: integer sums, the same result). Otherwise, where the first layer reads at most 128 channels and
+ * writes a multiple of 16, the depthwise layer is 3x3 stride 1 / 2 on an image at most 128 pixels wide (64 when the first
+ * layer reads more than 32 channels) and both clamp at zero or neither clamps, the first two layers can run as ONE
+ * launch that keeps the expanded rows in LDS, the last layer by itself; they do (otter_hip_conv_block_launches says 2)
+ * where that was measured faster, or wherever they can after otter_hip_conv_block_set_pair(1); any other block makes
+ * three launches. The blobs between the launches live in `workspace`;
+ * otter_hip_conv_block_workspace_bytes gives the size either way (0 for a single launch with one workgroup per band). */
 int otter_hip_conv_block_launches(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
                                   const otter_hip_conv_t* project, int n, int in_h, int in_w);
 size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* expand, const otter_hip_conv_t* depthwise,
@@ -253,6 +257,11 @@ int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_ch
  * launch, 0 = only the shapes measured faster that way (default). Process-wide; returns the previous value; a negative
  * argument only queries. */
 int otter_hip_conv_block_set_always(int on);
+/* Tuning / test hook with no counterpart in the reference: how a block that does not run as the single launch runs its
+ * first two layers: 0 = as one launch where that was measured faster (a stride-2 depthwise layer, or an expanded blob
+ * of 16 MiB or more; default), 1 = wherever the kernel takes the shapes, -1 = always one by one. Process-wide; returns
+ * the previous value; any other argument only queries. */
+int otter_hip_conv_block_set_pair(int mode);
 /* Tuning / test hook with no counterpart in the reference: force the single launch's output rows per band, the
  * expanded channels per LDS slice (64 or 128) and the workgroups a band's slices are dealt to, for blocks whose first
  * layer is `expand`; 0 = automatic. */

@@ -76,7 +76,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_chain_forward", "otter_hip_conv_chain_status", "otter_hip_conv_chain_launches",
            "otter_hip_conv_chain_last_launches", "otter_hip_conv_chain_clock_mhz",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
-           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always",
+           "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always", "otter_hip_conv_block_set_pair",
            "otter_hip_conv_block_plan"]
 
 
@@ -265,6 +265,7 @@ class Library:
             oh, ow = c.out_hw(oh, ow)
         if out is None:
             out = self.empty(n * convs[-1].K * oh * ow, np.int8)
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0  # what the buffer really holds
         self._check(self.lib.otter_hip_conv_chain_forward(hs, len(convs), self.ptr(x), n, h, w, self.ptr(out),
                                                           self.ptr(workspace) if workspace is not None else None,
                                                           C.c_size_t(ws_bytes), self.stream()))
@@ -285,6 +286,7 @@ class Library:
         ws_bytes = self.lib.otter_hip_conv_block_workspace_bytes(expand.h, dw.h, project.h, n, h, w)
         if ws_bytes and workspace is None:
             workspace = self.empty(ws_bytes, np.int8)
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0  # what the buffer really holds
         self._check(self.lib.otter_hip_conv_block_forward(
             expand.h, dw.h, project.h, self.ptr(x), n, h, w, self.ptr(residual) if residual is not None else None,
             self.ptr(out), out_layout, self.ptr(q) if q is not None else None, C.c_float(q_scale or 0.0), q_round_mode,
@@ -294,6 +296,10 @@ class Library:
     def conv_block_set_always(self, on):
         """otter_hip_conv_block_set_always: returns the previous setting."""
         return self.lib.otter_hip_conv_block_set_always(int(on))
+
+    def conv_block_set_pair(self, mode):
+        """otter_hip_conv_block_set_pair: returns the previous setting."""
+        return self.lib.otter_hip_conv_block_set_pair(int(mode))
 
     def conv_block_launches(self, expand, dw, project, n, h, w):
         r = self.lib.otter_hip_conv_block_launches(expand.h, dw.h, project.h, n, h, w)
@@ -376,6 +382,7 @@ class Conv:
         ws_bytes = self.L.lib.otter_hip_conv_workspace_bytes(self.h, in_layout, n, h, w)
         if ws_bytes and workspace is None:
             workspace = self.L.empty(ws_bytes, np.int8)
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0  # what the buffer really holds
         self.L._check(self.L.lib.otter_hip_conv_forward(
             self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout,
             self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))

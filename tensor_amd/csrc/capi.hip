@@ -96,6 +96,7 @@ struct otter_hip_conv {
     int8_t* w_stem = nullptr;    // MFMA lane order of the few-channel 3x3 kernel (C <= 5, K <= 64)
     int32_t* w_dw = nullptr;     // dot4 weight words          (depthwise, C % 8 == 0)
     int8_t* w_dw_mfma = nullptr; // block-diagonal MFMA operands (depthwise 3x3, C % 8 == 0)
+    int8_t* w_xdw = nullptr;     // MFMA operands of a pointwise int8 -> int8 layer for the launch it shares with its depthwise reader
     int32_t* blk_consts = nullptr; // the layer's constants (and depthwise 3x3 weights) as the fused block launch keeps them in LDS
     bool so_positive = true;     // every output scale is finite and > 0
     float* scale_in = nullptr;   // [Kpad]
@@ -215,6 +216,7 @@ int otter_hip_conv_destroy(otter_hip_conv_t* h) {
     (void)hipFree(h->w_stem);
     (void)hipFree(h->w_dw);
     (void)hipFree(h->w_dw_mfma);
+    (void)hipFree(h->w_xdw);
     (void)hipFree(h->blk_consts);
     (void)hipFree(h->scale_in);
     (void)hipFree(h->bias);
@@ -315,6 +317,12 @@ int otter_hip_conv_create(const otter_hip_conv_desc* desc, const int8_t* weight,
             std::vector<int8_t> wp(igemm_packed_weight_bytes(K, C, d.kernel_h, d.kernel_w));
             igemm_pack_weights(weight, K, C, d.kernel_h, d.kernel_w, wp.data());
             if ((rc = upload<int8_t>(&h->w_igemm, wp.data(), wp.size(), wp.size(), 0))) break;
+            if (maxk == 1 && d.out_kind == OTTER_HIP_OUT_I8 && K % 16 == 0 && C <= 128 && d.stride_h == 1 && d.stride_w == 1 &&
+                d.pad_h == 0 && d.pad_w == 0) {
+                std::vector<int8_t> wx(xdw_weight_bytes(C, K));
+                xdw_pack_weights(weight, C, K, wx.data());
+                if ((rc = upload<int8_t>(&h->w_xdw, wx.data(), wx.size(), wx.size(), 0))) break;
+            }
         } else if (g > 1 && !h->depthwise && (C / g) % 8 == 0) {
             // grouped: every group's weights packed by itself (one launch, a group per grid.z slice)
             std::vector<int8_t> wp(igemm_grouped_weight_bytes(K, C, g, d.kernel_h, d.kernel_w));
@@ -843,6 +851,25 @@ static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_
     return g[0].C <= 192 && g[0].W <= 28 && wgs >= 128 && wgs <= 512 && items <= 24;
 }
 
+// The first two layers of a block as one launch (conv_xdw.hip), the last by itself: where the single launch of the
+// whole block is not taken. 0: where it was measured faster than the two layers one by one; 1: wherever the kernel
+// takes the shapes; -1: never.
+static int g_block_pair = 0;
+
+static bool block_pair_launch(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const ConvGeom g[3]) {
+    if (g_block_pair < 0 || !e->w_xdw || e->c_pad || e->force_tm || !d->w_dw_mfma || d->c_pad || d->force_tm) return false;
+    const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8);
+    if (!xdw_applicable(g[0], e1, pick_epilogue(e1, g[0].K), e->so_positive, g[1], e2, dw_mfma_epilogue(e2, g[1].K), d->so_positive))
+        return false;
+    if (g[0].C > 32 && g[0].W > 64) return false;  // (those instances of the kernel do not fit the register file)
+    if (g_block_pair > 0) return true;
+    // Measured at batch 64 against the two layers one by one (kernel trace): with a stride-2 depthwise layer, where the
+    // expanded blob is four times what the launch writes, 16 -> 96 @112x112 29.5 us against 46, 24 -> 144 @56x56 17.9
+    // against 27, 32 -> 192 @28x28 9.7 against 15, 96 -> 576 @14x14 13.2 against 15; with stride 1 24 -> 144 @56x56 28.6
+    // against 31, and the 88 / 176-channel units of the detection model at 52x52 .. 13x13 (batch 16) no gain.
+    return g[1].sh == 2 || (size_t)g[0].N * g[0].K * g[0].OH * g[0].OW >= ((size_t)16 << 20);
+}
+
 static int block_default_out_layout(const otter_hip_conv_t* p) {
     return p->d.out_kind == OTTER_HIP_OUT_F32 ? OTTER_HIP_F32_P4 : OTTER_HIP_I8_P8;
 }
@@ -854,7 +881,8 @@ int otter_hip_conv_block_launches(const otter_hip_conv_t* e, const otter_hip_con
     ConvGeom g[3];
     if (!block_geoms(e, d, p, n, in_h, in_w, g)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_block_launches: empty output");
     int plan[6];
-    return n >= 1 && p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p), plan) ? 1 : 3;
+    if (n >= 1 && p->d.out_channels % 8 == 0 && block_single_launch(e, d, p, g, block_default_out_layout(p), plan)) return 1;
+    return n >= 1 && block_pair_launch(e, d, g) ? 2 : 3;
 }
 
 size_t otter_hip_conv_block_workspace_bytes(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
@@ -889,6 +917,12 @@ int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_ch
 int otter_hip_conv_block_set_always(int on) {
     const int before = g_block_always;
     if (on >= 0) g_block_always = on ? 1 : 0;
+    return before;
+}
+
+int otter_hip_conv_block_set_pair(int mode) {
+    const int before = g_block_pair;
+    if (mode >= -1 && mode <= 1) g_block_pair = mode;
     return before;
 }
 
@@ -947,10 +981,17 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* e, const otter_hip_conv
                                            "otter_hip_conv_block_workspace_bytes");
     void* t0 = workspace;
     void* t1 = (char*)workspace + (b0 + 255) / 256 * 256;
-    rc = conv_forward(e, in, OTTER_HIP_I8_P8, n, in_h, in_w, t0, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
-    if (rc) return rc;
-    rc = conv_forward(d, t0, OTTER_HIP_I8_P8, n, g[1].H, g[1].W, t1, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
-    if (rc) return rc;
+    if (block_pair_launch(e, d, g)) {
+        // the pointwise layer and its depthwise reader in one launch: the expanded blob is not made
+        const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8);
+        OHIP_CHECK(run_conv_xdw((const int8_t*)in, e->w_xdw, d->w_dw_mfma, t1, g[0], e1, g[1], e2, dw_mfma_epilogue(e2, g[1].K),
+                                e->block_rb, stream));
+    } else {
+        rc = conv_forward(e, in, OTTER_HIP_I8_P8, n, in_h, in_w, t0, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
+        if (rc) return rc;
+        rc = conv_forward(d, t0, OTTER_HIP_I8_P8, n, g[1].H, g[1].W, t1, OTTER_HIP_I8_P8, nullptr, 0, stream_, nullptr, 0.f, 0);
+        if (rc) return rc;
+    }
     return conv_forward(p, t1, OTTER_HIP_I8_P8, n, g[2].H, g[2].W, out, out_layout, nullptr, 0, stream_, (int8_t*)out_q, q_scale,
                         q_round_mode, residual);
 }

@@ -66,6 +66,13 @@ void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks,
 int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 // the same layer straight from an fp32 Float8 blob (quantize + depthwise convolution in one launch)
+// pointwise int8 -> int8 convolution + depthwise 3x3 int8 -> int8 convolution as one launch (conv_xdw.hip)
+size_t xdw_weight_bytes(int Cin, int K);
+void xdw_pack_weights(const int8_t* w, int Cin, int K, int8_t* dst);
+bool xdw_applicable(const ConvGeom& gx, const Epilogue& epx, int epi_x, bool sox_positive, const ConvGeom& gd, const Epilogue& ep,
+                    int epi_d, bool so_positive);
+hipError_t run_conv_xdw(const int8_t* x, const int8_t* wx, const int8_t* wa, void* out, const ConvGeom& gx, const Epilogue& epx,
+                        const ConvGeom& g, const Epilogue& ep, int epi_d, int strip_rows, hipStream_t stream);
 bool dw_f32in_applicable(const ConvGeom& g, int in_layout);
 hipError_t run_conv_dw_f32in(const float* x, const int8_t* wa, void* out, const ConvGeom& g, const Epilogue& ep, int epi,
                              const float* in_scale, int in_round_mode, int strip_rows, hipStream_t stream);

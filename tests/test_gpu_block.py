@@ -28,12 +28,12 @@ def quantize_weights(wf):
     return wq, ws
 
 
-def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1, out_round=capi.ROUND_SSE):
+def make_block(hip, rng, cin, ce, cout, act, f32_out, stride=1, out_round=capi.ROUND_SSE, dw_pad=1):
     """The three layers as a MobileNetV2 block has them: expand and depthwise with `act` and int8 results, a linear
     project layer with an fp32 or int8 result."""
     layers = []
     in_scale = np.float32(rng.uniform(20, 60))
-    specs = [(cin, ce, 1, 1, 0, 1, act, True), (ce, ce, 3, stride, 1, ce, act, True), (ce, cout, 1, 1, 0, 1, 0, not f32_out)]
+    specs = [(cin, ce, 1, 1, 0, 1, act, True), (ce, ce, 3, stride, dw_pad, ce, act, True), (ce, cout, 1, 1, 0, 1, 0, not f32_out)]
     for (ci, co, k, s, pad, groups, a, i8) in specs:
         wq, ws = quantize_weights(rng.normal(0, 0.3 if groups > 1 else 2.0 / np.sqrt(ci), (co, ci // groups, k, k)).astype(np.float32))
         bias = rng.normal(0, 0.05, co).astype(np.float32)
@@ -228,7 +228,7 @@ def test_block_replayed_from_a_captured_graph(hip):
 def test_default_policy_takes_the_measured_shapes_only(hip):
     hip.conv_block_set_always(0)
     rng = np.random.default_rng(3)
-    for (cin, ce, cout, n, hw, want) in [(64, 384, 64, 64, 14, 1), (32, 192, 32, 64, 28, 1), (24, 144, 24, 64, 56, 3),
+    for (cin, ce, cout, n, hw, want) in [(64, 384, 64, 64, 14, 1), (32, 192, 32, 64, 28, 1), (24, 144, 24, 64, 56, 2),
                                           (160, 960, 160, 64, 7, 1), (160, 960, 320, 64, 7, 1), (96, 576, 96, 64, 14, 1), (64, 384, 64, 4, 14, 3),
                                           (64, 384, 64, 16, 14, 1)]:
         layers = make_block(hip, rng, cin, ce, cout, 3, True)
@@ -239,13 +239,14 @@ def test_default_policy_takes_the_measured_shapes_only(hip):
 
 
 def test_block_falls_back_to_three_launches(hip):
-    """A stride-2 depthwise layer is not what the single launch takes: the same call runs the layers one by one."""
+    """A stride-2 depthwise layer is not what the single launch takes, and 160 input channels are more than the launch
+    of the first two layers takes: the same call runs the layers one by one."""
     rng = np.random.default_rng(5)
-    layers = make_block(hip, rng, 32, 192, 64, 3, True, stride=2)
+    layers = make_block(hip, rng, 160, 192, 64, 3, True, stride=2)
     e, d, p = (l["conv"] for l in layers)
     N, H, W = 2, 28, 28
     assert hip.conv_block_launches(e, d, p, N, H, W) == 3
-    x = rng.integers(-127, 128, (N, 32, H, W)).astype(np.int8)
+    x = rng.integers(-127, 128, (N, 160, H, W)).astype(np.int8)
     xd = hip.to_device(capi.pack_np(x, 8))
     got, got_q = hip.conv_block(e, d, p, xd, N, H, W, q_scale=30.0)
     t = e.forward(xd, capi.I8_P8, N, H, W, capi.I8_P8)

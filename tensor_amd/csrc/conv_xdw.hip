@@ -38,7 +38,7 @@ void xdw_pack_weights(const int8_t* w, int Cin, int K, int8_t* dst) {
 }
 
 template <int S, int EPI, bool XNN, int NG, int CK>
-__global__ void __launch_bounds__(256, 2) conv_xdw_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wx,
+__global__ void __launch_bounds__(256, ((CK == 32 && (NG <= 4 || S == 2)) || (S == 2 && NG <= 4)) ? 3 : 2) conv_xdw_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wx,
                                                        const int8_t* __restrict__ wa, void* __restrict__ out, ConvGeom g, int cin,
                                                        Epilogue epx, Epilogue ep, int n_strips, int rps, unsigned in_bytes,
                                                        unsigned out_bytes) {
@@ -174,6 +174,10 @@ __global__ void __launch_bounds__(256, 2) conv_xdw_kernel(const int8_t* __restri
             si[oo][t] = *reinterpret_cast<const v4i*>(ep.scale_in + ch + 4 * t);
             bi[oo][t] = *reinterpret_cast<const v4i*>(ep.bias + ch + 4 * t);
             so[oo][t] = *reinterpret_cast<const v4i*>(ep.scale_out + ch + 4 * t);
+            // the bias is the fma's vector operand in every row: keep it resident (the compiler would otherwise re-copy
+            // it from scalar registers value after value)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(bi[oo][t][e]));
             if constexpr (EPI == EPI_I8_P8_NONNEG) {
                 qh[oo][t][0] = dw_clamp_pair(ep, so[oo][t][0], so[oo][t][1]);
                 qh[oo][t][1] = dw_clamp_pair(ep, so[oo][t][2], so[oo][t][3]);
@@ -290,16 +294,23 @@ hipError_t run_conv_xdw(const int8_t* x, const int8_t* wx, const int8_t* wa, voi
     if (g.N == 0 || g.OH * g.OW == 0) return hipSuccess;
     const long planes = (long)g.N * (g.C / 16);
     if (planes > 65535) return hipErrorInvalidValue;
-    // strips of equal height, about two waves per SIMD over the chip, four strips (waves) to a workgroup where the
-    // rows allow
+    // Strips of equal height. The kernel is bound by the vector instructions of its rows, so the launch lasts about as
+    // long as the busiest of the chip's 1024 SIMDs: (waves per SIMD, rounded up) x (input rows a wave walks + about two
+    // rows' worth of set-up). More strips balance the SIMDs better and recompute more halo rows; take the count that
+    // minimises the product, the fewest strips among equals.
     int rps;
     if (strip_rows > 0) {
         rps = std::min(strip_rows, g.OH);
     } else {
-        int ns = 1;
-        while (ns < g.OH && ns * planes < 2048) ++ns;
-        if (ns > 2 && ns % 4 && (ns + 3) / 4 * 4 <= g.OH) ns = (ns + 3) / 4 * 4;
-        rps = (g.OH + ns - 1) / ns;
+        long best = -1;
+        rps = g.OH;
+        for (int r = g.OH; r >= 1; --r) {
+            const int ns = (g.OH + r - 1) / r;
+            const long per_simd = (planes * ns + 1023) / 1024;
+            // (a lone wave issues a vector instruction every 6 cycles where two or more reach the pipe's 4)
+            const long cost = per_simd * ((r - 1) * g.sh + 3 + 2) * (per_simd == 1 ? 15 : per_simd == 2 ? 11 : 10);
+            if (best < 0 || cost < best) best = cost, rps = r;
+        }
     }
     const int n_strips = (g.OH + rps - 1) / rps;
     const int wpb = n_strips % 4 == 0 ? 4 : (n_strips % 2 == 0 ? 2 : 1);

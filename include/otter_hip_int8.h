@@ -344,6 +344,17 @@ int otter_hip_activation(float* x, size_t count, int activation_type, float acti
  * (Tensor/LayerDeclaration.hpp:42-68); this is the fp32 mean over H*W that the MobileNetV2-style network needs. */
 int otter_hip_global_avgpool(const float* src, int src_layout, int n, int c, int h, int w, float* dst, void* stream);
 
+/* ConvolutionLayer::forward_int8 (Tensor/ConvolutionLayer.cpp:754-847) of a layer with an fp32 result, followed by the
+ * mean over H*W of that result to out[N, K] (what otter_hip_global_avgpool computes; the tail of a classifier). For a
+ * pointwise layer on a Byte8 input and an image of at most 64 pixels it is ONE launch and the layer's own blob is
+ * never made (otter_hip_conv_avgpool_launches says 1, the workspace is 0 bytes); otherwise the layer runs into
+ * `workspace` and the mean is taken from there. The convolution's values are those of otter_hip_conv_forward bit for
+ * bit; their sum is taken in another order than otter_hip_global_avgpool takes it (fp32, same tolerance). */
+int otter_hip_conv_avgpool_launches(const otter_hip_conv_t* conv, int in_layout, int n, int in_h, int in_w);
+size_t otter_hip_conv_avgpool_workspace_bytes(const otter_hip_conv_t* conv, int in_layout, int n, int in_h, int in_w);
+int otter_hip_conv_forward_avgpool(const otter_hip_conv_t* conv, const void* in, int in_layout, int n, int in_h, int in_w,
+                                   float* out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* InnerProductLayer::forward, fp32 (Tensor/InnerProductLayer.cpp:176-): y[n][o] = sum_i x[n][i]*weight[o][i] + bias[o].
  * bias may be NULL. */
 int otter_hip_inner_product(const float* x, int n, int in_features, const float* weight, const float* bias,

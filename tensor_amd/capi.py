@@ -77,6 +77,7 @@ EXPORTS = ["otter_hip_init", "otter_hip_shutdown", "otter_hip_last_error", "otte
            "otter_hip_conv_chain_last_launches", "otter_hip_conv_chain_clock_mhz",
            "otter_hip_conv_chain_set_min_tiles", "otter_hip_conv_block_launches", "otter_hip_conv_block_workspace_bytes",
            "otter_hip_conv_block_forward", "otter_hip_conv_block_set_plan", "otter_hip_conv_block_set_always", "otter_hip_conv_block_set_pair",
+           "otter_hip_conv_avgpool_launches", "otter_hip_conv_avgpool_workspace_bytes", "otter_hip_conv_forward_avgpool",
            "otter_hip_conv_block_plan"]
 
 
@@ -100,6 +101,7 @@ class Library:
         L.otter_hip_conv_workspace_bytes.restype = C.c_size_t
         L.otter_hip_conv_chain_workspace_bytes.restype = C.c_size_t
         L.otter_hip_conv_block_workspace_bytes.restype = C.c_size_t
+        L.otter_hip_conv_avgpool_workspace_bytes.restype = C.c_size_t
         self.device = torch.device("cuda", device)
         self._check(L.otter_hip_init(C.c_int(device)))
 
@@ -254,6 +256,12 @@ class Library:
     def conv(self, **kw):
         return Conv(self, **kw)
 
+    def global_avgpool(self, x, layout, n, c, h, w):
+        """otter_hip_global_avgpool: the mean over H*W of an fp32 blob, [n, c]."""
+        out = self.empty(n * c, np.float32)
+        self._check(self.lib.otter_hip_global_avgpool(self.ptr(x), layout, n, c, h, w, self.ptr(out), self.stream()))
+        return out
+
     def conv_chain(self, convs, x, n, h, w, out=None, workspace=None):
         """otter_hip_conv_chain_forward: x (int8 Byte8) through the layers `convs`, intermediate blobs in `workspace`."""
         hs = (C.c_void_p * len(convs))(*[c.h for c in convs])
@@ -385,6 +393,21 @@ class Conv:
         ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0  # what the buffer really holds
         self.L._check(self.L.lib.otter_hip_conv_forward(
             self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out), out_layout,
+            self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))
+        return out
+
+    def avgpool_launches(self, in_layout, n, h, w):
+        r = self.L.lib.otter_hip_conv_avgpool_launches(self.h, in_layout, n, h, w)
+        self.L._check(min(r, 0))
+        return r
+
+    def forward_avgpool(self, x, in_layout, n, h, w):
+        """otter_hip_conv_forward_avgpool: the layer's fp32 result averaged over the image, [n, K]."""
+        out = self.L.empty(n * self.K, np.float32)
+        ws_bytes = self.L.lib.otter_hip_conv_avgpool_workspace_bytes(self.h, in_layout, n, h, w)
+        workspace = self.L.empty(ws_bytes, np.int8) if ws_bytes else None
+        self.L._check(self.L.lib.otter_hip_conv_forward_avgpool(
+            self.h, self.L.ptr(x), in_layout, n, h, w, self.L.ptr(out),
             self.L.ptr(workspace) if workspace is not None else None, C.c_size_t(ws_bytes), self.L.stream()))
         return out
 

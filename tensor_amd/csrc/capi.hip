@@ -1103,6 +1103,58 @@ int otter_hip_global_avgpool(const float* src, int src_layout, int n, int c, int
     return OTTER_HIP_OK;
 }
 
+// ---- a convolution with an fp32 result and the global average pooling that is its only reader ----------------------
+
+static bool conv_avgpool_one_launch(const otter_hip_conv_t* h, int in_layout, const ConvGeom& g) {
+    if (in_layout != OTTER_HIP_I8_P8 || !h->w_igemm || h->c_pad || h->force_tm || h->d.out_kind != OTTER_HIP_OUT_F32) return false;
+    return conv_pw_avgpool_applicable(g, make_epilogue(h, otter_hip_conv_default_out_layout(h)));
+}
+
+int otter_hip_conv_avgpool_launches(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w) {
+    if (!h || !valid_layout(in_layout) || n < 0 || in_h < 1 || in_w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_avgpool_launches: bad argument");
+    if (h->d.out_kind != OTTER_HIP_OUT_F32) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_avgpool_launches: the layer must have an fp32 result");
+    const ConvGeom g = make_geom(h->d, n, in_h, in_w);
+    if (g.OH < 1 || g.OW < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_avgpool_launches: empty output");
+    return conv_avgpool_one_launch(h, in_layout, g) ? 1 : 2;
+}
+
+size_t otter_hip_conv_avgpool_workspace_bytes(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w) {
+    if (!h || !valid_layout(in_layout) || n < 1 || in_h < 1 || in_w < 1 || h->d.out_kind != OTTER_HIP_OUT_F32) return 0;
+    const ConvGeom g = make_geom(h->d, n, in_h, in_w);
+    if (g.OH < 1 || g.OW < 1 || conv_avgpool_one_launch(h, in_layout, g)) return 0;
+    const size_t ws = otter_hip_conv_workspace_bytes(h, in_layout, n, in_h, in_w);
+    return (ws + 255) / 256 * 256 + (size_t)n * g.K * g.OH * g.OW * sizeof(float);
+}
+
+int otter_hip_conv_forward_avgpool(const otter_hip_conv_t* h, const void* in, int in_layout, int n, int in_h, int in_w, float* out,
+                                   void* workspace, size_t workspace_bytes, void* stream_) {
+    if (!h || !in || !out) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_avgpool: null");
+    if (!valid_layout(in_layout) || n < 0 || in_h < 1 || in_w < 1)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_avgpool: bad argument");
+    if (h->d.out_kind != OTTER_HIP_OUT_F32)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_avgpool: the layer must have an fp32 result");
+    const ConvGeom g = make_geom(h->d, n, in_h, in_w);
+    if (g.OH < 1 || g.OW < 1) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_avgpool: empty output");
+    if (n == 0) return OTTER_HIP_OK;
+    if (conv_avgpool_one_launch(h, in_layout, g)) {
+        const Epilogue ep = make_epilogue(h, otter_hip_conv_default_out_layout(h));
+        OHIP_CHECK(run_conv_pw_avgpool((const int8_t*)in, h->w_igemm, out, g, ep, (hipStream_t)stream_));
+        return OTTER_HIP_OK;
+    }
+    // the layer into the workspace, then the mean of that blob
+    const size_t ws = (otter_hip_conv_workspace_bytes(h, in_layout, n, in_h, in_w) + 255) / 256 * 256;
+    const size_t need = ws + (size_t)n * g.K * g.OH * g.OW * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+        return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_forward_avgpool: needs the workspace reported by "
+                                           "otter_hip_conv_avgpool_workspace_bytes");
+    const int out_layout = otter_hip_conv_default_out_layout(h);
+    float* blob = (float*)((char*)workspace + ws);
+    int rc = conv_forward(h, in, in_layout, n, in_h, in_w, blob, out_layout, ws ? workspace : nullptr, ws, stream_, nullptr, 0.f, 0);
+    if (rc) return rc;
+    return otter_hip_global_avgpool(blob, out_layout, n, g.K, g.OH, g.OW, out, stream_);
+}
+
 int otter_hip_inner_product(const float* x, int n, int in_features, const float* weight, const float* bias,
                             int out_features, float* y, void* stream) {
     if (!x || !weight || !y) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_inner_product: null");

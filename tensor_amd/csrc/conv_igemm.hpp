@@ -66,6 +66,10 @@ void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks,
 int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 // the same layer straight from an fp32 Float8 blob (quantize + depthwise convolution in one launch)
+// pointwise int8 convolution with an fp32 result + the mean over the image, one launch (conv_pw.hip)
+bool conv_pw_avgpool_applicable(const ConvGeom& g, const Epilogue& ep);
+hipError_t run_conv_pw_avgpool(const int8_t* x, const int8_t* wpk, float* out, const ConvGeom& g, const Epilogue& ep,
+                               hipStream_t stream);
 // pointwise int8 -> int8 convolution + depthwise 3x3 int8 -> int8 convolution as one launch (conv_xdw.hip)
 size_t xdw_weight_bytes(int Cin, int K);
 void xdw_pack_weights(const int8_t* w, int Cin, int K, int8_t* dst);

@@ -221,4 +221,81 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
     return hipErrorInvalidValue;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// A pointwise int8 convolution with an fp32 result whose only reader is the mean over the image (the tail of a
+// classifier: head convolution, global average pooling): out[n][k] = mean over H*W of activation(acc * scale_in + bias),
+// one launch, the convolution's own blob (H*W times the size of the result) never written or read back.
+// A wave owns a pair of 16-row tiles (32 output channels, igemm_row_channel) x all pixels of one image (at most 64: four
+// groups of 16 as the B operands of every reduction step, loaded straight from the Byte8 blob; the four waves of a
+// workgroup read the same pixels, which the first one brings into the CU's cache). After the last step a lane holds,
+// per tile, four channels of its pixel in each group: it adds the activated values of its groups, the 16 lanes of a
+// row group add theirs (xor butterfly), and lane 0 of the group stores four means.
+__global__ void __launch_bounds__(256) conv_pw_avgpool_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
+                                                              float* __restrict__ out, ConvGeom g, Epilogue ep, int cgs,
+                                                              int mt16) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, q = lane >> 4;
+    const int pair = blockIdx.x * 4 + wave, img = blockIdx.y;
+    if (2 * pair >= mt16) return;  // whole wave
+    const int HW = g.H * g.W, C8 = g.C / 8;
+    v4i acc[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) acc[t][p] = v4i{0, 0, 0, 0};
+    const v4i* wv = reinterpret_cast<const v4i*>(wpk);
+    const v2i* xv = reinterpret_cast<const v2i*>(x) + (size_t)img * C8 * HW;
+    for (int cg = 0; cg < cgs; ++cg) {
+        const v4i a0 = wv[((size_t)cg * mt16 + 2 * pair) * 64 + lane];
+        const v4i a1 = 2 * pair + 1 < mt16 ? wv[((size_t)cg * mt16 + 2 * pair + 1) * 64 + lane] : v4i{0, 0, 0, 0};
+        const int oct = cg * 8 + 2 * q;
+        v4i b[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int pix = 16 * p + n;
+            const v2i lo = (pix < HW && oct < C8) ? xv[(size_t)oct * HW + pix] : v2i{0, 0};
+            const v2i hi = (pix < HW && oct + 1 < C8) ? xv[(size_t)(oct + 1) * HW + pix] : v2i{0, 0};
+            b[p] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            acc[0][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b[p], acc[0][p], 0, 0, 0);
+            acc[1][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b[p], acc[1][p], 0, 0, 0);
+        }
+    }
+    const float count = (float)HW;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int ch0 = 32 * pair + 8 * q + 4 * t;  // igemm_row_channel of rows 4q .. 4q+3 of tile 2 pair + t
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ch = ch0 + e;
+            const bool live = ch < g.K;
+            const float si = live ? ep.scale_in[ch] : 0.f, bi = live ? ep.bias[ch] : 0.f;
+            float s = 0.f;
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                if (16 * p + n < HW) s += activate(__fmaf_rn((float)acc[t][p][e], si, bi), ep.act, ep.act_p0);
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) s += __shfl_xor(s, o, 16);
+            if (n == 0 && live) out[(size_t)img * g.K + ch] = s / count;
+        }
+    }
+}
+
+bool conv_pw_avgpool_applicable(const ConvGeom& g, const Epilogue& ep) {
+    if (g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph || g.pw || g.groups != 1 || g.C % 8) return false;
+    if (ep.out_kind != OTTER_HIP_OUT_F32 || ep.twin || ep.residual) return false;
+    if ((size_t)g.N * g.C * g.H * g.W >= ((size_t)1 << 31)) return false;
+    return g.H * g.W <= 64 && g.N <= 65535;
+}
+
+hipError_t run_conv_pw_avgpool(const int8_t* x, const int8_t* wpk, float* out, const ConvGeom& g, const Epilogue& ep,
+                               hipStream_t stream) {
+    if (g.N == 0) return hipSuccess;
+    const int mt16 = igemm_padded_rows(g.K) / 16, pairs = (mt16 + 1) / 2;
+    hipLaunchKernelGGL(conv_pw_avgpool_kernel, dim3((unsigned)((pairs + 3) / 4), (unsigned)g.N), dim3(256), 0, stream, x, wpk, out, g,
+                       ep, igemm_channel_groups(g.C), mt16);
+    return hipGetLastError();
+}
+
 }  // namespace ohip

@@ -614,6 +614,28 @@ int ConvolutionLayer::forward_residual(const Tensor& bottom, const Tensor& short
     return forward_int8(bottom, &shortcut, q_scale, q_round, sum, opt);
 }
 
+int ConvolutionLayer::forward_avgpool(const Tensor& bottom_in, Tensor& mean, const NetOption& opt) const {
+    if (!handle_ || !int8_scale_term || int8_scale_term > 100 || force_out_layout >= 0 || !opt.use_packing_layout) return 1;
+    if (!bottom_in.defined() || bottom_in.dim() != 4) return 1;
+    Tensor bottom = bottom_in, twin;
+    if (base_of(bottom_in.scalar_type()) == ScalarType::Float && in_channels % 8 == 0 &&
+        bottom_in.quantized_twin(bottom_blob_int8_scales.data_ptr<float>()[0], input_round_mode(opt), twin))
+        bottom = twin;
+    if (bottom.scalar_type() != ScalarType::Byte8 || bottom.channels() != in_channels) return 1;
+    const int N = (int)bottom.size(0), H = (int)bottom.size(2), W = (int)bottom.size(3);
+    if (otter_hip_conv_avgpool_launches(handle_, OTTER_HIP_I8_P8, N, H, W) != 1) return 1;
+    try {
+        mean = Tensor::empty_device({N, out_channels, 1, 1}, ScalarType::Float);
+        const int rc = otter_hip_conv_forward_avgpool(handle_, bottom.device_ptr(), OTTER_HIP_I8_P8, N, H, W,
+                                                      (float*)mean.device_ptr(), nullptr, 0, nullptr);
+        if (rc) return rc;
+        mean.mark_device_written();
+    } catch (const Error&) {
+        return -100;
+    }
+    return 0;
+}
+
 // Tensor/ConvolutionLayer.cpp:754-847, whole batch in one launch; with `shortcut` the Eltwise sum behind it as well
 int ConvolutionLayer::forward_int8(const Tensor& bottom_in, const Tensor* shortcut, float q_scale, int q_round, Tensor& top,
                                    const NetOption& opt) const {
@@ -1662,6 +1684,26 @@ int Net::forward_layer(int li, std::vector<Tensor>& blobs, const NetOption& opt)
         }
     }
     {
+        const auto unit = pool_units_.find(li);
+        // only when the convolution's own result has not been computed (or set by the caller)
+        if (unit != pool_units_.end() && !blobs[layers_[unit->second]->tops[0]].defined()) {
+            const auto* conv = static_cast<const ConvolutionLayer*>(layers_[unit->second]);
+            const int b = conv->bottoms[0];
+            if (!blobs[b].defined()) {
+                const int rc = forward_layer(blobs_[b].producer, blobs, opt);
+                if (rc) return rc;
+            }
+            Tensor mean;
+            const int rc = conv->forward_avgpool(blobs[b], mean, opt);
+            if (rc < 0) return rc;
+            if (rc == 0) {
+                blobs[layer->tops[0]] = mean;
+                if (opt.lightmode && blobs_[b].consumers.size() == 1) blobs[b] = Tensor();
+                return 0;
+            }
+        }
+    }
+    {
         const auto unit = block_units_.find(li);
         // only when neither blob inside the block has been computed (or set by the caller) yet
         if (unit != block_units_.end() && !blobs[layers_[unit->second.expand]->tops[0]].defined() &&
@@ -1763,6 +1805,17 @@ void Net::plan_fused_quantize() const {
             if (best < 0 || pi > blobs_[e->bottoms[best]].producer) best = k;  // the later one: the other is ready by then
         }
         if (best >= 0) residual_units_[(int)ei] = ResidualUnit{blobs_[e->bottoms[best]].producer, (int)ei, e->bottoms[1 - best]};
+    }
+    // Classifier tails: a GlobalAvgPool layer on the fp32 result of an int8 convolution read by nothing else
+    pool_units_.clear();
+    for (size_t pi = 0; pi < layers_.size(); ++pi) {
+        const Layer* p = layers_[pi];
+        if (p->type() != "GlobalAvgPool" || p->bottoms.size() != 1) continue;
+        const int b = p->bottoms[0], ci = blobs_[b].producer;
+        const auto* pc = ci < 0 ? nullptr : dynamic_cast<const ConvolutionLayer*>(layers_[ci]);
+        if (!pc || !pc->int8_scale_term || pc->int8_scale_term > 100 || pc->force_out_layout >= 0 || pc->bottoms.size() != 1) continue;
+        if (blobs_[b].consumers.size() != 1) continue;
+        pool_units_[(int)pi] = ci;
     }
     // ShuffleNetV2 unit tails: Concat of two equal blobs -> ChannelShuffle(2) -> exactly the two half Crops
     shuffle_units_.clear();

@@ -214,6 +214,10 @@ public:
     // have the layouts that takes (the caller then runs the two layers one after the other).
     int forward_residual(const Tensor& bottom_blob, const Tensor& shortcut, float q_scale, int q_round, Tensor& sum,
                          const NetOption& opt) const;
+    // This layer (fp32 result) and the global average pooling that is its only reader through
+    // otter_hip_conv_forward_avgpool, when that is one launch for this input; `mean` is [N, K, 1, 1]. Returns 1, and does
+    // nothing, otherwise (the caller then runs the two layers one after the other).
+    int forward_avgpool(const Tensor& bottom_blob, Tensor& mean, const NetOption& opt) const;
     // A run of int8 -> int8 convolution layers, each reading the one before, as one call of the C ABI's chain entry point
     // when that takes the run as a single launch (otter_hip_conv_chain_launches == 1); `top` is the last layer's blob,
     // the blobs in between are not made. Returns 1, and does nothing, for any other run or input.
@@ -323,6 +327,10 @@ private:
     };
     mutable std::map<int, ResidualUnit> residual_units_;
     int forward_residual_unit(const ResidualUnit& u, std::vector<Tensor>& blobs, const NetOption& opt) const;
+    // The tail of a classifier, found by the plan: a GlobalAvgPool layer whose input is the fp32 result of an int8
+    // convolution that nothing else reads. Pooling layer's index -> the convolution's; forward_layer hands both to
+    // ConvolutionLayer::forward_avgpool when the convolution's result does not exist yet.
+    mutable std::map<int, int> pool_units_;
     // Runs of 2..8 int8 -> int8 convolution layers, each read only by the next, found by the plan: last layer's index ->
     // the run; forward_layer hands the run to ConvolutionLayer::forward_chain when none of its blobs exists yet.
     // Inverted-residual blocks, found by the plan: a 1x1 convolution whose only input is the int8 result of a depthwise

@@ -348,10 +348,11 @@ def build_layer(hip, capi, rng, name):
                 layer=(C, K, k, s, p, d, g))
 
 
-def build_block(hip, capi, rng, N=64, cin=64, ce=384, cout=64, hw=14):
-    """One inverted-residual block of the MobileNetV2-style network (1x1 expand, depthwise 3x3, 1x1 project, shortcut sum,
-    int8 twin of the sum) at 14x14, batch 64: a step is otter_hip_conv_block_forward (one launch); the same block as
-    three launches (forward, forward, forward_residual) is timed beside it."""
+def build_block(hip, capi, rng, N=64, cin=64, ce=384, cout=64, hw=14, stride=1, name="blk14"):
+    """One inverted-residual block of the MobileNetV2-style network (1x1 expand, depthwise 3x3, 1x1 project, shortcut sum
+    where the shapes allow one, int8 twin of the result): a step is otter_hip_conv_block_forward (blk14, 14x14 stride 1:
+    one launch; blk112s2, 112x112 with a stride-2 depthwise layer: one launch for the first two layers, one for the
+    last); the same block as three launches (forward, forward, forward_residual / _twin) is timed beside it."""
     layers = []
     in_scale = np.float32(40.0)
     for (ci, co, k, pad, groups, act, i8) in [(cin, ce, 1, 0, 1, 3, True), (ce, ce, 3, 1, ce, 3, True), (ce, cout, 1, 0, 1, 0, False)]:
@@ -359,38 +360,47 @@ def build_block(hip, capi, rng, N=64, cin=64, ce=384, cout=64, hw=14):
         bias = rng.normal(0, 0.05, co).astype(np.float32)
         out_scale = np.float32(25.0)
         conv = hip.conv(wq=wq, scale_in=host_scale_in(ws, in_scale), bias=bias, in_scale=float(in_scale),
-                        out_scale=[out_scale] if i8 else None, pad=(pad, pad), groups=groups, act=act,
-                        out_kind=capi.OUT_I8 if i8 else capi.OUT_F32, out_round=capi.ROUND_SSE)
+                        out_scale=[out_scale] if i8 else None, stride=(stride, stride) if groups > 1 else (1, 1), pad=(pad, pad),
+                        groups=groups, act=act, out_kind=capi.OUT_I8 if i8 else capi.OUT_F32, out_round=capi.ROUND_SSE)
         layers.append(dict(conv=conv, wq=wq, ws=ws, bias=bias, in_scale=float(in_scale), out_scale=float(out_scale), k=k,
-                           pad=pad, groups=groups, act=act, int8_out=i8))
+                           pad=pad, groups=groups, act=act, int8_out=i8, stride=stride if groups > 1 else 1))
         in_scale = out_scale
     e, d, p = (l["conv"] for l in layers)
     x = rng.integers(-127, 128, size=(N, cin, hw, hw), dtype=np.int8)
     xd = hip.to_device(capi.pack_np(x, 8))
-    res = hip.to_device(capi.pack_np(rng.normal(0, 1, (N, cout, hw, hw)).astype(np.float32), 4))
-    out = hip.empty(N * cout * hw * hw, np.float32)
-    q = hip.empty(N * cout * hw * hw, np.int8)
+    oh, _ = d.out_hw(hw, hw)
+    with_res = stride == 1 and cin == cout
+    res = hip.to_device(capi.pack_np(rng.normal(0, 1, (N, cout, oh, oh)).astype(np.float32), 4)) if with_res else None
+    out = hip.empty(N * cout * oh * oh, np.float32)
+    q = hip.empty(N * cout * oh * oh, np.int8)
     t0 = hip.empty(N * ce * hw * hw, np.int8)
-    t1 = hip.empty(N * ce * hw * hw, np.int8)
+    t1 = hip.empty(N * ce * oh * oh, np.int8)
+    ws_bytes = hip.lib.otter_hip_conv_block_workspace_bytes(e.h, d.h, p.h, N, hw, hw)
+    ws = hip.empty(ws_bytes, np.int8) if ws_bytes else None
     launches = hip.conv_block_launches(e, d, p, N, hw, hw)
 
     def step():
-        return hip.conv_block(e, d, p, xd, N, hw, hw, residual=res, q_scale=20.0, out=out, q=q)[0]
+        return hip.conv_block(e, d, p, xd, N, hw, hw, residual=res, q_scale=20.0, out=out, q=q, workspace=ws)[0]
 
     def three():
         e.forward(xd, capi.I8_P8, N, hw, hw, capi.I8_P8, out=t0)
         d.forward(t0, capi.I8_P8, N, hw, hw, capi.I8_P8, out=t1)
-        return p.forward_residual(t1, capi.I8_P8, N, hw, hw, res, q_scale=20.0)[0]
+        if with_res:
+            return p.forward_residual(t1, capi.I8_P8, N, oh, oh, res, q_scale=20.0)[0]
+        return p.forward_twin(t1, capi.I8_P8, N, oh, oh, 20.0, capi.ROUND_SSE)[0]
 
-    px = N * hw * hw
-    ops = 2.0 * px * (cin * ce + 9 * ce + ce * cout)
-    nbytes = px * (cin + 4 * cout + 4 * cout + cout) + cin * ce + 9 * ce + ce * cout  # in, shortcut, out, twin, weights
-    return dict(name="blk14", step=step, ops=ops, launches=launches, dom_ops=ops, dom_bytes=nbytes, bound="hbm",
-                workload="inverted-residual block %d->%d->%d (1x1 ReLU6, depthwise 3x3 ReLU6, 1x1 linear, + shortcut, + int8 "
-                         "twin) @%dx%d, batch %d, through otter_hip_conv_block_forward (%d launch%s)"
-                         % (cin, ce, cout, hw, hw, N, launches, "" if launches == 1 else "es"),
-                dom_kernel="conv_block_kernel (the block's one launch)", dom_fn=None, x=x, step_layers=three,
-                params=layers, shape=(N, cin, hw, hw), _keep=(xd, res, out, q, t0, t1))
+    px, opx = N * hw * hw, N * oh * oh
+    ops = 2.0 * (px * cin * ce + opx * (9 * ce + ce * cout))
+    # in, (shortcut,) out, twin, weights: what the block must move; the blobs between its layers are not in it
+    nbytes = px * cin + opx * ((4 * cout if with_res else 0) + 4 * cout + cout) + cin * ce + 9 * ce + ce * cout
+    how = {1: "one launch", 2: "one launch for the first two layers, one for the last", 3: "three launches"}[launches]
+    return dict(name=name, step=step, ops=ops, launches=launches, dom_ops=ops, dom_bytes=nbytes, bound="hbm",
+                workload="inverted-residual block %d->%d->%d (1x1 ReLU6, depthwise 3x3 stride %d ReLU6, 1x1 linear%s, + int8 "
+                         "twin) @%dx%d, batch %d, through otter_hip_conv_block_forward (%s)"
+                         % (cin, ce, cout, stride, ", + shortcut" if with_res else "", hw, hw, N, how),
+                dom_kernel="conv_block_kernel (the block's one launch)" if launches == 1 else
+                           "conv_xdw_kernel (pointwise + depthwise layer) and the last layer's launch",
+                dom_fn=None, x=x, step_layers=three, params=layers, shape=(N, cin, hw, hw), _keep=(xd, res, out, q, t0, t1, ws))
 
 
 def build_det(hip, capi, rng, batch=16):
@@ -473,6 +483,8 @@ def cpu_baseline(wl, budget_s=15.0):
 def _cpu_baseline(wl, budget_s=15.0):
     from oracle import binding
     name = wl["name"]
+    if name == "copy":  # the counter calibration: nothing of the reference to time
+        return None
     p = wl["params"]
     N, C, H, W = wl["shape"]
     x = wl["x"]
@@ -527,13 +539,13 @@ def _cpu_baseline(wl, budget_s=15.0):
         t = time.perf_counter() - t0
         return dict(value=algo_bytes / t / 1e9, unit="GB/s", cores=O.num_threads(), kind="port",
                     sample="%d images, scalar C restatement" % n_img)
-    if name == "blk14":
+    if name.startswith("blk"):
         n_img = 4
         if R is not None:
             cur, t_all = x[:n_img], 0.0
             for l in p:
                 co, cg, k, _ = l["wq"].shape
-                opts = {"type": "Convolution", "in_channels": cg * l["groups"], "out_channels": co, "kernel": k, "stride": 1,
+                opts = {"type": "Convolution", "in_channels": cg * l["groups"], "out_channels": co, "kernel": k, "stride": l["stride"],
                         "padding": l["pad"], "groups": l["groups"], "int8_scale_term": (101 if l["groups"] > 1 else 102) if l["int8_out"] else 2}
                 if l["act"] == 3:
                     opts["activation"] = "Relu6"
@@ -547,8 +559,9 @@ def _cpu_baseline(wl, budget_s=15.0):
         t0 = time.perf_counter()
         cur = x[:1]
         for l in p:
-            cur = O.conv_layer_forward(cur, l["wq"], l["ws"], l["in_scale"], pad=(l["pad"],) * 2, groups=l["groups"], bias=l["bias"],
-                                       top_scale=l["out_scale"], int8_out=l["int8_out"], act_type=l["act"])
+            cur = O.conv_layer_forward(cur, l["wq"], l["ws"], l["in_scale"], stride=(l["stride"],) * 2, pad=(l["pad"],) * 2,
+                                       groups=l["groups"], bias=l["bias"], top_scale=l["out_scale"], int8_out=l["int8_out"],
+                                       act_type=l["act"])
         t = time.perf_counter() - t0
         return dict(value=wl["ops"] / N / t / 1e12, unit="TOPS", cores=O.num_threads(), kind="port",
                     sample="1 image, C restatement of the three layers")
@@ -798,6 +811,7 @@ def main():
     for lname in LAYER_SHAPES:
         builders[lname] = lambda r, lname=lname: build_layer(hip, capi, r, lname)
     builders["blk14"] = lambda r: build_block(hip, capi, r)
+    builders["blk112s2"] = lambda r: build_block(hip, capi, r, cin=16, ce=96, cout=24, hw=112, stride=2, name="blk112s2")
     if a.workload not in builders:
         print("unknown workload %s (have %s)" % (a.workload, sorted(builders)), file=sys.stderr)
         sys.exit(2)
@@ -861,13 +875,13 @@ def main():
             line["cpu_baseline"] = {"error": str(e)[:200]}
     if not a.no_also:
         also = []
-        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det", "blk14") + tuple(LAYER_SHAPES) + ("copy",):
+        for name in ("c1s1", "c1s2", "c2", "c2i8", "c0", "c0n64", "c4", "det", "blk14", "blk112s2") + tuple(LAYER_SHAPES) + ("copy",):
             if name == a.workload or name not in builders:
                 continue
             w2 = builders[name](np.random.default_rng(0))
             r2 = measure(w2, timer, max(10, a.steps // 2), a.warmup, "")
             entry = dict(name=name, **r2)
-            if name == "blk14":  # the same block as three launches, in the same run
+            if name.startswith("blk"):  # the same block as three launches, in the same run
                 ms3, _ = timer.run(w2["step_layers"], max(10, a.steps // 2), a.warmup)
                 entry["three_launches_ms_per_step"] = ms3
             if name in ("c4", "det"):

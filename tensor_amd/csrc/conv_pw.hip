@@ -230,6 +230,7 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
 // workgroup read the same pixels, which the first one brings into the CU's cache). After the last step a lane holds,
 // per tile, four channels of its pixel in each group: it adds the activated values of its groups, the 16 lanes of a
 // row group add theirs (xor butterfly), and lane 0 of the group stores four means.
+template <int CGS>  // reduction steps of 64 input channels when they are at most 5 (all operands requested at once); 0: a loop
 __global__ void __launch_bounds__(256) conv_pw_avgpool_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                               float* __restrict__ out, ConvGeom g, Epilogue ep, int cgs,
                                                               int mt16) {
@@ -243,23 +244,49 @@ __global__ void __launch_bounds__(256) conv_pw_avgpool_kernel(const int8_t* __re
 #pragma unroll
         for (int p = 0; p < 4; ++p) acc[t][p] = v4i{0, 0, 0, 0};
     const v4i* wv = reinterpret_cast<const v4i*>(wpk);
-    const v2i* xv = reinterpret_cast<const v2i*>(x) + (size_t)img * C8 * HW;
-    for (int cg = 0; cg < cgs; ++cg) {
-        const v4i a0 = wv[((size_t)cg * mt16 + 2 * pair) * 64 + lane];
-        const v4i a1 = 2 * pair + 1 < mt16 ? wv[((size_t)cg * mt16 + 2 * pair + 1) * 64 + lane] : v4i{0, 0, 0, 0};
+    // (every load is unconditional: a pixel or an octet that does not exist carries an offset past the buffer and reads
+    // zero; behind per-lane branches the compiler would wait for each load before it issues the next)
+    const __amdgpu_buffer_rsrc_t rx =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x), 0, (int)((size_t)g.N * g.C * HW), 0x00020000);
+    const unsigned s_img = (unsigned)img * (unsigned)(C8 * HW) * 8u;
+    const int second = 2 * pair + 1 < mt16 ? 1 : 0;  // (an odd tile count: the pair's second tile repeats the first, unused)
+    auto load = [&](int cg, v4i (&a)[2], v4i (&b)[4]) {
+        a[0] = wv[((size_t)cg * mt16 + 2 * pair) * 64 + lane];
+        a[1] = wv[((size_t)cg * mt16 + 2 * pair + second) * 64 + lane];
         const int oct = cg * 8 + 2 * q;
-        v4i b[4];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int pix = 16 * p + n;
-            const v2i lo = (pix < HW && oct < C8) ? xv[(size_t)oct * HW + pix] : v2i{0, 0};
-            const v2i hi = (pix < HW && oct + 1 < C8) ? xv[(size_t)(oct + 1) * HW + pix] : v2i{0, 0};
+            const unsigned v0 = (pix < HW && oct < C8) ? (unsigned)(oct * HW + pix) * 8u : PW_OOB;
+            const unsigned v1 = (pix < HW && oct + 1 < C8) ? (unsigned)((oct + 1) * HW + pix) * 8u : PW_OOB;
+            const v2i lo = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rx, (int)v0, (int)s_img, 0));
+            const v2i hi = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rx, (int)v1, (int)s_img, 0));
             b[p] = v4i{lo[0], lo[1], hi[0], hi[1]};
         }
+    };
+    auto mac = [&](const v4i (&a)[2], const v4i (&b)[4]) {
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            acc[0][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b[p], acc[0][p], 0, 0, 0);
-            acc[1][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b[p], acc[1][p], 0, 0, 0);
+            acc[0][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[0], b[p], acc[0][p], 0, 0, 0);
+            acc[1][p] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[1], b[p], acc[1][p], 0, 0, 0);
+        }
+    };
+    if constexpr (CGS > 0) {
+        v4i a[CGS][2], b[CGS][4];
+#pragma unroll
+        for (int cg = 0; cg < CGS; ++cg) load(cg, a[cg], b[cg]);
+#pragma unroll
+        for (int cg = 0; cg < CGS; ++cg) mac(a[cg], b[cg]);
+    } else {
+        v4i a[2][2], b[2][4];
+        load(0, a[0], b[0]);
+        for (int cg = 0; cg < cgs; cg += 2) {  // the next step's operands are requested before this step's are used
+            load(min(cg + 1, cgs - 1), a[1], b[1]);
+            mac(a[0], b[0]);
+            if (cg + 1 < cgs) {
+                load(min(cg + 2, cgs - 1), a[0], b[0]);
+                mac(a[1], b[1]);
+            }
         }
     }
     const float count = (float)HW;
@@ -270,7 +297,7 @@ __global__ void __launch_bounds__(256) conv_pw_avgpool_kernel(const int8_t* __re
         for (int e = 0; e < 4; ++e) {
             const int ch = ch0 + e;
             const bool live = ch < g.K;
-            const float si = live ? ep.scale_in[ch] : 0.f, bi = live ? ep.bias[ch] : 0.f;
+            const float si = ep.scale_in[ch], bi = ep.bias[ch];  // (the arrays are padded to whole row blocks)
             float s = 0.f;
 #pragma unroll
             for (int p = 0; p < 4; ++p)
@@ -293,8 +320,18 @@ hipError_t run_conv_pw_avgpool(const int8_t* x, const int8_t* wpk, float* out, c
                                hipStream_t stream) {
     if (g.N == 0) return hipSuccess;
     const int mt16 = igemm_padded_rows(g.K) / 16, pairs = (mt16 + 1) / 2;
-    hipLaunchKernelGGL(conv_pw_avgpool_kernel, dim3((unsigned)((pairs + 3) / 4), (unsigned)g.N), dim3(256), 0, stream, x, wpk, out, g,
-                       ep, igemm_channel_groups(g.C), mt16);
+    const int cgs = igemm_channel_groups(g.C);
+    const dim3 grid((unsigned)((pairs + 3) / 4), (unsigned)g.N);
+#define OHIP_PWA(N_) hipLaunchKernelGGL(conv_pw_avgpool_kernel<N_>, grid, dim3(256), 0, stream, x, wpk, out, g, ep, cgs, mt16)
+    switch (cgs) {
+    case 1: OHIP_PWA(1); break;
+    case 2: OHIP_PWA(2); break;
+    case 3: OHIP_PWA(3); break;
+    case 4: OHIP_PWA(4); break;
+    case 5: OHIP_PWA(5); break;
+    default: OHIP_PWA(0); break;
+    }
+#undef OHIP_PWA
     return hipGetLastError();
 }
 

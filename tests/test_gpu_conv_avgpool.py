@@ -17,6 +17,8 @@ CASES = [
     (64, 40, 3, 8, 8, 1, 0, 0, True, 1),      # 64 pixels, K not a multiple of 32, signed values
     (24, 8, 2, 1, 1, 1, 0, 1, False, 1),      # one pixel, one octet of results
     (136, 100, 2, 5, 9, 1, 0, 2, True, 1),    # LeakyReLU, K % 4 == 0 only, 17 input octets
+    (448, 64, 2, 4, 4, 1, 0, 3, True, 1),     # seven reduction steps (the looped form of the kernel, odd count)
+    (384, 32, 1, 3, 5, 1, 0, 0, False, 1),    # six reduction steps
     (32, 64, 2, 9, 9, 1, 0, 3, True, 2),      # 81 pixels: the layer and the pooling one after the other
     (16, 32, 2, 6, 6, 3, 1, 1, True, 2),      # a 3x3 layer
 ]

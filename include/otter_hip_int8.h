@@ -254,8 +254,8 @@ int otter_hip_conv_block_forward(const otter_hip_conv_t* expand, const otter_hip
 int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_channels, int n, int in_h, int in_w,
                               int rows_per_band, int slice_channels, int split, int plan[6]);
 /* Tuning / test hook with no counterpart in the reference: 1 = every block that qualifies by shape runs as the single
- * launch, 0 = only the shapes measured faster that way (default). Process-wide; returns the previous value; a negative
- * argument only queries. */
+ * launch, 0 = only the shapes measured faster that way (default), 2 = none does. Process-wide; returns the previous
+ * value; a negative argument only queries. */
 int otter_hip_conv_block_set_always(int on);
 /* Tuning / test hook with no counterpart in the reference: how a block that does not run as the single launch runs its
  * first two layers: 0 = as one launch where that was measured faster (a stride-2 depthwise layer, or an expanded blob

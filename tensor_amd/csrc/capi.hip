@@ -831,13 +831,14 @@ static int g_block_always = 0;  // see block_single_launch
 
 static bool block_single_launch(const otter_hip_conv_t* e, const otter_hip_conv_t* d, const otter_hip_conv_t* p,
                                 const ConvGeom g[3], int out_layout, int plan[6]) {
+    if (g_block_always == 2) return false;  // (tuning hook: never)
     if (!e->w_igemm || e->c_pad || e->force_tm || !e->blk_consts || !d->depthwise || !d->blk_consts || d->c_pad || d->force_tm || !p->w_igemm ||
         p->c_pad || p->force_tm)
         return false;
     const Epilogue e1 = make_epilogue(e, OTTER_HIP_I8_P8), e2 = make_epilogue(d, OTTER_HIP_I8_P8), e3 = make_epilogue(p, out_layout);
     if (!conv_block_applicable(g[0], e1, g[1], e2, g[2], e3)) return false;
     if (!conv_block_plan(g[0], g[2], e->block_rb, e->block_sl, e->block_split, plan)) return false;
-    if (g_block_always || e->block_rb || e->block_sl || e->block_split) return true;
+    if (g_block_always == 1 || e->block_rb || e->block_sl || e->block_split) return true;
     // The single launch pays where the three layers are short, latency-bound launches and its workgroups (a band of
     // rows of one image each, or a share of a band's expanded channels) about fill the 256 compute units once.
     // Measured at batch 64 against the three launches (kernel trace; in brackets the three launches inside a network,
@@ -916,7 +917,7 @@ int otter_hip_conv_block_plan(int in_channels, int expanded_channels, int out_ch
 
 int otter_hip_conv_block_set_always(int on) {
     const int before = g_block_always;
-    if (on >= 0) g_block_always = on ? 1 : 0;
+    if (on >= 0) g_block_always = on > 2 ? 1 : on;
     return before;
 }
 

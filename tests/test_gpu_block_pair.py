@@ -103,3 +103,46 @@ def test_pair_launch_with_the_exact_rounding_mode(hip):
     assert hip.torch.equal(got, want)
     for l in layers:
         l["conv"].close()
+
+
+def test_pair_launch_random_shapes(hip):
+    """Seeded random blocks (channel counts, image sizes, strides, padding, activations, result kinds, strip heights):
+    wherever the launch of the first two layers takes the shape it equals the three layers one by one, bit for bit."""
+    rng = np.random.default_rng(77)
+    always = hip.conv_block_set_always(2)  # (never the single launch: every block here goes to the pair or to three)
+    pair = hip.conv_block_set_pair(1)
+    taken = 0
+    try:
+        for case in range(48):
+            cin = 8 * int(rng.integers(1, 17))
+            ce = 16 * int(rng.integers(1, 13))
+            cout = 8 * int(rng.integers(1, 9))
+            stride = int(rng.choice([1, 2]))
+            dw_pad = int(rng.choice([0, 1, 1]))
+            N, H = int(rng.integers(1, 4)), int(rng.integers(3, 40))
+            W = int(rng.integers(3, 129 if cin <= 32 else 65))
+            act = int(rng.choice([0, 1, 3]))
+            f32_out = bool(rng.integers(0, 2))
+            layers = make_block(hip, rng, cin, ce, cout, act, f32_out, stride=stride, dw_pad=dw_pad)
+            e, d, p = (l["conv"] for l in layers)
+            strip = int(rng.choice([0, 0, 1, 2, 3, 5, 9]))
+            if strip:
+                e.set_block_plan(strip, 0, 0)
+                hip.conv_block_set_always(2)
+            launches = hip.conv_block_launches(e, d, p, N, H, W)
+            x = rng.integers(-127, 128, (N, cin, H, W)).astype(np.int8)
+            xd = hip.to_device(capi.pack_np(x, 8))
+            q_scale = 17.0 if f32_out and rng.integers(0, 2) else None
+            got, got_q = hip.conv_block(e, d, p, xd, N, H, W, q_scale=q_scale)
+            want, want_q = one_by_one(hip, layers, xd, N, H, W, None, q_scale)
+            hip.torch.cuda.synchronize()
+            assert hip.torch.equal(got, want), (case, cin, ce, cout, stride, dw_pad, N, H, W, act, strip, launches)
+            if q_scale is not None:
+                assert hip.torch.equal(got_q, want_q), case
+            taken += launches == 2
+            for l in layers:
+                l["conv"].close()
+    finally:
+        hip.conv_block_set_always(always)
+        hip.conv_block_set_pair(pair)
+    assert taken >= 30

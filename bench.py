@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 convolution path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c2|c2i8|c0|c0n64|c4|det|dil2|grp8|s2|odd55] [--no-cpu] [--no-also]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1s1|c1s2|c1s1i8|c1s2i8|c1s1valu|c1s2valu|c2|c2i8|c0|c0n64|c4|det|blk14|blk112s2|dil2|grp8|s2|odd55|w224|copy]
+                    [--no-cpu] [--no-also]
 
 Prints ONE JSON line. The headline workload is the fourth benchmark configuration (the MFMA-bound case the metric's
 "int8 conv TOPS (% MFMA peak)" is quoted on): four chained int8-in/int8-out 3x3 convolutions 128->128 at
 56x56, batch 64, fused requantize+ReLU. One step = the four layers back to back on device-resident int8
 activations. The other single-GPU configurations (depthwise c1 at stride 1 and 2 with its HBM roofline, the
-1x1 GEMM c2 and its int8-output variant, the single-image c0 and the same layer at batch 64) are measured the same
-way and reported under "also", followed by a plain device-to-device copy of 256 MiB ("copy": what a copy reaches on
+1x1 GEMM c2 and its int8-output variant, the single-image c0 and the same layer at batch 64, the MobileNetV2-style
+network c4, the reference's detection model file, two inverted-residual blocks and five single layers outside the tuned
+shapes) are measured the same way and reported under "also", followed by a plain device-to-device copy of 256 MiB ("copy": what a copy reaches on
 the box the line was measured on). A bandwidth-bound kernel's roofline figure comes from a loop that rotates over enough
 buffer sets to exceed the 256 MB last-level cache; the figure of the loop over one (cache-resident) set is reported
 beside it as "roofline_resident".

@@ -446,11 +446,26 @@ static int pick_kernel(const otter_hip_conv* h, int int8_layout, const ConvGeom&
     return 0;
 }
 
+// A pointwise layer on an fp32 Float8 blob whose quantize_to_int8 runs in the loader of the implicit-GEMM kernel (one
+// launch, no int8 copy of the blob). Layers the streamed 1x1 kernel would take from an int8 blob go this way too from 64
+// input channels on or up to 65536 pixels. Measured, quantize + streamed kernel against this launch, us with cold
+// operands: 256 -> 512 @28x28 b32 20.9 / 20.0, 256 -> 64 @56x56 b16 19.8 / 15.2, 64 -> 384 @28x28 b64 16.4 / 15.7,
+// 32 -> 192 @28x28 b64 11.2 / 10.2, 40 -> 240 @28x28 b32 11.0 / 8.3, but 32 -> 192 @56x56 b64 23.0 / 32.9 and
+// 16 -> 96 @112x112 b64 35.3 / 72.0 (a 64-deep reduction step is mostly padding there, and the pixels are many).
+// set_tile(-6, 0) keeps the two launches; set_tile(-4, 0) takes this launch for every layer it can run.
+static bool use_igemm_f32in(const otter_hip_conv* h, int in_layout, const ConvGeom& g, const Epilogue& ep) {
+    if (in_layout != OTTER_HIP_F32_P8 || !h->w_igemm || h->c_pad || (h->force_tm != 0 && h->force_tm != -4)) return false;
+    if (g.OH < 1 || g.OW < 1 || !igemm_f32in_applicable(g, ep)) return false;
+    const int kind = pick_kernel(h, OTTER_HIP_I8_P8, g, ep);
+    return kind == 1 || (kind == 5 && (g.C >= 64 || (long)g.N * g.H * g.W <= 65536));
+}
+
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int out_layout) {
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
     ConvGeom g = make_geom(h->d, n, in_h, in_w);
     if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) return 4;
+    if (use_igemm_f32in(h, in_layout, g, make_epilogue(h, out_layout))) return 1;
     if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
     if (h->c_pad) l = OTTER_HIP_I8_P8, g.C = h->c_pad;
     return pick_kernel(h, l, g, make_epilogue(h, out_layout));
@@ -524,6 +539,21 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
         OHIP_CHECK(run_conv_dw_f32in((const float*)in, h->w_dw_mfma, out, g, ep, dw_mfma_epilogue(ep, g.K), h->in_scale,
                                      d.in_round_mode, h->force_tm == -2 ? h->force_tn : 0, stream));
         return quantize_twin();
+    }
+
+    // A pointwise layer on an fp32 Float8 blob: the implicit-GEMM kernel's loader quantizes.
+    {
+        Epilogue ep = make_epilogue(h, out_layout);
+        if (use_igemm_f32in(h, in_layout, g, ep)) {
+            if ((twin || residual) && (!twin || g.K % 8 == 0) && pick_epilogue(ep, g.K) == EPI_F32_P4) {
+                ep.twin = twin, ep.twin_scale = twin_scale;
+                ep.twin_half = twin_round == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+                ep.residual = residual;
+                twin = nullptr, residual = nullptr;  // done by the convolution itself
+            }
+            OHIP_CHECK(run_conv_igemm_f32in((const float*)in, h->w_igemm, out, g, ep, h->in_scale, d.in_round_mode, stream));
+            return quantize_twin();
+        }
     }
 
     // (1) quantize_to_int8 when the blob is not int8 yet (Tensor/ConvolutionLayer.cpp:770-775)

@@ -39,10 +39,14 @@ struct IgemmCfg {
 // global-memory latency per chunk: right for long reductions, where several workgroups per CU cover it). KC > 1: a
 // stage of KC chunks in a single LDS buffer, the whole next stage in registers meanwhile; a reduction of at most KC
 // chunks (pointwise layers) then pays the latency once per workgroup instead of once per chunk.
-template <int TM, int TN, int WM, int WN, int EPI, int KC>
+// INF: the input is the fp32 Float8 blob of a pointwise layer ([N][C/8][H*W][8 floats]); the loader reads the 32 bytes
+// of a pixel's octet and quantizes them with the layer's input scale and rounding primitive on the way into LDS
+// (quantize_to_int8, Tensor/ConvolutionLayer.cpp:770-775, without its own pass over the blob).
+template <int TM, int TN, int WM, int WN, int EPI, int KC, bool INF = false>
 __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ wpk,
                                                          void* __restrict__ out, ConvGeom g, Epilogue ep, int m_tiles16,
-                                                         int c_groups, int n_pix_tiles) {
+                                                         int c_groups, int n_pix_tiles, const float* __restrict__ in_scale_p,
+                                                         float in_half) {
     using Cfg = IgemmCfg<TM, TN, WM, WN>;
     constexpr int FM = Cfg::FM, FN = Cfg::FN;
     constexpr int NBUF = KC == 1 ? 2 : KC;
@@ -123,9 +127,14 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
     }
     constexpr unsigned IG_OOB = 0x80000000u;
     const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<int8_t*>(x), 0, (int)((unsigned)g.N * (unsigned)Cs8 * (unsigned)HW * 8u - (unsigned)blockIdx.z * (unsigned)(g.C / 8) * (unsigned)HW * 8u), 0x00020000);
+        const_cast<int8_t*>(x), 0,
+        (int)(((unsigned)g.N * (unsigned)Cs8 * (unsigned)HW * 8u - (unsigned)blockIdx.z * (unsigned)(g.C / 8) * (unsigned)HW * 8u) * (INF ? 4u : 1u)),
+        0x00020000);
 
-    v2i breg[KC][Cfg::B_V][2];
+    v2i breg[INF ? 1 : KC][INF ? 1 : Cfg::B_V][2];
+    v4i bregf[INF ? KC : 1][INF ? Cfg::B_V : 1][4];  // INF: two octets x 8 floats of a pixel
+    float in_scale = 0.f;
+    if constexpr (INF) in_scale = in_scale_p[0];
     v4i areg[KC][Cfg::A_V];
     // Few input channels (a group of a grouped convolution with at most 32): tap_pack kernel taps share a reduction
     // step, the 16-channel quarter j of the step being channels 16 (j % per) .. of tap tap_pack * kc + j / per with
@@ -162,9 +171,18 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
         for (int r = 0; r < Cfg::B_V; ++r) {
             const int o0 = cgp * 8 + 2 * (j0 + r * J_STEP);
             const unsigned v_lo = (unsigned)(px_ofs + tap_ofs + o0 * HW * 8);
-            breg[q][r][0] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(inb && o0 < C8 ? v_lo : IG_OOB), 0, 0));
-            breg[q][r][1] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(
-                rin, (int)(inb && o0 + 1 < C8 ? v_lo + (unsigned)(HW * 8) : IG_OOB), 0, 0));
+            if constexpr (INF) {
+                // (the fp32 element of a pixel's octet lies at four times the int8 element's offset)
+                const unsigned f0 = inb && o0 < C8 ? v_lo * 4u : IG_OOB, f1 = inb && o0 + 1 < C8 ? (v_lo + (unsigned)(HW * 8)) * 4u : IG_OOB;
+                bregf[q][r][0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)f0, 0, 0));
+                bregf[q][r][1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)f0, 16, 0));
+                bregf[q][r][2] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)f1, 0, 0));
+                bregf[q][r][3] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, (int)f1, 16, 0));
+            } else {
+                breg[q][r][0] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rin, (int)(inb && o0 < C8 ? v_lo : IG_OOB), 0, 0));
+                breg[q][r][1] = __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(
+                    rin, (int)(inb && o0 + 1 < C8 ? v_lo + (unsigned)(HW * 8) : IG_OOB), 0, 0));
+            }
         }
         }
         const int8_t* wa = wpk + ((size_t)kc * m_tiles16 + mt0) * 1024;
@@ -174,11 +192,28 @@ __global__ void __launch_bounds__(256) conv_igemm_kernel(const int8_t* __restric
             if (vi * 16 < Cfg::A_BYTES) areg[q][r] = *reinterpret_cast<const v4i*>(wa + (size_t)vi * 16);
         }
     };
+    // float2int8 of four values into four bytes (the arithmetic of otter_hip_quantize)
+    auto quant4 = [&](const v4i& f) -> int {
+        int k[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float t = __fmul_rn(__int_as_float(f[e]), in_scale);
+            k[e] = (int)__fadd_rn(t, __builtin_copysignf(in_half, t));  // toward zero, saturating
+        }
+        const ohip_v2s top = {127, 127}, bot = {-127, -127};
+        ohip_v2s a = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[0], k[1]));
+        ohip_v2s b = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[2], k[3]));
+        a = __builtin_elementwise_max(__builtin_elementwise_min(a, top), bot);
+        b = __builtin_elementwise_max(__builtin_elementwise_min(b, top), bot);
+        return (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, a), 0x06040200u);
+    };
     auto store_lds = [&](int buf, int q) {
 #pragma unroll
         for (int r = 0; r < Cfg::B_V; ++r) {
             const int j = j0 + r * J_STEP;
-            v4i t = {breg[q][r][0][0], breg[q][r][0][1], breg[q][r][1][0], breg[q][r][1][1]};
+            v4i t;
+            if constexpr (INF) t = v4i{quant4(bregf[q][r][0]), quant4(bregf[q][r][1]), quant4(bregf[q][r][2]), quant4(bregf[q][r][3])};
+            else t = v4i{breg[q][r][0][0], breg[q][r][0][1], breg[q][r][1][0], breg[q][r][1][1]};
             *reinterpret_cast<v4i*>(&lds_b[buf][(j * TN + p_l) * 16]) = t;
         }
 #pragma unroll
@@ -449,7 +484,31 @@ static hipError_t launch_igemm_k(const int8_t* x, const int8_t* wpk, void* out, 
     const int m_tiles = (g.K + TM - 1) / TM;  // row blocks that hold at least one real channel (the rows are padded further)
     const int grid_z = g.Cs ? g.Cs / g.C : 1;  // groups of a grouped convolution
     hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, EPI, KC>), dim3(n_pix_tiles, m_tiles, grid_z), dim3(256), 0,
-                       stream, x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles);
+                       stream, x, wpk, out, g, ep, mpad / 16, igemm_channel_groups(g.C), n_pix_tiles, (const float*)nullptr, 0.f);
+    return hipGetLastError();
+}
+
+// the same launch on the fp32 Float8 blob of a pointwise layer (one k-chunk per stage)
+template <int TM, int TN, int WM, int WN>
+static hipError_t launch_igemm_f32in(const float* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                                     const float* in_scale, float in_half, hipStream_t stream) {
+    const long total_pix = (long)g.N * g.OH * g.OW;
+    const int n_pix_tiles = (int)((total_pix + TN - 1) / TN);
+    const int mpad = igemm_padded_rows(g.K);
+    const dim3 grid(n_pix_tiles, (g.K + TM - 1) / TM, 1);
+#define OHIP_IGF(E_)                                                                                                        \
+    hipLaunchKernelGGL((conv_igemm_kernel<TM, TN, WM, WN, E_, 1, true>), grid, dim3(256), 0, stream, (const int8_t*)x, wpk, out, g, ep, \
+                       mpad / 16, igemm_channel_groups(g.C), n_pix_tiles, in_scale, in_half)
+    switch (pick_epilogue(ep, g.K)) {
+    case EPI_I8_P8: OHIP_IGF(EPI_I8_P8); break;
+    case EPI_I8_P8_NONNEG: OHIP_IGF(EPI_I8_P8_NONNEG); break;
+    case EPI_F32_P4:
+        if (ep.twin != nullptr || ep.residual != nullptr) OHIP_IGF(EPI_F32_P4_FUSED);
+        else OHIP_IGF(EPI_F32_P4);
+        break;
+    default: return hipErrorInvalidValue;
+    }
+#undef OHIP_IGF
     return hipGetLastError();
 }
 
@@ -573,6 +632,35 @@ hipError_t run_conv_igemm(const int8_t* x, const int8_t* wpk, void* out, const C
     OHIP_IG(32, 128, 1, 4)
     OHIP_IG(32, 64, 1, 4)
 #undef OHIP_IG
+    return hipErrorInvalidValue;
+}
+
+// true when run_conv_igemm_f32in takes this layer: a pointwise layer (1x1, stride 1, no padding, one group) on a Float8
+// blob with one of the packed epilogues
+bool igemm_f32in_applicable(const ConvGeom& g, const Epilogue& ep) {
+    if (g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph || g.pw || g.groups != 1 || g.C % 8) return false;
+    const int epi = pick_epilogue(ep, g.K);
+    if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4) return false;
+    return (size_t)g.N * g.C * g.H * g.W * 4 < ((size_t)1 << 31);  // 32-bit byte offsets into the fp32 blob
+}
+
+hipError_t run_conv_igemm_f32in(const float* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                                const float* in_scale, int in_round_mode, hipStream_t stream) {
+    if (!igemm_f32in_applicable(g, ep)) return hipErrorInvalidValue;
+    int tm, tn;
+    igemm_choose_tiles(g, &tm, &tn);
+    if (igemm_padded_rows(g.K) % tm != 0) return hipErrorInvalidValue;
+    const float half = in_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+#define OHIP_IGF(TM_, TN_, WM_, WN_) \
+    if (tm == TM_ && tn == TN_) return launch_igemm_f32in<TM_, TN_, WM_, WN_>(x, wpk, out, g, ep, in_scale, half, stream);
+    OHIP_IGF(128, 64, 4, 1)
+    OHIP_IGF(64, 256, 2, 2)
+    OHIP_IGF(64, 128, 2, 2)
+    OHIP_IGF(64, 64, 2, 2)
+    OHIP_IGF(32, 256, 1, 4)
+    OHIP_IGF(32, 128, 1, 4)
+    OHIP_IGF(32, 64, 1, 4)
+#undef OHIP_IGF
     return hipErrorInvalidValue;
 }
 

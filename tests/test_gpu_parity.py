@@ -678,6 +678,79 @@ def test_depthwise3x3_from_an_fp32_blob_in_one_launch(hip, oracle, s):
     assert (outs[capi.ROUND_SSE] != outs[capi.ROUND_EXACT]).any()
 
 
+@pytest.mark.parametrize("C,K,N,H,W,int8_out,tile_shape,small", [
+    (72, 512, 2, 9, 11, True, "128x64", True),
+    (72, 512, 1, 7, 7, False, "128x64", True),
+    (136, 64, 1, 30, 30, True, "64x64", True),
+    (72, 64, 8, 128, 128, True, "64x128", False),
+    (8, 64, 8, 256, 256, False, "64x256", False),
+    (80, 24, 2, 9, 11, True, "32x64", True),
+    (80, 32, 2, 128, 128, True, "32x128", False),
+    (8, 16, 8, 256, 256, False, "32x256", False),
+    (200, 100, 3, 5, 13, False, "64x64", True),    # channel octets that end inside a 64-deep step, K % 8 != 0
+])
+def test_pointwise_from_an_fp32_blob_in_one_launch(hip, oracle, C, K, N, H, W, int8_out, tile_shape, small):
+    """A pointwise layer of the implicit-GEMM kernel on an fp32 Float8 blob quantizes in the kernel's loader (one launch,
+    no int8 copy of the blob). Bit for bit against the two launches (set_tile(-6, 0)) at every tile shape the launcher
+    picks -- values on rounding ties, on the float the two primitives round differently and beyond saturation, every
+    packed epilogue -- and, at the sizes the oracle finishes in seconds, against the oracle's layer."""
+    rng = np.random.default_rng(C * 7 + K)
+    x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+    in_scale = np.float32(100.0)
+    flat = x.reshape(-1)
+    flat[::7] = (rng.integers(-140, 141, flat[::7].size) + 0.5) / in_scale
+    flat[3::11] = np.nextafter(np.float32(0.5), np.float32(0)) / in_scale * rng.choice([-1, 1], flat[3::11].size)
+    for act in ((3, 0, 2) if int8_out else (1, 2)):
+        args = dict(bias=bias, top_scale=9.0, act=act, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, **args)
+        two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **args)
+        assert kind == 1
+        assert out.tobytes() == two.tobytes(), (act, tile_shape)
+        if small:
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, bias=bias, top_scale=9.0, int8_out=int8_out, act_type=act,
+                                             act_params=[0.1] if act == 2 else None)
+            if int8_out:
+                np.testing.assert_array_equal(out, want)
+            else:
+                assert_f32_close(out, want)
+
+
+@pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT], ids=["sse", "exact"])
+def test_pointwise_from_an_fp32_blob_twin_and_shortcut(hip, oracle, mode):
+    """The same launch with the shortcut sum and the quantized twin in its epilogue, and with either rounding primitive on
+    the input side: against the oracle's quantize -> convolution -> dequantize -> add -> quantize."""
+    rng = np.random.default_rng(77 + mode)
+    C, K, N, H, W = 96, 24, 3, 14, 13
+    x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+    x.reshape(-1)[::5] = np.nextafter(np.float32(0.5), np.float32(0)) / np.float32(128.0)
+    si = (np.float32(1.0) / (np.float32(128.0) * ws)).astype(np.float32)
+    conv = hip.conv(wq=wq, scale_in=si, bias=bias, in_scale=128.0, out_scale=None, stride=(1, 1), pad=(0, 0), groups=1,
+                    act=0, out_kind=capi.OUT_F32, in_round=mode)
+    xq = oracle.quantize(x, [np.float32(128.0)], mode)
+    plain_want = oracle.dequantize(oracle.conv_int32(xq, wq, (1, 1), (0, 0), (1, 1), 1), si, bias)
+    xd = hip.to_device(capi.pack_np(x, 8))
+    assert conv.kernel_kind(capi.F32_P8, N, H, W, capi.F32_P4) == 1
+    plain = capi.unpack_np(conv.forward(xd, capi.F32_P8, N, H, W, capi.F32_P4).cpu().numpy(), 4, (N, K, H, W))
+    assert_f32_close(plain, plain_want)
+    short = (rng.normal(0, 1, plain.shape) * np.abs(plain).mean()).astype(np.float32)
+    want = plain + short
+    q_scale = 127.0 / float(np.abs(want).max()) * 1.3
+    out, q = conv.forward_residual(xd, capi.F32_P8, N, H, W, hip.to_device(capi.pack_np(short, 4)), q_scale, capi.ROUND_SSE,
+                                   capi.F32_P4)
+    hip.torch.cuda.synchronize()
+    got = capi.unpack_np(out.cpu().numpy(), 4, (N, K, H, W))
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_array_equal(capi.unpack_np(q.cpu().numpy(), 8, (N, K, H, W)),
+                                  oracle.quantize(want, np.float32(q_scale), capi.ROUND_SSE))
+    out2, q2 = conv.forward_twin(xd, capi.F32_P8, N, H, W, q_scale, capi.ROUND_EXACT, capi.F32_P4)
+    hip.torch.cuda.synchronize()
+    got2 = capi.unpack_np(out2.cpu().numpy(), 4, (N, K, H, W))
+    np.testing.assert_array_equal(got2.view(np.uint32), plain.view(np.uint32))
+    np.testing.assert_array_equal(capi.unpack_np(q2.cpu().numpy(), 8, (N, K, H, W)),
+                                  oracle.quantize(plain, np.float32(q_scale), capi.ROUND_EXACT))
+    conv.close()
+
+
 def test_fp32_input_is_quantized_like_the_reference(hip, oracle):
     rng = np.random.default_rng(11)
     for C in (3, 4, 8, 32):

@@ -269,7 +269,10 @@ int otter_hip_conv_block_set_plan(otter_hip_conv_t* expand, int rows_per_band, i
 
 /* Which kernel family forward() would launch for this input: 0 direct (scalar fallback), 1 MFMA implicit
  * GEMM, 2 depthwise, 3 MFMA 3x3 halo kernel, 4 few-channel 3x3 kernel (an image stem read straight from the unpacked
- * blob), 5 streamed 1x1 kernel (int8 -> int8 over at most 64 input channels). For tests and profiling. */
+ * blob), 5 streamed 1x1 kernel (int8 -> int8 over at most 64 input channels), 6 pointwise layer on an fp32 Float8 blob
+ * of 64..256 channels, quantize and convolution in one launch that reads the blob once. (Other pointwise and depthwise 3x3
+ * layers on an fp32 Float8 blob also quantize inside the convolution's launch; they report 1 and 2.) For tests and
+ * profiling. */
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, int n, int in_h, int in_w,
                                int out_layout);
 
@@ -283,7 +286,10 @@ int otter_hip_conv_kernel_kind(const otter_hip_conv_t* handle, int in_layout, in
  * strip height of (8 >> tn) output rows for stride 1 and (4 >> tn) for stride 2, tn in 0..2. tm == -4: the generic
  * implicit-GEMM kernel with its automatic tile choice, where the LDS-halo or the streamed 1x1 kernel would be picked.
  * tm == -5 on a layer the streamed 1x1 kernel takes: tn = groups | slices << 3 forces the 16-pixel groups a wave owns
- * (2 or 4) and the slices the output channels are cut into (0 = automatic for either). */
+ * (2 or 4) and the slices the output channels are cut into (0 = automatic for either). tm == -6: quantize an fp32 blob
+ * in a launch of its own (the two launches of the reference's order) where the convolution's launch would do it.
+ * tm == -7 on a pointwise layer: kernel 6 above wherever it can run, tn = groups | pairs << 3 forcing the 16-pixel
+ * groups a wave owns (1 or 2) and the pairs of 16 output channels per LDS round (0 = automatic for either). */
 int otter_hip_conv_set_tile(otter_hip_conv_t* handle, int tm, int tn);
 
 /* Test hook with no counterpart in the reference, host arithmetic only (no GPU needed): the launch plan of the 3x3

@@ -423,7 +423,7 @@ static bool use_stem(const otter_hip_conv* h, int in_layout, const ConvGeom& g_i
 }
 
 // 0 direct, 1 MFMA implicit GEMM, 2 depthwise, 3 MFMA 3x3 with the halo in LDS, 4 few-channel 3x3 (image stem),
-// 5 streamed 1x1 over few input channels
+// 5 streamed 1x1 over few input channels, 6 pointwise layer straight from an fp32 blob (the blob read once)
 // a depthwise 3x3 layer that reads an fp32 Float8 blob and can run quantize + convolution as one launch
 static bool use_dw_f32in(const otter_hip_conv* h, int in_layout, const ConvGeom& g, int out_layout) {
     if (in_layout != OTTER_HIP_F32_P8 || !h->w_dw_mfma || h->c_pad || h->force_tm == -3 || h->force_tm == -6) return false;
@@ -460,11 +460,26 @@ static bool use_igemm_f32in(const otter_hip_conv* h, int in_layout, const ConvGe
     return kind == 1 || (kind == 5 && (g.C >= 64 || (long)g.N * g.H * g.W <= 65536));
 }
 
+// The same layers with 64 .. 256 input channels and 128 output channels or more on the kernel that reads the fp32 blob
+// once and walks all output channels per pixel group (conv_pw_f32in_kernel). Measured against the launch above, us with
+// cold operands / the same buffers every time: 256 -> 512 @28x28 b32 fp32 out 21.7 / 17.0 against 24.6 / 20.0, int8 out
+// 18.4 / 15.1 against 20.8 / 16.5; 64 -> 384 @28x28 b64 14.2 / 11.3 against 17.1 / 13.7; 128 -> 128 @28x28 b64 11.5 / 8.9
+// against 12.8 / 9.1; with fewer output channels (256 -> 64 @56x56 b16, 96 -> 24 @56x56 b64) the two are level, and below
+// 64 input channels the copy of the weights per workgroup costs more than the pixels it serves (16 -> 96 @112x112 b64:
+// 50.7 against 38.4). set_tile(-7, groups | pairs << 3) takes this kernel for every layer it can run.
+static bool use_pw_f32in(const otter_hip_conv* h, int in_layout, const ConvGeom& g, const Epilogue& ep) {
+    if (in_layout != OTTER_HIP_F32_P8 || !h->w_igemm || h->c_pad || (h->force_tm != 0 && h->force_tm != -7)) return false;
+    if (g.OH < 1 || g.OW < 1 || !conv_pw_f32in_applicable(g, ep)) return false;
+    if (pick_epilogue(ep, g.K) == EPI_I8_P8_NONNEG && !h->clamp_hi) return false;
+    return h->force_tm == -7 || (g.C >= 64 && g.K >= 128);
+}
+
 int otter_hip_conv_kernel_kind(const otter_hip_conv_t* h, int in_layout, int n, int in_h, int in_w, int out_layout) {
     if (!h || !valid_layout(in_layout)) return fail(OTTER_HIP_ERR_INVALID, "otter_hip_conv_kernel_kind: bad argument");
     int l = in_layout;
     ConvGeom g = make_geom(h->d, n, in_h, in_w);
     if (use_stem(h, in_layout, g, make_epilogue(h, out_layout))) return 4;
+    if (use_pw_f32in(h, in_layout, g, make_epilogue(h, out_layout))) return 6;
     if (use_igemm_f32in(h, in_layout, g, make_epilogue(h, out_layout))) return 1;
     if (layout_elem(l) == 0) l = h->d.in_channels % 8 == 0 ? OTTER_HIP_I8_P8 : OTTER_HIP_I8;
     if (h->c_pad) l = OTTER_HIP_I8_P8, g.C = h->c_pad;
@@ -541,9 +556,14 @@ static int conv_forward(const otter_hip_conv_t* h, const void* in, int in_layout
         return quantize_twin();
     }
 
-    // A pointwise layer on an fp32 Float8 blob: the implicit-GEMM kernel's loader quantizes.
+    // A pointwise layer on an fp32 Float8 blob: quantize_to_int8 inside the convolution's launch.
     {
         Epilogue ep = make_epilogue(h, out_layout);
+        if (!twin && !residual && use_pw_f32in(h, in_layout, g, ep)) {
+            OHIP_CHECK(run_conv_pw_f32in((const float*)in, h->w_igemm, h->clamp_hi, out, g, ep, h->in_scale, d.in_round_mode,
+                                         h->force_tm == -7 ? (h->force_tn & 7) : 0, h->force_tm == -7 ? (h->force_tn >> 3) : 0, stream));
+            return OTTER_HIP_OK;
+        }
         if (use_igemm_f32in(h, in_layout, g, ep)) {
             if ((twin || residual) && (!twin || g.K % 8 == 0) && pick_epilogue(ep, g.K) == EPI_F32_P4) {
                 ep.twin = twin, ep.twin_scale = twin_scale;

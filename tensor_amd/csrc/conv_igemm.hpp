@@ -66,6 +66,10 @@ void dw_mfma_pack_weights(const int8_t* w, int C, int stride, int pad_w, int ks,
 int dw_mfma_epilogue(const Epilogue& ep, int K);
 bool dw_mfma_applicable(const ConvGeom& g, const Epilogue& ep, int epi, bool scale_out_positive);
 // the same layer straight from an fp32 Float8 blob (quantize + depthwise convolution in one launch)
+// a pointwise layer of at most 256 input channels straight from an fp32 Float8 blob, the blob read once (conv_pw.hip)
+bool conv_pw_f32in_applicable(const ConvGeom& g, const Epilogue& ep);
+hipError_t run_conv_pw_f32in(const float* x, const int8_t* wpk, const unsigned* qh, void* out, const ConvGeom& g, const Epilogue& ep,
+                             const float* in_scale, int in_round_mode, int force_groups, int force_pairs, hipStream_t stream);
 // a pointwise layer straight from an fp32 Float8 blob: quantize_to_int8 in the loader of the implicit-GEMM kernel
 bool igemm_f32in_applicable(const ConvGeom& g, const Epilogue& ep);
 hipError_t run_conv_igemm_f32in(const float* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,

@@ -25,6 +25,7 @@ namespace ohip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef unsigned v2u_store __attribute__((__vector_size__(2 * sizeof(unsigned))));
+typedef unsigned v4u_store __attribute__((__vector_size__(4 * sizeof(unsigned))));
 
 constexpr unsigned PW_OOB = 0x80000000u;  // past any buffer: the load returns zero, the store is dropped
 
@@ -218,6 +219,272 @@ hipError_t run_conv_pw_stream(const int8_t* x, const int8_t* wpk, const unsigned
     OHIP_PW(2, 1)
     OHIP_PW(2, 4)
 #undef OHIP_PW
+    return hipErrorInvalidValue;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The pointwise layer on an fp32 Float8 blob (quantize_to_int8 of Tensor/ConvolutionLayer.cpp:770-775 and the convolution
+// as one launch), int8 or fp32 result, up to 256 input channels.
+//
+// The blob is four times the bytes of its int8 copy, so it is read ONCE: a wave owns G groups of 16 pixels of one image,
+// requests all their channels at the start of the kernel (4 x 16 bytes per lane, group and reduction step: the bytes in
+// flight per wave are what keeps HBM busy on a layer of a few thousand waves), quantizes them into the B operands it
+// keeps for the whole kernel, and walks ALL output channels in pairs of 16-row tiles. The pairs' weights and constants
+// go through LDS in rounds of `pairs_per_round` (the image of conv_pw_stream_kernel; a barrier on either side of a
+// round's copy), so a round's LDS stays small enough for several workgroups per compute unit.
+// fp32 result (EPI_F32_P4): after the MFMAs of a pair a lane holds two Float4 elements of its pixel (igemm_row_channel).
+constexpr int PW_F32IN_COPIES = 9;  // 16-byte loads per thread and round of the weight image
+
+template <int EPI, int G, int CG>
+__global__ void __launch_bounds__(256) conv_pw_f32in_kernel(const float* __restrict__ x, const int8_t* __restrict__ wpk,
+                                                            void* __restrict__ out, Epilogue ep,
+                                                            const unsigned* __restrict__ qh, int C8, int K, int HW,
+                                                            int pairs_per_round, int mt, const float* __restrict__ in_scale_p,
+                                                            float in_half) {
+    constexpr int PW_PAIR_V4 = pw_pair_v4(CG);
+    constexpr bool F32 = EPI == EPI_F32_P4;
+    constexpr int W4 = 128 * CG;
+    extern __shared__ v4i pw_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q = lane >> 4, p = lane & 15;
+    const int n = blockIdx.y;
+    const int pix0 = (blockIdx.x * 4 + wave) * (16 * G);
+    const bool active = pix0 < HW;  // (a wave past the image still copies and meets the barriers)
+
+    const size_t in_img = (size_t)C8 * HW * 32, out_img = (size_t)K * HW * (F32 ? 4 : 1);
+    const __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(reinterpret_cast<const char*>(x)) + (size_t)n * in_img, 0, (int)in_img, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rout =
+        __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(out) + (size_t)n * out_img, 0, (int)out_img, 0x00020000);
+
+    // every byte the wave will read, requested now (pixels or octets that do not exist: past the buffer, zeros)
+    v4i raw[G][CG][4];
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) {
+        const int pix = pix0 + 16 * gi + p;
+        const bool in = pix < HW;
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) {
+            const int oct = 8 * cg + 2 * q;
+            const unsigned o0 = ((unsigned)oct * HW + pix) * 32u;
+            const int v0 = (int)(in && oct < C8 ? o0 : PW_OOB), v1 = (int)(in && oct + 1 < C8 ? o0 + (unsigned)HW * 32u : PW_OOB);
+            raw[gi][cg][0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, v0, 0, 0));
+            raw[gi][cg][1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, v0 + 16, 0, 0));
+            raw[gi][cg][2] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, v1, 0, 0));
+            raw[gi][cg][3] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rin, v1 + 16, 0, 0));
+        }
+    }
+    const float in_scale = in_scale_p[0];
+    // float2int8 of four values into four bytes (the arithmetic of otter_hip_quantize)
+    auto quant4 = [&](const v4i& f) -> int {
+        int k[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float t = __fmul_rn(__int_as_float(f[e]), in_scale);
+            k[e] = (int)__fadd_rn(t, __builtin_copysignf(in_half, t));  // toward zero, saturating
+        }
+        const ohip_v2s top = {127, 127}, bot = {-127, -127};
+        ohip_v2s a = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[0], k[1]));
+        ohip_v2s b = __builtin_bit_cast(ohip_v2s, __builtin_amdgcn_cvt_pk_i16(k[2], k[3]));
+        a = __builtin_elementwise_max(__builtin_elementwise_min(a, top), bot);
+        b = __builtin_elementwise_max(__builtin_elementwise_min(b, top), bot);
+        return (int)__builtin_amdgcn_perm(__builtin_bit_cast(unsigned, b), __builtin_bit_cast(unsigned, a), 0x06040200u);
+    };
+    v4i b[G][CG];
+
+    const int pairs = (K + 31) / 32;
+    const v4i* wg = reinterpret_cast<const v4i*>(wpk);
+    const v4i* sg = reinterpret_cast<const v4i*>(ep.scale_in);
+    const v4i* bg = reinterpret_cast<const v4i*>(ep.bias);
+    const v4i* og = reinterpret_cast<const v4i*>(ep.scale_out);
+    const v4i* cq = reinterpret_cast<const v4i*>(qh);
+    // A round's image, copied by all threads with PW_F32IN_COPIES loads each: slot k of a thread is element
+    // threadIdx.x + 256 k of the image, i.e. always the same array and the same place in a pair, one round further each
+    // time (a pointer and its step per slot). The loads are unconditional (a slot past the image or past the last pair
+    // reads the first weights again and lands in the slack of the buffer) and are requested before the round in front
+    // is computed; the image goes into the other of two LDS buffers once that is done: one barrier per round.
+    // The per-channel arrays are padded to the weight rows, so every pair is whole in memory.
+    constexpr int BUF_V4 = 256 * PW_F32IN_COPIES;
+    const v4i* src[PW_F32IN_COPIES];
+    int step[PW_F32IN_COPIES], prk[PW_F32IN_COPIES];
+#pragma unroll
+    for (int k = 0; k < PW_F32IN_COPIES; ++k) {
+        const int i = threadIdx.x + 256 * k;
+        const int pr = i / PW_PAIR_V4, r = i % PW_PAIR_V4;
+        src[k] = wg + ((size_t)(r / 128) * mt + 2 * pr) * 64 + r % 128;  // (step, the pair's two tiles, lane)
+        step[k] = 2 * pairs_per_round * 64;
+        if (r >= W4) src[k] = sg + pr * 8 + r - W4, step[k] = pairs_per_round * 8;
+        if (r >= W4 + 8) src[k] = bg + pr * 8 + r - W4 - 8;
+        if (r >= W4 + 16) {
+            if constexpr (F32) src[k] = wg, step[k] = 0;
+            else src[k] = og + pr * 8 + r - W4 - 16;
+        }
+        if (r >= W4 + 24) {
+            if constexpr (EPI == EPI_I8_P8_NONNEG) src[k] = cq + pr * 4 + r - W4 - 24, step[k] = pairs_per_round * 4;
+            else src[k] = wg, step[k] = 0;
+        }
+        prk[k] = pr;
+        if (pr >= pairs_per_round) src[k] = wg, step[k] = 0, prk[k] = 0;
+    }
+    v4i cp[PW_F32IN_COPIES];
+    auto copy_request = [&](int pr0) {
+#pragma unroll
+        for (int k = 0; k < PW_F32IN_COPIES; ++k) {
+            cp[k] = *(pr0 + prk[k] < pairs ? src[k] : wg);
+            src[k] += step[k];
+        }
+    };
+    auto copy_store = [&](int buf) {
+#pragma unroll
+        for (int k = 0; k < PW_F32IN_COPIES; ++k) pw_lds[buf * BUF_V4 + threadIdx.x + 256 * k] = cp[k];
+    };
+    // A pair in two steps: its products (the A operands from LDS, two chains of CG matrix instructions per group) and
+    // its epilogue (constants from LDS, dequantize or requantize, stores). (Issuing the next pair's products in front of
+    // the current epilogue changed nothing measurable: the rounds wait for the stores, not for the matrix pipe.)
+    auto products = [&](const v4i* l, v4i (&c0)[G], v4i (&c1)[G]) {
+        v4i a0[CG], a1[CG];
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg) a0[cg] = l[128 * cg + lane], a1[cg] = l[128 * cg + 64 + lane];
+#pragma unroll
+        for (int gi = 0; gi < G; ++gi) {
+            c0[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b[gi][0], v4i{0, 0, 0, 0}, 0, 0, 0);
+            c1[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b[gi][0], v4i{0, 0, 0, 0}, 0, 0, 0);
+        }
+#pragma unroll
+        for (int cg = 1; cg < CG; ++cg)
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+                c0[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[cg], b[gi][cg], c0[gi], 0, 0, 0);
+                c1[gi] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[cg], b[gi][cg], c1[gi], 0, 0, 0);
+            }
+    };
+    auto epilogue = [&](const v4i* l, int pr, const v4i (&c0)[G], const v4i (&c1)[G]) {
+        const v4i s0 = l[W4 + 2 * q], s1 = l[W4 + 1 + 2 * q], b0 = l[W4 + 8 + 2 * q], b1 = l[W4 + 9 + 2 * q];
+        const int ch0 = 32 * pr + 8 * q;
+        if constexpr (F32) {
+            float si[8], bi[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                si[e] = __int_as_float(s0[e]), si[4 + e] = __int_as_float(s1[e]);
+                bi[e] = __int_as_float(b0[e]), bi[4 + e] = __int_as_float(b1[e]);
+            }
+            const unsigned orow = (unsigned)(ch0 >> 2) * HW;
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+                const int pix = pix0 + 16 * gi + p;
+                const v4i r0 = ep.lrelu ? epi4_dequant_f32p4<true>(ep, si, bi, c0[gi][0], c0[gi][1], c0[gi][2], c0[gi][3])
+                                        : epi4_dequant_f32p4<false>(ep, si, bi, c0[gi][0], c0[gi][1], c0[gi][2], c0[gi][3]);
+                const v4i r1 = ep.lrelu ? epi4_dequant_f32p4<true>(ep, si + 4, bi + 4, c1[gi][0], c1[gi][1], c1[gi][2], c1[gi][3])
+                                        : epi4_dequant_f32p4<false>(ep, si + 4, bi + 4, c1[gi][0], c1[gi][1], c1[gi][2], c1[gi][3]);
+                const unsigned oo = (orow + pix) * 16u;
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, r0), rout,
+                                                       (int)(ch0 < K && pix < HW ? oo : PW_OOB), 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u_store, r1), rout,
+                                                       (int)(ch0 + 4 < K && pix < HW ? oo + (unsigned)HW * 16u : PW_OOB), 0, 0);
+            }
+        } else {
+            Epi8 prm;
+            const v4i o0 = l[W4 + 16 + 2 * q], o1 = l[W4 + 17 + 2 * q], c = l[W4 + 24 + q];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                prm.si[e] = __int_as_float(s0[e]), prm.si[4 + e] = __int_as_float(s1[e]);
+                prm.bi[e] = __int_as_float(b0[e]), prm.bi[4 + e] = __int_as_float(b1[e]);
+                prm.so[e] = __int_as_float(o0[e]), prm.so[4 + e] = __int_as_float(o1[e]);
+                prm.qh[e] = (unsigned)c[e];
+            }
+            const bool live = ch0 < K;
+            const unsigned orow = (unsigned)(ch0 >> 3) * HW;
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) {
+                const int a8[8] = {c0[gi][0], c0[gi][1], c0[gi][2], c0[gi][3], c1[gi][0], c1[gi][1], c1[gi][2], c1[gi][3]};
+                const v2i r = epi8_quant_i8p8<EPI == EPI_I8_P8_NONNEG>(ep, prm, a8);
+                const int pix = pix0 + 16 * gi + p;
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u_store, r), rout,
+                                                      (int)(live && pix < HW ? (orow + pix) * 8u : PW_OOB), 0, 0);
+            }
+        }
+    };
+    auto compute = [&](int pr0, int pr1, int buf) {
+        const v4i* l = pw_lds + buf * BUF_V4;
+        for (int pr = pr0; pr < pr1; ++pr, l += PW_PAIR_V4) {
+            v4i c0[G], c1[G];
+            products(l, c0, c1);
+            epilogue(l, pr, c0, c1);
+        }
+    };
+
+    copy_request(0);
+    __builtin_amdgcn_sched_barrier(0);  // (everything in flight before anything waits for the first)
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+        for (int cg = 0; cg < CG; ++cg)
+            b[gi][cg] = v4i{quant4(raw[gi][cg][0]), quant4(raw[gi][cg][1]), quant4(raw[gi][cg][2]), quant4(raw[gi][cg][3])};
+    copy_store(0);
+    __syncthreads();
+    for (int pr0 = 0, buf = 0; pr0 < pairs; pr0 += pairs_per_round, buf ^= 1) {
+        const bool more = pr0 + pairs_per_round < pairs;
+        if (more) copy_request(pr0 + pairs_per_round);
+        if (active) compute(pr0, min(pr0 + pairs_per_round, pairs), buf);
+        if (more) copy_store(buf ^ 1);  // (last read before the barrier that ended the round in front)
+        __syncthreads();
+    }
+}
+
+// a round is what the 256 threads copy with PW_F32IN_COPIES loads each (36 KB: four workgroups fit a compute unit)
+static int pw_f32in_pairs_per_round(int cgs, int pairs) { return std::max(1, std::min(pairs, 256 * PW_F32IN_COPIES / pw_pair_v4(cgs))); }
+
+bool conv_pw_f32in_applicable(const ConvGeom& g, const Epilogue& ep) {
+    if (g.groups != 1 || g.kh != 1 || g.kw != 1 || g.sh != 1 || g.sw != 1 || g.ph != 0 || g.pw != 0) return false;
+    if (g.Cs || g.Ks || g.C % 8 || g.C > 64 * PW_MAX_CG || g.N < 1 || g.N > 65535) return false;
+    if (ep.twin != nullptr || ep.residual != nullptr) return false;
+    const int epi = pick_epilogue(ep, g.K);
+    if (epi != EPI_I8_P8 && epi != EPI_I8_P8_NONNEG && epi != EPI_F32_P4) return false;
+    if (g.K % (epi == EPI_F32_P4 ? 4 : 8)) return false;
+    // 32-bit byte offsets inside an image of either blob
+    return (size_t)g.C * g.H * g.W * 4 < (1ull << 31) && (size_t)g.K * g.H * g.W * 4 < (1ull << 31);
+}
+
+template <int EPI, int G, int CG>
+static hipError_t launch_pw_f32in(const float* x, const int8_t* wpk, void* out, const ConvGeom& g, const Epilogue& ep,
+                                  const unsigned* qh, int per, const float* in_scale, float in_half, hipStream_t stream) {
+    auto kern = conv_pw_f32in_kernel<EPI, G, CG>;
+    constexpr size_t lds = (size_t)2 * 256 * PW_F32IN_COPIES * 16;  // two buffers of a round's image
+    static bool attr_set = false;  // idempotent; a race only repeats the call
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int HW = g.H * g.W;
+    const dim3 grid((HW + 64 * G - 1) / (64 * G), g.N, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, x, wpk, out, ep, qh, g.C / 8, g.K, HW, per,
+                       igemm_padded_rows(g.K) / 16, in_scale, in_half);
+    return hipGetLastError();
+}
+
+// qh: conv_pw_stream_clamps of the layer's output scales (read by the ReLU / clip epilogue only)
+// force_groups / force_pairs: 0 = automatic
+hipError_t run_conv_pw_f32in(const float* x, const int8_t* wpk, const unsigned* qh, void* out, const ConvGeom& g, const Epilogue& ep,
+                             const float* in_scale, int in_round_mode, int force_groups, int force_pairs, hipStream_t stream) {
+    if (!conv_pw_f32in_applicable(g, ep)) return hipErrorInvalidValue;
+    const int HW = g.H * g.W, pairs = (g.K + 31) / 32, cgs = (g.C + 63) / 64;
+    // two groups per wave halve the LDS reads per output; one group while two would leave SIMDs without a wave
+    int G = (long)g.N * ((HW + 31) / 32) >= 1024 ? 2 : 1;
+    if (force_groups) G = force_groups;
+    if (G != 1 && G != 2) return hipErrorInvalidValue;
+    int per = pw_f32in_pairs_per_round(cgs, pairs);
+    if (force_pairs) per = std::min(std::min(force_pairs, per), pairs);
+    const int epi = pick_epilogue(ep, g.K);
+    if (epi == EPI_I8_P8_NONNEG && !qh) return hipErrorInvalidValue;
+    const float half = in_round_mode == OTTER_HIP_ROUND_SSE ? 0.5f : 0.49999997f;
+#define OHIP_PWF(E_, G_, CG_) \
+    if (epi == E_ && G == G_ && cgs == CG_) return launch_pw_f32in<E_, G_, CG_>(x, wpk, out, g, ep, qh, per, in_scale, half, stream);
+#define OHIP_PWF_E(G_, CG_) OHIP_PWF(EPI_I8_P8, G_, CG_) OHIP_PWF(EPI_I8_P8_NONNEG, G_, CG_) OHIP_PWF(EPI_F32_P4, G_, CG_)
+    OHIP_PWF_E(1, 1) OHIP_PWF_E(1, 2) OHIP_PWF_E(1, 3) OHIP_PWF_E(1, 4)
+    OHIP_PWF_E(2, 1) OHIP_PWF_E(2, 2) OHIP_PWF_E(2, 3) OHIP_PWF_E(2, 4)
+#undef OHIP_PWF_E
+#undef OHIP_PWF
     return hipErrorInvalidValue;
 }
 

@@ -158,7 +158,9 @@ def test_c2_as_stated_fp32_input(hip, oracle):
     in_scale = np.float32(127) / np.abs(x).max()
     kw = dict(bias=bias, act=1, out_kind=capi.OUT_F32)
     full, kind = run_conv(hip, oracle, x, wq, ws, in_scale, **kw)
-    assert kind == 1
+    assert kind == 6   # quantize + convolution in one launch that reads the fp32 blob once
+    two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **kw)   # the reference's order: two launches
+    assert full.tobytes() == two.tobytes()
     for n in (0, 17, N - 1):
         want = oracle.conv_layer_forward(x[n:n + 1], wq, ws, in_scale, bias=bias, act_type=1)
         np.testing.assert_allclose(full[n:n + 1], want, rtol=1e-5, atol=1e-30, err_msg="image %d" % n)

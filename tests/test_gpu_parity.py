@@ -678,6 +678,16 @@ def test_depthwise3x3_from_an_fp32_blob_in_one_launch(hip, oracle, s):
     assert (outs[capi.ROUND_SSE] != outs[capi.ROUND_EXACT]).any()
 
 
+def _fp32_blob_with_ties(rng, shape, in_scale):
+    """fp32 values with some exactly on a tie of the quantization, on the float the two rounding primitives round
+    differently, and beyond saturation."""
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[::7] = (rng.integers(-140, 141, flat[::7].size) + 0.5) / in_scale
+    flat[3::11] = np.nextafter(np.float32(0.5), np.float32(0)) / in_scale * rng.choice([-1, 1], flat[3::11].size)
+    return x
+
+
 @pytest.mark.parametrize("C,K,N,H,W,int8_out,tile_shape,small", [
     (72, 512, 2, 9, 11, True, "128x64", True),
     (72, 512, 1, 7, 7, False, "128x64", True),
@@ -689,20 +699,19 @@ def test_depthwise3x3_from_an_fp32_blob_in_one_launch(hip, oracle, s):
     (8, 16, 8, 256, 256, False, "32x256", False),
     (200, 100, 3, 5, 13, False, "64x64", True),    # channel octets that end inside a 64-deep step, K % 8 != 0
 ])
-def test_pointwise_from_an_fp32_blob_in_one_launch(hip, oracle, C, K, N, H, W, int8_out, tile_shape, small):
+def test_pointwise_from_an_fp32_blob_in_the_igemm_loader(hip, oracle, C, K, N, H, W, int8_out, tile_shape, small):
     """A pointwise layer of the implicit-GEMM kernel on an fp32 Float8 blob quantizes in the kernel's loader (one launch,
-    no int8 copy of the blob). Bit for bit against the two launches (set_tile(-6, 0)) at every tile shape the launcher
-    picks -- values on rounding ties, on the float the two primitives round differently and beyond saturation, every
-    packed epilogue -- and, at the sizes the oracle finishes in seconds, against the oracle's layer."""
+    no int8 copy of the blob; set_tile(-4, 0) keeps the layers on this kernel that would otherwise go to the kernel of
+    the next test). Bit for bit against the two launches (set_tile(-6, 0)) at every tile shape the launcher picks --
+    values on rounding ties, on the float the two primitives round differently and beyond saturation, every packed
+    epilogue -- and, at the sizes the oracle finishes in seconds, against the oracle's layer."""
     rng = np.random.default_rng(C * 7 + K)
-    x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+    _, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
     in_scale = np.float32(100.0)
-    flat = x.reshape(-1)
-    flat[::7] = (rng.integers(-140, 141, flat[::7].size) + 0.5) / in_scale
-    flat[3::11] = np.nextafter(np.float32(0.5), np.float32(0)) / in_scale * rng.choice([-1, 1], flat[3::11].size)
+    x = _fp32_blob_with_ties(rng, (N, C, H, W), in_scale)
     for act in ((3, 0, 2) if int8_out else (1, 2)):
         args = dict(bias=bias, top_scale=9.0, act=act, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
-        out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, **args)
+        out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-4, 0), **args)
         two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **args)
         assert kind == 1
         assert out.tobytes() == two.tobytes(), (act, tile_shape)
@@ -715,12 +724,74 @@ def test_pointwise_from_an_fp32_blob_in_one_launch(hip, oracle, C, K, N, H, W, i
                 assert_f32_close(out, want)
 
 
+@pytest.mark.parametrize("C,K,N,H,W,int8_out,auto,small", [
+    (72, 512, 2, 9, 11, True, True, True),        # two reduction steps, the second one 8 channels; four LDS rounds
+    (256, 136, 1, 7, 7, False, True, True),       # K % 32 != 0: a pair with one live tile and a half
+    (64, 128, 3, 5, 13, True, True, True),        # one reduction step; 65 pixels: a wave with one live pixel
+    (200, 100, 3, 5, 13, False, False, True),     # K % 8 != 0 (fp32 out only), channel octets ending inside a step
+    (8, 16, 2, 9, 11, True, False, True),         # one octet, one output tile
+    (40, 24, 2, 17, 3, True, False, True),
+    (136, 264, 1, 30, 30, True, True, True),      # three steps, 9 pairs: a last round of one pair
+    (256, 512, 32, 28, 28, False, True, False),   # the benchmark layer: one group per wave by the launcher's choice
+    (128, 128, 64, 28, 28, True, True, False),    # two groups per wave by the launcher's choice
+])
+def test_pointwise_from_an_fp32_blob_read_once(hip, oracle, C, K, N, H, W, int8_out, auto, small):
+    """conv_pw_f32in_kernel: a pointwise layer of up to 256 input channels on an fp32 Float8 blob, the blob read once, all
+    output channels walked per pixel group through LDS rounds of weights. Taken by itself from 64 input and 128 output
+    channels on (`auto`), forced otherwise (set_tile(-7, groups | pairs << 3)). Bit for bit against the two launches with
+    one and two pixel groups per wave and with rounds of one, two and the default number of pairs; against the oracle's
+    layer at the sizes it finishes in seconds."""
+    rng = np.random.default_rng(C * 11 + K)
+    _, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+    in_scale = np.float32(100.0)
+    x = _fp32_blob_with_ties(rng, (N, C, H, W), in_scale)
+    for act in ((3, 0, 2) if int8_out else (1, 2)):
+        args = dict(bias=bias, top_scale=9.0, act=act, act_p0=0.1, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **args)
+        tiles = [None] if auto else []
+        tiles += [(-7, 1), (-7, 2)] + ([(-7, 1 | 1 << 3), (-7, 2 | 2 << 3)] if small else [])
+        for tile in tiles:
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, tile=tile, **args)
+            assert kind == 6, tile
+            assert out.tobytes() == two.tobytes(), (act, tile)
+        if small:
+            want = oracle.conv_layer_forward(x, wq, ws, in_scale, bias=bias, top_scale=9.0, int8_out=int8_out, act_type=act,
+                                             act_params=[0.1] if act == 2 else None)
+            if int8_out:
+                np.testing.assert_array_equal(two, want)
+            else:
+                assert_f32_close(two, want)
+
+
+def test_pointwise_from_an_fp32_blob_read_once_exact_rounding(hip, oracle):
+    """The scalar rounding primitive on the input side through conv_pw_f32in_kernel: with a power-of-two input scale a fifth
+    of the values land exactly on the one float the two primitives round differently."""
+    rng = np.random.default_rng(91)
+    C, K, N, H, W = 64, 128, 2, 9, 20
+    x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+    x.reshape(-1)[::5] = np.nextafter(np.float32(0.5), np.float32(0)) / np.float32(128.0)
+    si = (np.float32(1.0) / (np.float32(128.0) * ws)).astype(np.float32)
+    outs = {}
+    for mode in (capi.ROUND_SSE, capi.ROUND_EXACT):
+        conv = hip.conv(wq=wq, scale_in=si, bias=bias, in_scale=128.0, out_scale=[900.0], act=0, out_kind=capi.OUT_I8, in_round=mode)
+        assert conv.kernel_kind(capi.F32_P8, N, H, W, capi.I8_P8) == 6
+        xq = oracle.quantize(x, [np.float32(128.0)], mode)
+        want = oracle.requantize(oracle.conv_int32(xq, wq, (1, 1), (0, 0), (1, 1), 1), si, [900.0], bias, 0, None, capi.ROUND_SSE)
+        got = conv.forward(hip.to_device(capi.pack_np(x, 8)), capi.F32_P8, N, H, W, capi.I8_P8)
+        outs[mode] = capi.unpack_np(got.cpu().numpy(), 8, (N, K, H, W))
+        np.testing.assert_array_equal(outs[mode], want)
+        conv.close()
+    assert (outs[capi.ROUND_SSE] != outs[capi.ROUND_EXACT]).any()
+
+
+@pytest.mark.parametrize("C,K,kind", [(96, 24, 1), (96, 136, 6)])
 @pytest.mark.parametrize("mode", [capi.ROUND_SSE, capi.ROUND_EXACT], ids=["sse", "exact"])
-def test_pointwise_from_an_fp32_blob_twin_and_shortcut(hip, oracle, mode):
-    """The same launch with the shortcut sum and the quantized twin in its epilogue, and with either rounding primitive on
-    the input side: against the oracle's quantize -> convolution -> dequantize -> add -> quantize."""
+def test_pointwise_from_an_fp32_blob_twin_and_shortcut(hip, oracle, mode, C, K, kind):
+    """A pointwise layer on an fp32 blob with the shortcut sum and the quantized twin (the implicit-GEMM launch writes both
+    from its epilogue, also for a layer whose plain forward takes the read-once kernel), and with either rounding
+    primitive on the input side: against the oracle's quantize -> convolution -> dequantize -> add -> quantize."""
     rng = np.random.default_rng(77 + mode)
-    C, K, N, H, W = 96, 24, 3, 14, 13
+    N, H, W = 3, 14, 13
     x, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
     x.reshape(-1)[::5] = np.nextafter(np.float32(0.5), np.float32(0)) / np.float32(128.0)
     si = (np.float32(1.0) / (np.float32(128.0) * ws)).astype(np.float32)
@@ -729,7 +800,7 @@ def test_pointwise_from_an_fp32_blob_twin_and_shortcut(hip, oracle, mode):
     xq = oracle.quantize(x, [np.float32(128.0)], mode)
     plain_want = oracle.dequantize(oracle.conv_int32(xq, wq, (1, 1), (0, 0), (1, 1), 1), si, bias)
     xd = hip.to_device(capi.pack_np(x, 8))
-    assert conv.kernel_kind(capi.F32_P8, N, H, W, capi.F32_P4) == 1
+    assert conv.kernel_kind(capi.F32_P8, N, H, W, capi.F32_P4) == kind
     plain = capi.unpack_np(conv.forward(xd, capi.F32_P8, N, H, W, capi.F32_P4).cpu().numpy(), 4, (N, K, H, W))
     assert_f32_close(plain, plain_want)
     short = (rng.normal(0, 1, plain.shape) * np.abs(plain).mean()).astype(np.float32)

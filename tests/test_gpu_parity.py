@@ -734,6 +734,9 @@ def test_pointwise_from_an_fp32_blob_in_the_igemm_loader(hip, oracle, C, K, N, H
     (136, 264, 1, 30, 30, True, True, True),      # three steps, 9 pairs: a last round of one pair
     (256, 512, 32, 28, 28, False, True, False),   # the benchmark layer: one group per wave by the launcher's choice
     (128, 128, 64, 28, 28, True, True, False),    # two groups per wave by the launcher's choice
+    (8, 4, 1, 1, 1, False, False, True),          # one pixel, one Float4 element of output
+    (16, 8, 5, 1, 3, True, False, True),          # three pixels per image, one Byte8 element
+    (256, 128, 1, 1, 1, True, True, True),        # one pixel, every reduction step
 ])
 def test_pointwise_from_an_fp32_blob_read_once(hip, oracle, C, K, N, H, W, int8_out, auto, small):
     """conv_pw_f32in_kernel: a pointwise layer of up to 256 input channels on an fp32 Float8 blob, the blob read once, all

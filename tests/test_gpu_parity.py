@@ -766,6 +766,36 @@ def test_pointwise_from_an_fp32_blob_read_once(hip, oracle, C, K, N, H, W, int8_
                 assert_f32_close(two, want)
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_pointwise_from_an_fp32_blob_drawn_shapes(hip, oracle, seed):
+    """Eight pointwise layers per seed on fp32 Float8 blobs, drawn over channel counts (8..256 in, 4..520 out), image
+    sizes, batch, activation and output kind, through whichever launch the library picks and through both one-launch
+    kernels forced (set_tile(-4, 0): the implicit-GEMM loader; set_tile(-7, g): the read-once kernel where it takes the
+    shape): bit for bit equal to the two launches, and equal to the oracle's layer."""
+    rng = np.random.default_rng(4000 + seed)
+    for _ in range(8):
+        C = 8 * int(rng.integers(1, 33))
+        int8_out = bool(rng.integers(0, 2))
+        K = (8 if int8_out else 4) * int(rng.integers(1, 66 if int8_out else 131))
+        N, H, W = int(rng.integers(1, 4)), int(rng.integers(1, 20)), int(rng.integers(1, 40))
+        act = int(rng.choice([0, 1, 2, 3]))
+        _, wq, ws, bias = _rand_problem(rng, C, K, 1, 1, N, H, W, in_i8=False)
+        in_scale = np.float32(100.0)
+        x = _fp32_blob_with_ties(rng, (N, C, H, W), in_scale)
+        what = (C, K, N, H, W, act, int8_out)
+        args = dict(bias=bias, top_scale=11.0, act=act, act_p0=0.25, out_kind=capi.OUT_I8 if int8_out else capi.OUT_F32)
+        want = oracle.conv_layer_forward(x, wq, ws, in_scale, bias=bias, top_scale=11.0, int8_out=int8_out, act_type=act,
+                                         act_params=[0.25])
+        two, _ = run_conv(hip, oracle, x, wq, ws, in_scale, tile=(-6, 0), **args)
+        if int8_out:
+            np.testing.assert_array_equal(two, want, err_msg=str(what))
+        else:
+            np.testing.assert_allclose(two, want, rtol=FP32_RTOL, atol=1e-30, err_msg=str(what))
+        for tile in (None, (-4, 0), (-7, 1), (-7, 2)):
+            out, kind = run_conv(hip, oracle, x, wq, ws, in_scale, tile=tile, **args)
+            assert out.tobytes() == two.tobytes(), (what, tile, kind)
+
+
 def test_pointwise_from_an_fp32_blob_read_once_exact_rounding(hip, oracle):
     """The scalar rounding primitive on the input side through conv_pw_f32in_kernel: with a power-of-two input scale a fifth
     of the values land exactly on the one float the two primitives round differently."""
